@@ -1,0 +1,338 @@
+#!/usr/bin/env python3
+"""Benchmark of the custom-kernel hot path on one MI355X.
+
+Default workload (BASELINE.json configs[1]): decode attention at head_dim 128, batch 1,
+32 query / 8 KV heads, bf16, KV length swept over every power of two from 512 to 32768.
+One step = one pass over the seven lengths (split-KV kernel + combine each).  Inputs are
+resident in HBM before the timed region; each length owns several copies of its K/V and a
+pass uses the next copy, so that >1 GB of other traffic separates two reads of the same
+bytes and the 256 MB Infinity Cache cannot serve them.  The passes are captured in a HIP
+graph (launch-bound otherwise) and replayed; the clock is wall time around the replays with
+a device synchronisation on both sides.
+
+Prints ONE JSON line: value = algorithmic GB/s (K+V+Q read, O written) over the timed
+steps; "roofline" prices the same bytes against the 8 TB/s HBM peak from HIP-event timing;
+"cpu_baseline" is stock PyTorch on the host cores for a bounded sample of the same sweep.
+
+Other workloads (--workload c1|c3a|c3b|rms|rope|e2e) report the remaining BASELINE configs
+in the same format.
+"""
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "llama3-custom-inference_amd")
+for _p in (ROOT, PKG):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+SEED = 42               # the reference's default seed (benchmark_kernel.py:126)
+
+
+def attn_bytes(B, QH, KVH, S, HD):
+    """K+V+Q read, O written, bf16 (the reference counts K+V only: benchmark_kernel.py:48)."""
+    return 2 * B * KVH * S * HD * 2 + 2 * B * QH * HD * 2
+
+
+class AttnCase:
+    """One attention shape with `slots` independent copies of its inputs, pre-allocated outputs
+    and workspace, launched straight through the C ABI (no per-call allocation)."""
+
+    def __init__(self, torch, lib, l3, dev, B, QH, KVH, S, HD, slots, src_k=None, src_v=None, src_q=None):
+        self.torch, self.lib = torch, lib
+        self.B, self.QH, self.KVH, self.S, self.HD = B, QH, KVH, S, HD
+        self.bytes = attn_bytes(B, QH, KVH, S, HD)
+        self.slots = slots
+        g = torch.Generator().manual_seed(SEED)
+        q = src_q if src_q is not None else torch.randn((B, 1, QH, HD), generator=g).to(torch.bfloat16)
+        k = src_k if src_k is not None else torch.randn((B, S, KVH, HD), generator=g).to(torch.bfloat16)
+        v = src_v if src_v is not None else torch.randn((B, S, KVH, HD), generator=g).to(torch.bfloat16)
+        self.cpu = (q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
+        # token-major storage, transposed views: the model's cache layout (benchmark_kernel.py:165-173)
+        self.q = [q.to(dev).transpose(1, 2) for _ in range(slots)]
+        self.k = [k.to(dev).transpose(1, 2) for _ in range(slots)]
+        self.v = [v.to(dev).transpose(1, 2) for _ in range(slots)]
+        self.out = [torch.empty_like(t) for t in self.q]
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        self.num_splits = lib.l3_attn_choose_splits(B, KVH, S, HD, cus)
+        self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.num_splits)
+        self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
+        self._args = []
+        for i in range(slots):
+            qt, kt, vt, ot = self.q[i], self.k[i], self.v[i], self.out[i]
+            self._args.append((
+                qt.data_ptr(), kt.data_ptr(), vt.data_ptr(), ot.data_ptr(), self.ws.data_ptr(), self.ws_bytes,
+                B, QH, KVH, S, HD,
+                l3.i64_array((qt.stride(0), qt.stride(1))), l3.i64_array((kt.stride(0), kt.stride(1), kt.stride(2))),
+                l3.i64_array((vt.stride(0), vt.stride(1), vt.stride(2))), l3.i64_array((ot.stride(0), ot.stride(1))),
+                1.0 / math.sqrt(HD), self.num_splits))
+
+    def launch(self, slot, stream_ptr):
+        rc = self.lib.l3_attn_decode(*self._args[slot % self.slots], stream_ptr)
+        if rc != 0:
+            raise RuntimeError(f"l3_attn_decode failed: {rc}")
+
+
+def capture_graph(torch, fn):
+    """Capture fn() (which launches on torch's current stream) into a HIP graph."""
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        fn()  # warm-up outside capture (module load, allocator)
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    return graph
+
+
+def event_time_ms(torch, run, reps):
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        run()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / reps
+
+
+def time_cpu(fn, min_seconds, min_reps=3, max_reps=100000):
+    fn()
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        fn()
+        n += 1
+        el = time.perf_counter() - t0
+        if (el >= min_seconds and n >= min_reps) or n >= max_reps:
+            return el / n, n
+
+
+# ------------------------------------------------------------------------------ workloads
+def run_attention(args, torch, lib, l3, dev, name):
+    from oracle.cpu_baseline import attention_cpu
+
+    QH, KVH = 32, 8
+    if name == "c2":
+        B, HD, lengths = 1, 128, [512, 1024, 2048, 4096, 8192, 16384, 32768]
+        label = "decode attention sweep: B1 QH32 KVH8 HD128 bf16, KV length 512..32768 (x2), split+combine"
+    elif name == "c1":
+        B, HD, lengths = 1, 64, [256]
+        label = "decode attention: B1 QH32 KVH8 HD64 bf16, KV length 256, split+combine"
+    elif name == "c3a":
+        B, HD, lengths = 256, 64, [256]
+        label = "batched decode attention: B256 QH32 KVH8 HD64 bf16, KV length 256"
+    elif name == "c3b":
+        B, HD, lengths = 16, 64, [4096]
+        label = "batched decode attention: B16 QH32 KVH8 HD64 bf16, KV length 4096, split+combine"
+    elif name == "hd64":
+        B, HD, lengths = 1, 64, [512, 1024, 2048, 4096, 8192, 16384, 32768]
+        label = "decode attention sweep: B1 QH32 KVH8 HD64 bf16, KV length 512..32768 (x2), split+combine"
+    else:
+        raise ValueError(name)
+
+    smax = max(lengths)
+    g = torch.Generator().manual_seed(SEED)
+    q = torch.randn((B, 1, QH, HD), generator=g).to(torch.bfloat16)
+    k = torch.randn((B, smax, KVH, HD), generator=g).to(torch.bfloat16)
+    v = torch.randn((B, smax, KVH, HD), generator=g).to(torch.bfloat16)
+    pass_bytes = sum(attn_bytes(B, QH, KVH, S, HD) for S in lengths)
+    # enough copies that a pass over all of them moves > 1 GiB between two uses of the same bytes
+    slots = max(4, int(math.ceil((1 << 30) / pass_bytes)))
+    slots = min(slots, 64)
+    cases = [AttnCase(torch, lib, l3, dev, B, QH, KVH, S, HD, slots, src_k=k[:, :S].contiguous(),
+                      src_v=v[:, :S].contiguous(), src_q=q) for S in lengths]
+
+    def one_pass(slot):
+        sp = torch.cuda.current_stream().cuda_stream
+        for c in cases:
+            c.launch(slot, sp)
+
+    passes_per_graph = slots
+    graph = capture_graph(torch, lambda: [one_pass(s) for s in range(passes_per_graph)])
+
+    steps = max(passes_per_graph, (args.steps + passes_per_graph - 1) // passes_per_graph * passes_per_graph)
+    warm = max(1, (args.warmup + passes_per_graph - 1) // passes_per_graph)
+    for _ in range(warm):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps // passes_per_graph):
+        graph.replay()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / steps
+    value = pass_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # HIP-event timing of the same replays (events on the stream the kernels run on)
+    ev_ms = event_time_ms(torch, graph.replay, max(1, steps // passes_per_graph)) / passes_per_graph
+    achieved = pass_bytes / (ev_ms * 1e-3) / 1e9
+
+    # per-length detail: each length alone, rotating over its copies, graph-replayed
+    detail = []
+    for c in cases:
+        reps_in_graph = max(slots, 16)
+        gph = capture_graph(torch, lambda c=c: [c.launch(s, torch.cuda.current_stream().cuda_stream)
+                                                for s in range(reps_in_graph)])
+        gph.replay()
+        ms = event_time_ms(torch, gph.replay, 5) / reps_in_graph
+        gbps = c.bytes / (ms * 1e-3) / 1e9
+        detail.append({"kv_len": c.S, "splits": c.num_splits, "us": round(ms * 1e3, 3), "GBps": round(gbps, 1),
+                       "frac": round(gbps / HBM_PEAK_GBPS, 4), "bytes": c.bytes,
+                       "cold": bool(c.bytes * slots > (300 << 20))})
+        del gph
+
+    cpu = None
+    if not args.no_cpu_baseline and name in ("c2", "c1"):
+        def cpu_pass():
+            for c in cases:
+                attention_cpu(*c.cpu)
+        sec, n = time_cpu(cpu_pass, args.cpu_seconds)
+        cpu = {"value": round(pass_bytes / sec / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
+               "kind": "port", "host_cpus": os.cpu_count(),
+               "sample": f"{n} passes of the same sweep with torch CPU scaled_dot_product_attention "
+                         f"(bf16, enable_gqa) in {sec * n:.1f} s"}
+
+    return {
+        "metric": "decode_attn_hbm_GBps", "value": round(value, 1), "unit": "GB/s",
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "steps": steps, "ms_per_step": round(ms_per_step, 5), "dtype": "bf16",
+        "config": {"workload": label, "kv_copies_per_length": slots, "accumulate": "f32", "launch": "hip graph",
+                   "seed": SEED},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "attn_splitkv_kernel (+ attn_combine_kernel), per pass of the workload",
+                     "algorithmic_bytes_per_pass": pass_bytes},
+        "cpu_baseline": cpu, "per_length": detail,
+    }
+
+
+def run_rows(args, torch, lib, l3, dev, name):
+    """RMSNorm / rotary embedding at the largest BASELINE config-4 shape, plus the small ones."""
+    from custom_kernels import custom_kernels_extension as cke
+    from custom_kernels import precompute_freqs_cis
+    from oracle.cpu_baseline import rms_norm_cpu, rot_embed_cpu
+
+    detail = []
+    head = None
+    if name == "rms":
+        for C in (2048, 4096):
+            for (B, T) in ((1, 1), (1, 64), (1, 256), (2, 2048)):
+                copies = max(2, min(64, (1 << 30) // max(1, 2 * B * T * C * 2)))
+                g = torch.Generator().manual_seed(SEED)
+                xs = [torch.randn((B, T, C), generator=g).to(torch.bfloat16).to(dev) for _ in range(min(copies, 4))]
+                xs = xs + [xs[0].clone() for _ in range(copies - len(xs))]
+                w = (torch.randn((C,), generator=g) * 0.02 + 1).to(torch.bfloat16).to(dev)
+                ys = [torch.empty_like(x) for x in xs]
+                sp = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+                gph = capture_graph(torch, lambda: [lib.l3_rms_norm(x.data_ptr(), w.data_ptr(), y.data_ptr(), B * T, C,
+                                                                    1e-5, sp()) for x, y in zip(xs, ys)])
+                gph.replay()
+                ms = event_time_ms(torch, gph.replay, 10) / copies
+                nbytes = 2 * B * T * C * 2 + C * 2
+                rec = {"rows": B * T, "C": C, "us": round(ms * 1e3, 3), "GBps": round(nbytes / ms / 1e6, 1),
+                       "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nbytes}
+                detail.append(rec)
+                if C == 4096 and B * T == 4096:
+                    head = (rec, ms, nbytes, lambda x=xs[0].cpu(), w=w.cpu(): rms_norm_cpu(x, w, 1e-5))
+        label = "fused RMSNorm: 4096 rows x C 4096 bf16 (2x2048-token prefill), eps 1e-5"
+        metric = "rms_norm_hbm_GBps"
+    else:
+        for HD in (64, 128):
+            tab = precompute_freqs_cis(HD, 4096, 500000.0, True, scale_factor=32.0, device=dev)
+            for (B, T) in ((1, 1), (1, 64), (1, 256), (2, 2048)):
+                NH = 32
+                copies = max(2, min(64, (1 << 30) // max(1, 2 * B * T * NH * HD * 2)))
+                g = torch.Generator().manual_seed(SEED)
+                buf0 = torch.randn((B, T, (NH + 16) * HD), generator=g).to(torch.bfloat16).to(dev)
+                bufs = [buf0] + [buf0.clone() for _ in range(copies - 1)]
+                xs = [b[..., : NH * HD].view(B, T, NH, HD) for b in bufs]
+                ys = [torch.empty((B, T, NH, HD), dtype=torch.bfloat16, device=dev) for _ in xs]
+                fr = tab[:T].contiguous()
+                st = l3.i64_array((xs[0].stride(0), xs[0].stride(1), xs[0].stride(2)))
+                sp = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+                gph = capture_graph(torch, lambda: [lib.l3_rot_embed(x.data_ptr(), fr.data_ptr(), y.data_ptr(), B, T,
+                                                                     NH, HD, st, sp()) for x, y in zip(xs, ys)])
+                gph.replay()
+                ms = event_time_ms(torch, gph.replay, 10) / copies
+                nbytes = 2 * B * T * NH * HD * 2 + T * HD * 4
+                rec = {"tokens": B * T, "NH": NH, "HD": HD, "us": round(ms * 1e3, 3),
+                       "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                       "bytes": nbytes}
+                detail.append(rec)
+                if HD == 128 and B * T == 4096:
+                    head = (rec, ms, nbytes, lambda x=xs[0].cpu(), f=fr.cpu(): rot_embed_cpu(x, f))
+        label = "fused rotary embedding: 4096 tokens x 32 heads x HD 128 bf16 from a strided qkv view"
+        metric = "rot_embed_hbm_GBps"
+
+    rec, ms, nbytes, cpu_fn = head
+    cpu = None
+    if not args.no_cpu_baseline:
+        sec, n = time_cpu(cpu_fn, min(args.cpu_seconds, 5.0))
+        cpu = {"value": round(nbytes / sec / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
+               "kind": "port", "host_cpus": os.cpu_count(), "sample": f"{n} runs of the same shape in torch on the CPU"}
+    return {
+        "metric": metric, "value": rec["GBps"], "unit": "GB/s", "frac_of_hbm_peak": rec["frac"],
+        "steps": args.steps, "ms_per_step": round(ms, 5), "dtype": "bf16",
+        "config": {"workload": label, "accumulate": "f32", "launch": "hip graph", "seed": SEED},
+        "roofline": {"bound": "hbm", "achieved": rec["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": rec["frac"], "traffic": None, "algorithmic_bytes_per_launch": nbytes},
+        "cpu_baseline": cpu, "per_shape": detail,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "e2e"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall time spent on the CPU baseline sample")
+    ap.add_argument("--e2e-batch", type=int, default=1)
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print(f"bench.py: this path runs on one GPU with no sharding; --gpus {args.gpus} is not supported "
+              "(every (batch, kv head) pair is independent, see DESIGN.md for how it would shard)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from custom_kernels import _l3lib as l3
+
+    lib = l3.load()  # raises if the HIP library is missing: nothing else can run this path
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the hot path has no CPU implementation to measure", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):
+        res = run_attention(args, torch, lib, l3, dev, args.workload)
+    elif args.workload in ("rms", "rope"):
+        res = run_rows(args, torch, lib, l3, dev, args.workload)
+    else:
+        import llama_arch
+
+        res = llama_arch.bench_e2e(args, torch, dev)
+
+    line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
+            "steps": res.pop("steps"), "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": res.pop("dtype"),
+            "data": "synthetic", "config": res.pop("config")}
+    line.update(res)
+    line["device"] = torch.cuda.get_device_name(0)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

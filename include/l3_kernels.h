@@ -1,0 +1,122 @@
+/*
+ * C ABI of libl3kernels.so: MI355X (gfx950) kernels for the custom-operator hot path of
+ * llama3-custom-inference -- split-KV decode attention with its log-sum-exp combine,
+ * fused RMSNorm and fused rotary embedding.
+ *
+ * The three compute entry points replace the three host launchers the reference binds
+ * in custom_kernels/main.cpp:2-8.  Conventions shared by all of them:
+ *   - every pointer is a device pointer to bfloat16 (uint16 bit patterns) unless stated;
+ *   - strides are in ELEMENTS, as torch reports them; the innermost dimension must be
+ *     contiguous (the reference assumes it: custom_kernels.cu:44,55,401);
+ *   - the library never allocates, frees or retains device memory: outputs and the
+ *     attention workspace are caller-owned;
+ *   - work is enqueued on the caller's `stream` (a hipStream_t; NULL = the null stream)
+ *     and the call returns without synchronising (the reference launches on the legacy
+ *     stream, custom_kernels.cu:274-275,386,439);
+ *   - the return value is L3_OK or a negative L3_ERR_* code; argument checks run before
+ *     any HIP call, so they can be exercised on a machine without a GPU.  Nothing here
+ *     calls exit() (the reference's unused cudaCheck would: custom_kernels.cu:224-229).
+ */
+#ifndef L3_KERNELS_H
+#define L3_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    L3_OK = 0,
+    L3_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
+    L3_ERR_HEAD_SIZE = -2,      /* head size not 64 or 128 (custom_kernels.cu:317-319) */
+    L3_ERR_HEAD_RATIO = -3,     /* QH/KVH not one of 1,2,3,4,8 (custom_kernels.cu:289-291,312-314) */
+    L3_ERR_SHAPE = -4,          /* a dimension is <= 0, too large, or QH is not a multiple of KVH */
+    L3_ERR_STRIDE = -5,         /* a stride is negative or not a multiple of what the loads need */
+    L3_ERR_ALIGNMENT = -6,      /* a base pointer is not aligned for the vector loads */
+    L3_ERR_WORKSPACE = -7,      /* workspace NULL or smaller than l3_attn_decode_workspace_bytes */
+    L3_ERR_SPLITS = -8,         /* num_splits negative or above L3_ATTN_MAX_SPLITS */
+    L3_ERR_HIP = -9             /* the HIP runtime reported an error at launch */
+};
+
+#define L3_ATTN_MAX_SPLITS 512
+
+/* Library version: major*10000 + minor*100 + patch. */
+int l3_version(void);
+
+/* Static, NUL-terminated description of an error code (never NULL). */
+const char* l3_strerror(int code);
+
+/*
+ * Split count the attention kernel would pick for this problem on a device with
+ * `num_cus` compute units (<= 0: ask the current HIP device, 256 if there is none).
+ * Pure integer host logic.  Replaces the fixed rule n_step = ceil(S / 64) of
+ * custom_kernels.cu:243,251; the count is chosen so that B*KVH*splits workgroups fill
+ * the device while every split keeps enough tokens to amortise its merge.
+ * Returns a value in [1, L3_ATTN_MAX_SPLITS], or a negative error code.
+ */
+int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus);
+
+/*
+ * Bytes of workspace l3_attn_decode needs for `num_splits` (0 = the automatic choice for
+ * the current device).  0 when the plan has a single split (the kernel then writes the
+ * output directly).  Replaces the three per-call temporaries of custom_kernels.cu:269-271
+ * (tmp_result, score_maxes, softmax_sums); partial outputs are kept in float32 here.
+ */
+size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int num_splits);
+
+/*
+ * out[b, h, :] = softmax(scale * q[b, h, :] . k[b, h / (QH/KVH), :, :]^T) @ v[b, h / (QH/KVH), :, :]
+ *
+ * Replaces flash_attention_decode(query, keys, values), custom_kernels.cu:233-338
+ * (main.cpp:2,6), i.e. the split-KV kernel :13-177 followed by the combine kernel
+ * :179-223, for one query token per sequence.
+ *   q, out : (B, QH, 1, HD) bf16; q_strides / out_strides = {batch, head} strides
+ *   k, v   : (B, KVH, S, HD) bf16; k_strides / v_strides = {batch, head, token} strides.
+ *            Token rows must start on 16-byte boundaries (base pointers 16-byte aligned,
+ *            strides multiples of 8).  q and out need 16-byte aligned rows as well.
+ *   scale  : softmax scale; the reference uses 1/sqrt(HD) (custom_kernels.cu:253)
+ *   num_splits : 0 = automatic, otherwise 1..L3_ATTN_MAX_SPLITS (the kernel may use fewer
+ *            when S is short); results do not depend on it beyond float32 rounding
+ *   workspace : >= l3_attn_decode_workspace_bytes(...) bytes, 256-byte aligned; may be NULL
+ *            when that size is 0.  Contents on entry are ignored.
+ * Supported: HD in {64, 128}, QH/KVH in {1, 2, 3, 4, 8}, S >= 1.
+ */
+int l3_attn_decode(const void* q, const void* k, const void* v, void* out,
+                   void* workspace, size_t workspace_bytes,
+                   int B, int QH, int KVH, int S, int HD,
+                   const int64_t q_strides[2], const int64_t k_strides[3],
+                   const int64_t v_strides[3], const int64_t out_strides[2],
+                   float scale, int num_splits, void* stream);
+
+/*
+ * y[r, :] = bf16( x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * w[:] ), float32 inside, one rounding.
+ *
+ * Replaces rms_norm(input, weight, eps), custom_kernels.cu:369-389 (kernel :340-367,
+ * main.cpp:3,7).  x and y are `rows` contiguous rows of C bf16 values (the reference
+ * indexes its (B, T, C) input as contiguous: custom_kernels.cu:355), w is C bf16 values.
+ * Any C >= 1; rows of C % 8 == 0 with 16-byte aligned pointers take the vector path.
+ */
+int l3_rms_norm(const void* x, const void* w, void* y, int64_t rows, int C, float eps, void* stream);
+
+/*
+ * Rotary embedding on adjacent pairs:
+ *   y[b,t,h,2i]   = bf16( x[b,t,h,2i] * freq[t,2i] - x[b,t,h,2i+1] * freq[t,2i+1] )
+ *   y[b,t,h,2i+1] = bf16( x[b,t,h,2i] * freq[t,2i+1] + x[b,t,h,2i+1] * freq[t,2i] )
+ *
+ * Replaces rot_embed(input, freq), custom_kernels.cu:418-442 (kernel :391-416,
+ * main.cpp:4,8).  x is (B, T, NH, HD) bf16 with x_strides = {batch, token, head} strides
+ * (q and k arrive as views into the fused qkv projection: model.py:96-97); freq is a
+ * contiguous (T, HD) float32 table of interleaved cos/sin (model.py:59-60); y is a
+ * CONTIGUOUS (B, T, NH, HD) bf16 tensor, as the reference writes it
+ * (custom_kernels.cu:414).  HD must be even; pairs must be 4-byte aligned.  16-byte
+ * aligned rows with HD % 8 == 0 take the vector path.
+ */
+int l3_rot_embed(const void* x, const float* freq, void* y, int B, int T, int NH, int HD,
+                 const int64_t x_strides[3], void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* L3_KERNELS_H */

@@ -1,0 +1,200 @@
+// C ABI of libl3kernels.so: argument checks, split planning and dispatch.  Every check runs
+// before the first HIP call so the error paths can be driven on a machine without a GPU.
+// Takes the place of the host launchers flash_attention_decode / rms_norm / rot_embed
+// (custom_kernels.cu:233-338, 369-389, 418-442) and of the pybind table in main.cpp:5-9.
+#include <math.h>
+
+#include <mutex>
+
+#include "l3_host.hpp"
+
+namespace l3 {
+
+namespace {
+
+constexpr int kVersion = 100;  // 0.1.0
+constexpr size_t kWorkspaceAlign = 256;
+
+bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+bool ratio_supported(int R) { return R == 1 || R == 2 || R == 3 || R == 4 || R == 8; }
+
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+size_t round_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
+
+int check_attn_shape(int B, int QH, int KVH, int S, int HD) {
+    if (HD != 64 && HD != 128) return L3_ERR_HEAD_SIZE;
+    if (B <= 0 || QH <= 0 || KVH <= 0 || S <= 0) return L3_ERR_SHAPE;
+    if (QH % KVH != 0) return L3_ERR_SHAPE;
+    if (!ratio_supported(QH / KVH)) return L3_ERR_HEAD_RATIO;
+    // grid = B * KVH * splits workgroups and B * QH combine workgroups must fit 31 bits
+    if (int64_t(B) * QH * L3_ATTN_MAX_SPLITS >= (int64_t(1) << 31)) return L3_ERR_SHAPE;
+    return L3_OK;
+}
+
+size_t attn_workspace_bytes(int B, int QH, int HD, int num_splits) {
+    if (num_splits <= 1) return 0;
+    const size_t rows = size_t(B) * size_t(QH) * size_t(num_splits);
+    return round_up(rows * HD * sizeof(float), kWorkspaceAlign) + round_up(rows * sizeof(float2), kWorkspaceAlign);
+}
+
+}  // namespace
+
+int current_device_cus() {
+    static std::once_flag once;
+    static int cus = 256;
+    std::call_once(once, [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) {
+            cus = n;
+        } else {
+            (void)hipGetLastError();  // do not leave a sticky "no device" behind
+        }
+    });
+    return cus;
+}
+
+AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus) {
+    const int tile = attn_block_tile_tokens(HD);
+    const int max_by_len = ceil_div(S, tile);  // a split shorter than one tile leaves waves idle
+    int splits;
+    if (requested > 0) {
+        splits = requested;
+    } else {
+        // Two 4-wave workgroups per compute unit keep 128 KiB of K/V in flight per CU; more
+        // splits than that only add partials for the combine to re-read.
+        const int64_t units = int64_t(B) * KVH;
+        const int64_t target = int64_t(num_cus) * 2;
+        splits = int((target + units - 1) / units);
+    }
+    if (splits > max_by_len) splits = max_by_len;
+    if (splits > L3_ATTN_MAX_SPLITS) splits = L3_ATTN_MAX_SPLITS;
+    if (splits < 1) splits = 1;
+    int tps = ceil_div(ceil_div(S, splits), tile) * tile;
+    AttnPlan plan;
+    plan.tokens_per_split = tps;
+    plan.num_splits = ceil_div(S, tps);  // every split is non-empty
+    return plan;
+}
+
+}  // namespace l3
+
+using namespace l3;
+
+extern "C" {
+
+int l3_version(void) { return kVersion; }
+
+const char* l3_strerror(int code) {
+    switch (code) {
+        case L3_OK: return "success";
+        case L3_ERR_NULL_POINTER: return "null pointer argument";
+        case L3_ERR_HEAD_SIZE: return "Unsupported head size for splitkv kernel";
+        case L3_ERR_HEAD_RATIO: return "Unsupported QKV head ratio for splitkv kernel";
+        case L3_ERR_SHAPE: return "invalid shape";
+        case L3_ERR_STRIDE: return "unsupported stride";
+        case L3_ERR_ALIGNMENT: return "misaligned pointer";
+        case L3_ERR_WORKSPACE: return "workspace missing or too small";
+        case L3_ERR_SPLITS: return "num_splits out of range";
+        case L3_ERR_HIP: return "HIP runtime error at kernel launch";
+        default: return "unknown error code";
+    }
+}
+
+int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus) {
+    if (HD != 64 && HD != 128) return L3_ERR_HEAD_SIZE;
+    if (B <= 0 || KVH <= 0 || S <= 0) return L3_ERR_SHAPE;
+    if (num_cus <= 0) num_cus = current_device_cus();
+    return attn_make_plan(B, KVH, S, HD, 0, num_cus).num_splits;
+}
+
+size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int num_splits) {
+    if (check_attn_shape(B, QH, KVH, S, HD) != L3_OK) return 0;
+    if (num_splits < 0 || num_splits > L3_ATTN_MAX_SPLITS) return 0;
+    const int cus = (num_splits == 0) ? current_device_cus() : 0;
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus);
+    return attn_workspace_bytes(B, QH, HD, plan.num_splits);
+}
+
+int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void* workspace,
+                   size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
+                   const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
+                   const int64_t out_strides[2], float scale, int num_splits, void* stream) {
+    if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !out_strides)
+        return L3_ERR_NULL_POINTER;
+    if (int rc = check_attn_shape(B, QH, KVH, S, HD); rc != L3_OK) return rc;
+    if (num_splits < 0 || num_splits > L3_ATTN_MAX_SPLITS) return L3_ERR_SPLITS;
+    // 16-byte vector loads: every row must start on a 16-byte boundary.
+    // (strides of size-1 dimensions are never used to form an address and are not checked)
+    const int q_dims[2] = {B, QH};
+    for (int i = 0; i < 2; ++i) {
+        if (q_dims[i] == 1) continue;
+        if (q_strides[i] < 0 || out_strides[i] < 0 || q_strides[i] % 8 || out_strides[i] % 8) return L3_ERR_STRIDE;
+    }
+    const int kv_dims[3] = {B, KVH, S};
+    for (int i = 0; i < 3; ++i) {
+        if (kv_dims[i] == 1) continue;
+        if (k_strides[i] < 0 || v_strides[i] < 0 || k_strides[i] % 8 || v_strides[i] % 8) return L3_ERR_STRIDE;
+    }
+    if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 16)) return L3_ERR_ALIGNMENT;
+
+    const int cus = (num_splits == 0) ? current_device_cus() : 0;
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus);
+    const size_t need = attn_workspace_bytes(B, QH, HD, plan.num_splits);
+    if (need > 0) {
+        if (!workspace || workspace_bytes < need) return L3_ERR_WORKSPACE;
+        if (!aligned(workspace, kWorkspaceAlign)) return L3_ERR_ALIGNMENT;
+    }
+
+    AttnParams p;
+    p.q = static_cast<const uint16_t*>(q);
+    p.k = static_cast<const uint16_t*>(k);
+    p.v = static_cast<const uint16_t*>(v);
+    p.out = static_cast<uint16_t*>(out);
+    const size_t rows = size_t(B) * size_t(QH) * size_t(plan.num_splits);
+    p.part_o = static_cast<float*>(workspace);
+    p.part_ml = reinterpret_cast<float2*>(static_cast<char*>(workspace) +
+                                          round_up(rows * HD * sizeof(float), kWorkspaceAlign));
+    p.B = B; p.QH = QH; p.KVH = KVH; p.S = S;
+    p.num_splits = plan.num_splits;
+    p.tokens_per_split = plan.tokens_per_split;
+    p.q_sb = q_strides[0]; p.q_sh = q_strides[1];
+    p.k_sb = k_strides[0]; p.k_sh = k_strides[1]; p.k_st = k_strides[2];
+    p.v_sb = v_strides[0]; p.v_sh = v_strides[1]; p.v_st = v_strides[2];
+    p.o_sb = out_strides[0]; p.o_sh = out_strides[1];
+    p.scale_log2e = scale * 1.4426950408889634f;
+    return launch_attn_decode(p, HD, QH / KVH, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_rms_norm(const void* x, const void* w, void* y, int64_t rows, int C, float eps, void* stream) {
+    if (!x || !w || !y) return L3_ERR_NULL_POINTER;
+    if (rows <= 0 || C <= 0 || rows >= (int64_t(1) << 31)) return L3_ERR_SHAPE;
+    if (!aligned(x, 2) || !aligned(w, 2) || !aligned(y, 2)) return L3_ERR_ALIGNMENT;
+    const bool vec_ok = (C % 8 == 0) && aligned(x, 16) && aligned(w, 16) && aligned(y, 16);
+    return launch_rms_norm(static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w),
+                           static_cast<uint16_t*>(y), rows, C, eps, vec_ok,
+                           static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_rot_embed(const void* x, const float* freq, void* y, int B, int T, int NH, int HD,
+                 const int64_t x_strides[3], void* stream) {
+    if (!x || !freq || !y || !x_strides) return L3_ERR_NULL_POINTER;
+    if (B <= 0 || T <= 0 || NH <= 0 || HD <= 0 || (HD % 2) != 0) return L3_ERR_SHAPE;
+    if (int64_t(B) * T * NH * (HD / 2) >= (int64_t(1) << 38)) return L3_ERR_SHAPE;  // grid size
+    const int x_dims[3] = {B, T, NH};
+    bool strides8 = true;
+    for (int i = 0; i < 3; ++i) {
+        if (x_dims[i] == 1) continue;
+        if (x_strides[i] < 0 || x_strides[i] % 2) return L3_ERR_STRIDE;
+        strides8 = strides8 && (x_strides[i] % 8 == 0);
+    }
+    if (!aligned(x, 4) || !aligned(y, 4) || !aligned(freq, 8)) return L3_ERR_ALIGNMENT;
+    const bool vec_ok = (HD % 8 == 0) && aligned(x, 16) && aligned(y, 16) && aligned(freq, 16) && strides8;
+    return launch_rot_embed(static_cast<const uint16_t*>(x), freq, static_cast<uint16_t*>(y), B, T, NH, HD,
+                            x_strides[0], x_strides[1], x_strides[2], vec_ok,
+                            static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+}  // extern "C"

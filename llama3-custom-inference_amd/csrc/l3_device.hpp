@@ -1,0 +1,104 @@
+// Device-side helpers shared by the gfx950 kernels: bf16 <-> f32 on raw bit patterns and
+// wave64 cross-lane reductions built on DPP.  These take the place of the reference's
+// dtype_bfloat16.cuh:47-54 (casts) and reduce_kernels.cuh:8-64 (32-lane shuffle
+// butterflies plus a shared-memory stage), re-thought for 64-wide wavefronts.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace l3 {
+
+constexpr int kWaveSize = 64;
+
+// ---------------------------------------------------------------- bf16 bit patterns
+// A 32-bit word holds two bf16 values: element 2i in the low half, 2i+1 in the high half.
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(uint32_t(h) << 16); }
+
+// Round-to-nearest-even f32 -> bf16 bit pattern (NaN stays a quiet NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);
+    r = (f != f) ? 0x7fc00000u : r;
+    return r >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// Unpack the 8 bf16 values of a 16-byte vector into f32.
+__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
+    f[0] = bf16lo_to_f32(v.x); f[1] = bf16hi_to_f32(v.x);
+    f[2] = bf16lo_to_f32(v.y); f[3] = bf16hi_to_f32(v.y);
+    f[4] = bf16lo_to_f32(v.z); f[5] = bf16hi_to_f32(v.z);
+    f[6] = bf16lo_to_f32(v.w); f[7] = bf16hi_to_f32(v.w);
+}
+
+// ------------------------------------------------------------------ DPP cross-lane
+// dpp_ctrl encodings (GCN3+/CDNA): quad_perm = perm bits, 0x140 row_mirror,
+// 0x141 row_half_mirror.  All lanes read a valid source for these patterns.
+constexpr int kDppQuadXor1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;  // lane i <-> 7-i within each 8 lanes
+constexpr int kDppRowMirror = 0x140;      // lane i <-> 15-i within each 16 lanes
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over aligned groups of N consecutive lanes (N in {4, 8, 16}); every lane of a
+// group ends with the same bits (each step adds the two halves commutatively).
+template <int N>
+__device__ __forceinline__ float group_sum(float x) {
+    static_assert(N == 4 || N == 8 || N == 16, "group size");
+    x += dpp_move<kDppQuadXor1>(x);
+    x += dpp_move<kDppQuadXor2>(x);
+    if constexpr (N >= 8) x += dpp_move<kDppRowHalfMirror>(x);
+    if constexpr (N >= 16) x += dpp_move<kDppRowMirror>(x);
+    return x;
+}
+
+template <int N>
+__device__ __forceinline__ float group_max(float x) {
+    static_assert(N == 4 || N == 8 || N == 16, "group size");
+    x = fmaxf(x, dpp_move<kDppQuadXor1>(x));
+    x = fmaxf(x, dpp_move<kDppQuadXor2>(x));
+    if constexpr (N >= 8) x = fmaxf(x, dpp_move<kDppRowHalfMirror>(x));
+    if constexpr (N >= 16) x = fmaxf(x, dpp_move<kDppRowMirror>(x));
+    return x;
+}
+
+// Whole-wavefront sum / max, result uniform across the 64 lanes: DPP inside each row of
+// 16 lanes, then the four row results are read back through scalar lane reads.
+__device__ __forceinline__ float wave_sum(float x) {
+    x = group_sum<16>(x);
+    int xi = __builtin_bit_cast(int, x);
+    float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 0));
+    float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 16));
+    float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 32));
+    float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 48));
+    return (a + b) + (c + d);
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+    x = group_max<16>(x);
+    int xi = __builtin_bit_cast(int, x);
+    float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 0));
+    float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 16));
+    float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 32));
+    float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+// 2^x through the hardware v_exp_f32 (inputs here are <= 0 or small; no denormal fix-up).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// 16-byte global load / store on element pointers.
+__device__ __forceinline__ uint4 load16(const uint16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ void store16(uint16_t* p, const uint4& v) { *reinterpret_cast<uint4*>(p) = v; }
+
+}  // namespace l3

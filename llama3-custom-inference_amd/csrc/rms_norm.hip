@@ -1,0 +1,130 @@
+// Fused RMSNorm for gfx950.  Takes the place of custom_rms_norm_kernel
+// (custom_kernels.cu:340-367).  Differences by design: each row is read from HBM once
+// (16-byte loads kept in registers between the sum of squares and the scaling), the
+// product x * inv_rms * w is formed in float32 and rounded to bf16 once (the reference
+// rounds inv_rms and both products to bf16, custom_kernels.cu:362-366), and the row is
+// reduced with wave64 DPP steps instead of 32-lane shuffles plus a 32-entry shared stage.
+#include "l3_device.hpp"
+#include "l3_host.hpp"
+
+namespace l3 {
+
+namespace {
+
+constexpr int kRmsThreads = 256;
+
+// One row per group of LANES threads (64: a wavefront per row, four rows per workgroup;
+// 256: the whole workgroup on one row).  A thread keeps up to MAXV 16-byte vectors of its
+// row in registers; requires C % 8 == 0 and C / 8 <= LANES * MAXV.
+template <int LANES, int MAXV>
+__global__ void __launch_bounds__(kRmsThreads)
+rms_norm_rows_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, uint16_t* __restrict__ y,
+                     int64_t rows, int C, float eps) {
+    constexpr int ROWS_PER_BLOCK = kRmsThreads / LANES;
+    const int tid = threadIdx.x;
+    const int sub = tid / LANES;
+    const int t = tid % LANES;
+    const int64_t row = int64_t(blockIdx.x) * ROWS_PER_BLOCK + sub;
+    const bool live = row < rows;
+    const int nvec = C / 8;
+    const uint16_t* xr = x + (live ? row : 0) * int64_t(C);
+
+    uint4 xv[MAXV];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int vi = t + j * LANES;
+        if (vi < nvec) {
+            xv[j] = load16(xr + vi * 8);
+            float f[8];
+            unpack8(xv[j], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+        }
+    }
+    ss = wave_sum(ss);
+    if constexpr (LANES > kWaveSize) {
+        __shared__ float s_part[kRmsThreads / kWaveSize];
+        if ((tid & (kWaveSize - 1)) == 0) s_part[tid / kWaveSize] = ss;
+        __syncthreads();
+        ss = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+    }
+    const float inv = rsqrtf(ss / float(C) + eps);
+    if (!live) return;
+
+    uint16_t* yr = y + row * int64_t(C);
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int vi = t + j * LANES;
+        if (vi < nvec) {
+            float f[8], g[8];
+            unpack8(xv[j], f);
+            unpack8(load16(w + vi * 8), g);
+            uint4 o;
+            o.x = pack_bf16x2(f[0] * inv * g[0], f[1] * inv * g[1]);
+            o.y = pack_bf16x2(f[2] * inv * g[2], f[3] * inv * g[3]);
+            o.z = pack_bf16x2(f[4] * inv * g[4], f[5] * inv * g[5]);
+            o.w = pack_bf16x2(f[6] * inv * g[6], f[7] * inv * g[7]);
+            store16(yr + vi * 8, o);
+        }
+    }
+}
+
+// Any C, any alignment: one workgroup per row, 2-byte accesses, the row is read twice.
+__global__ void __launch_bounds__(kRmsThreads)
+rms_norm_generic_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, uint16_t* __restrict__ y,
+                        int C, float eps) {
+    const int tid = threadIdx.x;
+    const uint16_t* xr = x + int64_t(blockIdx.x) * C;
+    uint16_t* yr = y + int64_t(blockIdx.x) * C;
+    float ss = 0.f;
+    for (int i = tid; i < C; i += kRmsThreads) {
+        const float f = bf16_to_f32(xr[i]);
+        ss = fmaf(f, f, ss);
+    }
+    ss = wave_sum(ss);
+    __shared__ float s_part[kRmsThreads / kWaveSize];
+    if ((tid & (kWaveSize - 1)) == 0) s_part[tid / kWaveSize] = ss;
+    __syncthreads();
+    ss = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+    const float inv = rsqrtf(ss / float(C) + eps);
+    for (int i = tid; i < C; i += kRmsThreads) {
+        yr[i] = uint16_t(f32_to_bf16_bits(bf16_to_f32(xr[i]) * inv * bf16_to_f32(w[i])));
+    }
+}
+
+}  // namespace
+
+int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
+                    bool vec_ok, hipStream_t stream) {
+    const int nvec = C / 8;
+    if (vec_ok && rows >= 1024 && nvec <= 64 * 8) {
+        // plenty of rows: a wavefront per row, no workgroup barrier
+        const unsigned blocks = unsigned((rows + 3) / 4);
+        if (nvec <= 64 * 4) {
+            hipLaunchKernelGGL((rms_norm_rows_kernel<64, 4>), dim3(blocks), dim3(kRmsThreads), 0, stream, x, w, y,
+                               rows, C, eps);
+        } else {
+            hipLaunchKernelGGL((rms_norm_rows_kernel<64, 8>), dim3(blocks), dim3(kRmsThreads), 0, stream, x, w, y,
+                               rows, C, eps);
+        }
+    } else if (vec_ok && nvec <= 256 * 4) {
+        // few rows (decode): the whole workgroup on one row keeps the latency short
+        if (nvec <= 256) {
+            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 1>), dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x,
+                               w, y, rows, C, eps);
+        } else if (nvec <= 512) {
+            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 2>), dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x,
+                               w, y, rows, C, eps);
+        } else {
+            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 4>), dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x,
+                               w, y, rows, C, eps);
+        }
+    } else {
+        hipLaunchKernelGGL(rms_norm_generic_kernel, dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x, w, y, C,
+                           eps);
+    }
+    return int(hipGetLastError());
+}
+
+}  // namespace l3

@@ -1,0 +1,95 @@
+// Fused rotary embedding for gfx950.  Takes the place of custom_rot_embed_kernel
+// (custom_kernels.cu:391-416): same arithmetic (float32 complex multiply of adjacent
+// pairs by the (cos, sin) table row of the token, one rounding), same strided-input /
+// contiguous-output contract, but each lane moves 16 bytes (four pairs) instead of 4 and
+// the grid is a flat range over 16-byte items rather than one 32/64-thread block per
+// (batch, token, head).
+#include "l3_device.hpp"
+#include "l3_host.hpp"
+
+namespace l3 {
+
+namespace {
+
+constexpr int kRopeThreads = 256;
+
+__device__ __forceinline__ uint32_t rotate_pair(uint32_t xw, float c, float s) {
+    const float x0 = bf16lo_to_f32(xw);
+    const float x1 = bf16hi_to_f32(xw);
+    // x0*c - x1*s can cancel; a plain float32 evaluation then carries the rounding error of
+    // the larger product into a much smaller result and can miss the exact answer by more
+    // than one bf16 ulp.  The second product's rounding error is recovered exactly with an
+    // fma (e = x1*s - p) so that the error stays relative to the result itself.
+    const float p0 = x1 * s;
+    const float e0 = fmaf(x1, s, -p0);
+    const float y0 = fmaf(x0, c, -p0) - e0;
+    const float p1 = x1 * c;
+    const float e1 = fmaf(x1, c, -p1);
+    const float y1 = fmaf(x0, s, p1) + e1;
+    return pack_bf16x2(y0, y1);
+}
+
+// One 16-byte item (8 values = 4 pairs) per thread.  VPR = HD / 8 items per (b, t, h) row.
+__global__ void __launch_bounds__(kRopeThreads)
+rot_embed_vec_kernel(const uint16_t* __restrict__ x, const float* __restrict__ freq, uint16_t* __restrict__ y,
+                     int64_t total_items, int T, int NH, int HD, int64_t sb, int64_t st, int64_t sh) {
+    const int64_t item = int64_t(blockIdx.x) * kRopeThreads + threadIdx.x;
+    if (item >= total_items) return;
+    const int vpr = HD / 8;
+    const int c = int(item % vpr);
+    int64_t r = item / vpr;
+    const int h = int(r % NH);
+    r /= NH;
+    const int t = int(r % T);
+    const int64_t b = r / T;
+
+    const uint4 xv = load16(x + b * sb + t * st + h * sh + c * 8);
+    const float4* fp = reinterpret_cast<const float4*>(freq + int64_t(t) * HD + c * 8);
+    const float4 f0 = fp[0];
+    const float4 f1 = fp[1];
+    uint4 o;
+    o.x = rotate_pair(xv.x, f0.x, f0.y);
+    o.y = rotate_pair(xv.y, f0.z, f0.w);
+    o.z = rotate_pair(xv.z, f1.x, f1.y);
+    o.w = rotate_pair(xv.w, f1.z, f1.w);
+    store16(y + item * 8, o);
+}
+
+// Fallback: one pair per thread with 4-byte accesses (any even HD, 4-byte aligned rows).
+__global__ void __launch_bounds__(kRopeThreads)
+rot_embed_pair_kernel(const uint16_t* __restrict__ x, const float* __restrict__ freq, uint16_t* __restrict__ y,
+                      int64_t total_pairs, int T, int NH, int HD, int64_t sb, int64_t st, int64_t sh) {
+    const int64_t item = int64_t(blockIdx.x) * kRopeThreads + threadIdx.x;
+    if (item >= total_pairs) return;
+    const int ppr = HD / 2;
+    const int c = int(item % ppr);
+    int64_t r = item / ppr;
+    const int h = int(r % NH);
+    r /= NH;
+    const int t = int(r % T);
+    const int64_t b = r / T;
+    const uint32_t xw = *reinterpret_cast<const uint32_t*>(x + b * sb + t * st + h * sh + c * 2);
+    const float2 f = *reinterpret_cast<const float2*>(freq + int64_t(t) * HD + c * 2);
+    *reinterpret_cast<uint32_t*>(y + item * 2) = rotate_pair(xw, f.x, f.y);
+}
+
+}  // namespace
+
+int launch_rot_embed(const uint16_t* x, const float* freq, uint16_t* y, int B, int T, int NH, int HD,
+                     int64_t sb, int64_t st, int64_t sh, bool vec_ok, hipStream_t stream) {
+    const int64_t rows = int64_t(B) * T * NH;
+    if (vec_ok) {
+        const int64_t items = rows * (HD / 8);
+        const unsigned blocks = unsigned((items + kRopeThreads - 1) / kRopeThreads);
+        hipLaunchKernelGGL(rot_embed_vec_kernel, dim3(blocks), dim3(kRopeThreads), 0, stream, x, freq, y, items, T,
+                           NH, HD, sb, st, sh);
+    } else {
+        const int64_t items = rows * (HD / 2);
+        const unsigned blocks = unsigned((items + kRopeThreads - 1) / kRopeThreads);
+        hipLaunchKernelGGL(rot_embed_pair_kernel, dim3(blocks), dim3(kRopeThreads), 0, stream, x, freq, y, items, T,
+                           NH, HD, sb, st, sh);
+    }
+    return int(hipGetLastError());
+}
+
+}  // namespace l3

@@ -1,0 +1,83 @@
+"""ctypes binding of libl3kernels.so (declared in include/l3_kernels.h).
+
+Loading fails loudly: there is no CPU or PyTorch fallback for any operator.
+"""
+
+import ctypes
+import os
+
+_LIB_NAME = "libl3kernels.so"
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+L3_OK = 0
+L3_ERR_NULL_POINTER = -1
+L3_ERR_HEAD_SIZE = -2
+L3_ERR_HEAD_RATIO = -3
+L3_ERR_SHAPE = -4
+L3_ERR_STRIDE = -5
+L3_ERR_ALIGNMENT = -6
+L3_ERR_WORKSPACE = -7
+L3_ERR_SPLITS = -8
+L3_ERR_HIP = -9
+L3_ATTN_MAX_SPLITS = 512
+
+# name -> (restype, argtypes); mirrors include/l3_kernels.h line by line
+_c_i64p = ctypes.POINTER(ctypes.c_int64)
+SIGNATURES = {
+    "l3_version": (ctypes.c_int, []),
+    "l3_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "l3_attn_choose_splits": (ctypes.c_int, [ctypes.c_int] * 5),
+    "l3_attn_decode_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 6),
+    "l3_attn_decode": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v out
+         ctypes.c_void_p, ctypes.c_size_t,                                    # workspace, bytes
+         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,  # B QH KVH S HD
+         _c_i64p, _c_i64p, _c_i64p, _c_i64p,                                  # strides
+         ctypes.c_float, ctypes.c_int, ctypes.c_void_p],                      # scale splits stream
+    ),
+    "l3_rms_norm": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
+         ctypes.c_void_p],
+    ),
+    "l3_rot_embed": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         ctypes.c_int, _c_i64p, ctypes.c_void_p],
+    ),
+}
+
+_lib = None
+
+
+def library_path() -> str:
+    return os.environ.get("L3_KERNELS_LIB", os.path.join(_HERE, _LIB_NAME))
+
+
+def load():
+    """Return the loaded library (cached); raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise ImportError(
+            f"{path} not found: build it with `python llama3-custom-inference_amd/build.py` "
+            "(hipcc --offload-arch=gfx950). There is no fallback implementation."
+        )
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here = library/header mismatch
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def strerror(code: int) -> str:
+    return load().l3_strerror(int(code)).decode()
+
+
+def i64_array(values):
+    return (ctypes.c_int64 * len(values))(*[int(v) for v in values])

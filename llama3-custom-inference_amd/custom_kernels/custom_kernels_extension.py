@@ -1,0 +1,163 @@
+"""The three operators the reference binds in custom_kernels/main.cpp:5-9, same names and
+positional signatures, backed by the gfx950 kernels of libl3kernels.so.
+
+    flash_attention_decode(query, keys, values) -> Tensor    custom_kernels.cu:233-338
+    rms_norm(input, weight, eps) -> Tensor                   custom_kernels.cu:369-389
+    rot_embed(input, freq) -> Tensor                         custom_kernels.cu:418-442
+
+Outputs are fresh tensors with the reference's shapes, dtypes and strides
+(``empty_like(query)``, ``empty_like(input)``, and a contiguous (B, T, NH, HD) tensor for
+rot_embed).  Unsupported arguments raise RuntimeError like the reference's TORCH_CHECKs.
+Kernels are enqueued on torch's current stream of the input's device and the call does
+not synchronise.  There is no fallback path: a missing library or a non-GPU tensor raises.
+"""
+
+import math
+
+import torch
+
+from . import _l3lib
+
+__all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits"]
+
+_cu_count = {}
+
+
+def _fail(code: int, detail: str = ""):
+    msg = _l3lib.strerror(code)
+    raise RuntimeError(f"{msg}{': ' + detail if detail else ''} (l3 error {code})")
+
+
+def _require_gpu_bf16(name: str, t: torch.Tensor):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be on the GPU (got {t.device}); there is no CPU path")
+    if t.dtype != torch.bfloat16:
+        # the reference's data_ptr<at::BFloat16>() raises the same way (custom_kernels.cu:274)
+        raise RuntimeError(f"expected scalar type BFloat16 for {name} but found {t.dtype}")
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _cus(device) -> int:
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    n = _cu_count.get(idx)
+    if n is None:
+        n = torch.cuda.get_device_properties(idx).multi_processor_count
+        _cu_count[idx] = n
+    return n
+
+
+def attention_num_splits(B: int, KVH: int, S: int, HD: int, num_cus: int = 256) -> int:
+    """Split count the kernel picks for this problem (pure host logic, runs without a GPU)."""
+    n = _l3lib.load().l3_attn_choose_splits(B, KVH, S, HD, num_cus)
+    if n < 0:
+        _fail(n)
+    return n
+
+
+def flash_attention_decode(query, keys, values, num_splits: int = 0):
+    """query (B, QH, 1, HD); keys/values (B, KVH, S, HD) views of the KV cache (model.py:107-118).
+
+    ``num_splits`` (0 = automatic) is an extension for tests and sweeps; the reference
+    signature is the three tensors.
+    """
+    lib = _l3lib.load()
+    _require_gpu_bf16("query", query)
+    _require_gpu_bf16("keys", keys)
+    _require_gpu_bf16("values", values)
+    if query.dim() != 4 or keys.dim() != 4 or values.dim() != 4:
+        raise RuntimeError("flash_attention_decode expects 4-D query, keys and values")
+    if keys.device != query.device or values.device != query.device:
+        raise RuntimeError("query, keys and values must be on the same device")
+    B, KVH, S, HD = keys.shape
+    QH = query.size(1)
+    if query.size(0) != B or query.size(2) != 1 or query.size(3) != HD or tuple(values.shape) != tuple(keys.shape):
+        raise RuntimeError(
+            f"shape mismatch: query {tuple(query.shape)}, keys {tuple(keys.shape)}, values {tuple(values.shape)}")
+    if query.stride(3) != 1 or keys.stride(3) != 1 or values.stride(3) != 1:
+        raise RuntimeError("the head dimension of query, keys and values must be contiguous")
+    if HD not in (64, 128):
+        _fail(_l3lib.L3_ERR_HEAD_SIZE, str(HD))
+    if KVH == 0 or QH % KVH != 0 or (QH // KVH) not in (1, 2, 3, 4, 8):
+        _fail(_l3lib.L3_ERR_HEAD_RATIO, f"{QH}/{KVH}")
+
+    out = torch.empty_like(query)
+    if out.stride(3) != 1:
+        out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
+    if B == 0 or S == 0:
+        raise RuntimeError("flash_attention_decode needs at least one sequence and one cached token")
+
+    with torch.cuda.device(query.device):
+        if num_splits == 0:
+            num_splits = lib.l3_attn_choose_splits(B, KVH, S, HD, _cus(query.device))
+            if num_splits < 0:
+                _fail(num_splits)
+        ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, num_splits)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=query.device) if ws_bytes else None
+        rc = lib.l3_attn_decode(
+            query.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws_bytes,
+            B, QH, KVH, S, HD,
+            _l3lib.i64_array((query.stride(0), query.stride(1))),
+            _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
+            _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
+            _l3lib.i64_array((out.stride(0), out.stride(1))),
+            1.0 / math.sqrt(HD), num_splits, _stream_ptr(query.device))
+    if rc != 0:
+        _fail(rc, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
+    return out
+
+
+def rms_norm(input, weight, eps):
+    """input (B, T, C) bf16, weight (C,) bf16 -> (B, T, C) bf16 (model.py:70-72)."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("input", input)
+    _require_gpu_bf16("weight", weight)
+    if input.dim() != 3:
+        raise RuntimeError("rms_norm expects a 3-D (B, T, C) input")
+    C = input.size(2)
+    if weight.numel() != C:
+        raise RuntimeError(f"weight has {weight.numel()} elements, expected {C}")
+    x = input if input.is_contiguous() else input.contiguous()
+    w = weight if weight.is_contiguous() else weight.contiguous()
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    rows = x.size(0) * x.size(1)
+    if rows == 0:
+        return out
+    with torch.cuda.device(x.device):
+        rc = lib.l3_rms_norm(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, C, float(eps),
+                             _stream_ptr(x.device))
+    if rc != 0:
+        _fail(rc, f"rows={rows} C={C}")
+    return out
+
+
+def rot_embed(input, freq):
+    """input (B, T, NH, HD) bf16 (any strides on the first three dims), freq (T, HD) float32
+    interleaved cos/sin -> contiguous (B, T, NH, HD) bf16 (model.py:100-101)."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("input", input)
+    if not freq.is_cuda or freq.dtype != torch.float32:
+        raise RuntimeError(f"expected a GPU float32 freq table but found {freq.dtype} on {freq.device}")
+    if input.dim() != 4 or freq.dim() != 2:
+        raise RuntimeError("rot_embed expects a 4-D (B, T, NH, HD) input and a 2-D (T, HD) freq table")
+    B, T, NH, HD = input.shape
+    if freq.size(0) != T or freq.size(1) != HD:
+        raise RuntimeError(f"freq is {tuple(freq.shape)}, expected {(T, HD)}")
+    if input.stride(3) != 1:
+        raise RuntimeError("the head dimension of input must be contiguous")
+    f = freq if freq.is_contiguous() else freq.contiguous()
+    out = torch.empty((B, T, NH, HD), dtype=input.dtype, device=input.device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(input.device):
+        rc = lib.l3_rot_embed(input.data_ptr(), f.data_ptr(), out.data_ptr(), B, T, NH, HD,
+                              _l3lib.i64_array((input.stride(0), input.stride(1), input.stride(2))),
+                              _stream_ptr(input.device))
+    if rc != 0:
+        _fail(rc, f"B={B} T={T} NH={NH} HD={HD} strides={tuple(input.stride())}")
+    return out

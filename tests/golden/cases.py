@@ -1,0 +1,73 @@
+"""Case table shared by make_golden.py and the tests that read the fixtures.
+
+Inputs are not stored: they are re-drawn from the seed with the CPU generator (helpers.py)
+and guarded by a CRC of their bits, so a drift in the generator is reported as such rather
+than as a kernel failure.
+"""
+
+import zlib
+
+import numpy as np
+
+from helpers import make_qkv, randn_bf16, t2bits
+
+ATTN_CASES = {
+    # name: (B, QH, KVH, S, HD, cache_len, seed)
+    "c1_llama32_1b_s256": (1, 32, 8, 256, 64, None, 42),          # BASELINE config 1
+    "hd128_s130_cacheview": (1, 32, 8, 130, 128, 192, 43),        # ragged S, batch stride of a longer cache
+    "b2_r4_s200": (2, 8, 2, 200, 64, None, 44),
+    "r1_s65": (2, 4, 4, 65, 64, None, 45),
+    "r3_hd128_s77": (1, 24, 8, 77, 128, None, 46),                # Llama-3.2-3B ratio
+    "r8_hd128_s300": (1, 16, 2, 300, 128, 512, 47),               # Llama-3.3-70B ratio
+    "s1": (3, 8, 2, 1, 64, 16, 48),
+}
+
+RMS_CASES = {
+    # name: (B, T, C, seed)
+    "decode_c2048": (3, 1, 2048, 50),
+    "rows_c4096": (1, 5, 4096, 51),
+    "odd_c136": (2, 3, 136, 52),
+    "generic_c100": (1, 4, 100, 53),
+}
+
+ROPE_CASES = {
+    # name: (B, T, NH, HD, start_pos, factor, seed)
+    "q_hd64": (2, 5, 32, 64, 0, 32.0, 60),
+    "k_hd128": (1, 4, 8, 128, 1000, 8.0, 61),
+    "decode_hd64": (3, 1, 8, 64, 8191, 32.0, 62),
+}
+
+FREQ_CASES = {
+    # name: (HD, factor, positions)
+    "hd64_f32": (64, 32.0, (0, 1, 2, 100, 8191, 16383)),
+    "hd128_f8": (128, 8.0, (0, 1, 255, 4096, 16383)),
+}
+
+
+def crc(*arrays) -> int:
+    c = 0
+    for a in arrays:
+        c = zlib.crc32(np.ascontiguousarray(a).tobytes(), c)
+    return c
+
+
+def attn_inputs(name):
+    B, QH, KVH, S, HD, L, seed = ATTN_CASES[name]
+    return make_qkv(B, QH, KVH, S, HD, seed=seed, cache_len=L)
+
+
+def rms_inputs(name):
+    B, T, C, seed = RMS_CASES[name]
+    return randn_bf16((B, T, C), seed), randn_bf16((C,), seed + 1, scale=0.02, mean=1.0)
+
+
+def rope_inputs(name):
+    """x is a strided view into a fused qkv-like buffer (model.py:96-97)."""
+    B, T, NH, HD, start, factor, seed = ROPE_CASES[name]
+    buf = randn_bf16((B, T, (NH + 16) * HD), seed)
+    x = buf[..., : NH * HD].view(B, T, NH, HD)
+    return x, start, factor
+
+
+def bits_crc(*tensors) -> int:
+    return crc(*[t2bits(t) for t in tensors])

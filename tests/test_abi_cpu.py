@@ -1,0 +1,132 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol include/l3_kernels.h
+declares, rejects bad arguments before any launch, and plans splits sanely."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from custom_kernels import _l3lib
+from custom_kernels import custom_kernels_extension as cke
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "l3_kernels.h")
+FAKE = 0x7F0000001000  # 4 KiB-aligned non-null address that is never dereferenced on the host
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(l3_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = _l3lib.load()
+    names = _declared()
+    assert names == sorted(_l3lib.SIGNATURES), "header and ctypes table disagree"
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.l3_version() >= 100
+
+
+def test_error_codes_match_header():
+    text = open(HEADER).read()
+    for name, val in re.findall(r"(L3_(?:OK|ERR_[A-Z_]+))\s*=\s*(-?\d+)", text):
+        assert getattr(_l3lib, name) == int(val)
+        assert _l3lib.strerror(int(val))
+    assert int(re.search(r"#define L3_ATTN_MAX_SPLITS (\d+)", text).group(1)) == _l3lib.L3_ATTN_MAX_SPLITS
+    assert "unknown" in _l3lib.strerror(-12345)
+
+
+def _attn(q=FAKE, k=FAKE, v=FAKE, out=FAKE, ws=None, ws_bytes=0, B=1, QH=32, KVH=8, S=256, HD=64,
+          qs=(2048, 64), ks=(131072, 64, 512), vs=(131072, 64, 512), os_=(2048, 64), splits=1):
+    return _l3lib.load().l3_attn_decode(q, k, v, out, ws, ws_bytes, B, QH, KVH, S, HD, _l3lib.i64_array(qs),
+                                        _l3lib.i64_array(ks), _l3lib.i64_array(vs), _l3lib.i64_array(os_),
+                                        0.125, splits, None)
+
+
+def test_attention_argument_checks_run_before_any_launch():
+    assert _attn(q=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert _attn(out=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert _attn(HD=96) == _l3lib.L3_ERR_HEAD_SIZE           # custom_kernels.cu:317-319
+    assert _attn(HD=256) == _l3lib.L3_ERR_HEAD_SIZE
+    assert _attn(QH=40, KVH=8) == _l3lib.L3_ERR_HEAD_RATIO   # ratio 5: custom_kernels.cu:289-291
+    assert _attn(QH=30, KVH=8) == _l3lib.L3_ERR_SHAPE
+    assert _attn(S=0) == _l3lib.L3_ERR_SHAPE
+    assert _attn(B=-1) == _l3lib.L3_ERR_SHAPE
+    assert _attn(splits=-1) == _l3lib.L3_ERR_SPLITS
+    assert _attn(splits=_l3lib.L3_ATTN_MAX_SPLITS + 1) == _l3lib.L3_ERR_SPLITS
+    assert _attn(ks=(131072, 64, 516)) == _l3lib.L3_ERR_STRIDE      # rows off 16-byte boundaries
+    assert _attn(vs=(131072, 60, 512)) == _l3lib.L3_ERR_STRIDE
+    assert _attn(qs=(2048, -64)) == _l3lib.L3_ERR_STRIDE
+    assert _attn(k=FAKE + 2) == _l3lib.L3_ERR_ALIGNMENT
+    assert _attn(S=1024, ks=(524288, 64, 512), vs=(524288, 64, 512), splits=4) == _l3lib.L3_ERR_WORKSPACE
+    assert _attn(S=1024, ks=(524288, 64, 512), vs=(524288, 64, 512), splits=4, ws=FAKE, ws_bytes=16) \
+        == _l3lib.L3_ERR_WORKSPACE
+    need = _l3lib.load().l3_attn_decode_workspace_bytes(1, 32, 8, 1024, 64, 4)
+    assert _attn(S=1024, ks=(524288, 64, 512), vs=(524288, 64, 512), splits=4, ws=FAKE + 64, ws_bytes=need) \
+        == _l3lib.L3_ERR_ALIGNMENT
+
+
+def test_rms_norm_and_rot_embed_argument_checks():
+    lib = _l3lib.load()
+    assert lib.l3_rms_norm(None, FAKE, FAKE, 4, 2048, 1e-5, None) == _l3lib.L3_ERR_NULL_POINTER
+    assert lib.l3_rms_norm(FAKE, FAKE, FAKE, 0, 2048, 1e-5, None) == _l3lib.L3_ERR_SHAPE
+    assert lib.l3_rms_norm(FAKE, FAKE, FAKE, 4, 0, 1e-5, None) == _l3lib.L3_ERR_SHAPE
+    assert lib.l3_rms_norm(FAKE + 1, FAKE, FAKE, 4, 2048, 1e-5, None) == _l3lib.L3_ERR_ALIGNMENT
+    st = _l3lib.i64_array((3072 * 5, 3072, 64))
+    assert lib.l3_rot_embed(FAKE, None, FAKE, 1, 5, 32, 64, st, None) == _l3lib.L3_ERR_NULL_POINTER
+    assert lib.l3_rot_embed(FAKE, FAKE, FAKE, 1, 5, 32, 63, st, None) == _l3lib.L3_ERR_SHAPE
+    assert lib.l3_rot_embed(FAKE, FAKE, FAKE, 1, 0, 32, 64, st, None) == _l3lib.L3_ERR_SHAPE
+    assert lib.l3_rot_embed(FAKE, FAKE, FAKE, 1, 5, 32, 64, _l3lib.i64_array((15360, 3071, 64)), None) \
+        == _l3lib.L3_ERR_STRIDE
+    assert lib.l3_rot_embed(FAKE + 2, FAKE, FAKE, 1, 5, 32, 64, st, None) == _l3lib.L3_ERR_ALIGNMENT
+
+
+def test_split_planning():
+    lib = _l3lib.load()
+    for HD, tile in ((64, 128), (128, 64)):
+        prev = 0
+        for S in (1, 63, 64, 65, 256, 512, 1000, 4096, 32768, 131072):
+            n = lib.l3_attn_choose_splits(1, 8, S, HD, 256)
+            assert 1 <= n <= _l3lib.L3_ATTN_MAX_SPLITS
+            assert n <= max(1, -(-S // tile)), "no split shorter than one workgroup tile"
+            assert n >= prev, "more tokens never means fewer splits at fixed batch"
+            prev = n
+            ws = lib.l3_attn_decode_workspace_bytes(1, 32, 8, S, HD, 0)
+            if n == 1:
+                assert ws == 0
+            else:
+                rows = 32 * n
+                assert rows * (HD + 2) * 4 <= ws <= rows * (HD + 2) * 4 + 512
+        # enough (batch, kv head) pairs to fill the device: no split, no combine
+        assert lib.l3_attn_choose_splits(256, 8, 256, HD, 256) == 1
+        # the device size matters
+        assert lib.l3_attn_choose_splits(1, 8, 32768, HD, 64) < lib.l3_attn_choose_splits(1, 8, 32768, HD, 256)
+    assert lib.l3_attn_choose_splits(1, 8, 256, 96, 256) == _l3lib.L3_ERR_HEAD_SIZE
+    assert lib.l3_attn_choose_splits(0, 8, 256, 64, 256) == _l3lib.L3_ERR_SHAPE
+    assert cke.attention_num_splits(16, 8, 4096, 64) == lib.l3_attn_choose_splits(16, 8, 4096, 64, 256)
+    # an explicit request is honoured up to what the length allows
+    assert lib.l3_attn_decode_workspace_bytes(1, 32, 8, 4096, 128, 7) == 32 * 7 * 128 * 4 + 32 * 7 * 8
+
+
+def test_shim_rejects_cpu_tensors_and_has_no_fallback():
+    import torch
+
+    x = torch.zeros(1, 1, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        cke.rms_norm(x, torch.ones(64, dtype=torch.bfloat16), 1e-5)
+    with pytest.raises(RuntimeError, match="GPU"):
+        cke.rot_embed(torch.zeros(1, 1, 1, 64, dtype=torch.bfloat16), torch.zeros(1, 64))
+    with pytest.raises(RuntimeError, match="GPU"):
+        cke.flash_attention_decode(torch.zeros(1, 4, 1, 64, dtype=torch.bfloat16),
+                                   torch.zeros(1, 4, 8, 64, dtype=torch.bfloat16),
+                                   torch.zeros(1, 4, 8, 64, dtype=torch.bfloat16))
+
+
+def test_missing_library_raises(monkeypatch, tmp_path):
+    monkeypatch.setenv("L3_KERNELS_LIB", str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_l3lib, "_lib", None)
+    with pytest.raises(ImportError, match="no fallback"):
+        _l3lib.load()

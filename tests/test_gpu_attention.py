@@ -1,0 +1,165 @@
+"""GPU parity: split-KV decode attention + combine (through the C ABI) against the float64
+oracle on the same seeded inputs.  Tolerance: atol 2e-2 / rtol 1.6e-2 on the bf16 output
+(helpers.ATTN_ATOL / ATTN_RTOL)."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_attn_close, make_qkv, randn_bf16, t2bits, t2f32
+from oracle import attention_decode_ref
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(gpu, B, QH, KVH, S, HD, seed=42, cache_len=None, splits=0, tweak=None):
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"attention B={B} QH={QH} KVH={KVH} S={S} HD={HD} L={cache_len} splits={splits} seed={seed}", flush=True)
+    q, k, v = make_qkv(B, QH, KVH, S, HD, seed=seed, cache_len=cache_len)
+    if tweak is not None:
+        tweak(q, k, v)
+    qg, kg, vg = make_qkv(B, QH, KVH, S, HD, seed=seed, cache_len=cache_len, device=gpu)
+    if tweak is not None:
+        tweak(qg, kg, vg)
+    out = cke.flash_attention_decode(qg, kg, vg, splits)
+    torch.cuda.synchronize()
+    assert out.shape == qg.shape and out.stride() == qg.stride()
+    ref = attention_decode_ref(t2f32(q), t2f32(k), t2f32(v))
+    err = assert_attn_close(out, ref, what=f"B{B} QH{QH} KVH{KVH} S{S} HD{HD} splits{splits}")
+    return out, ref, err
+
+
+@pytest.mark.parametrize("HD", [64, 128])
+@pytest.mark.parametrize("S", [1, 2, 7, 31, 32, 33, 63, 64, 65, 127, 128, 129, 200, 257, 1000])
+def test_ragged_lengths(gpu, HD, S):
+    _run(gpu, 2, 8, 2, S, HD, seed=S)
+
+
+@pytest.mark.parametrize("HD,QH,KVH", [(64, 4, 4), (64, 8, 4), (64, 12, 4), (64, 32, 8), (64, 16, 2),
+                                        (128, 4, 4), (128, 4, 2), (128, 24, 8), (128, 32, 8), (128, 64, 8)])
+@pytest.mark.parametrize("splits", [0, 1, 4])
+def test_head_ratios(gpu, HD, QH, KVH, splits):
+    _run(gpu, 2, QH, KVH, 333, HD, seed=QH + KVH, splits=splits)
+
+
+@pytest.mark.parametrize("HD", [64, 128])
+@pytest.mark.parametrize("splits", [1, 2, 5, 16, 512])
+def test_result_independent_of_split_count(gpu, HD, splits):
+    base, ref, _ = _run(gpu, 1, 32, 8, 2048, HD, seed=5, splits=1)
+    out, _, _ = _run(gpu, 1, 32, 8, 2048, HD, seed=5, splits=splits)
+    d = np.abs(t2f32(out).astype(np.float64) - t2f32(base).astype(np.float64))
+    assert d.max() <= 2.0 ** -7 * max(1.0, np.abs(ref).max()), "split count changes the result beyond bf16 rounding"
+
+
+@pytest.mark.parametrize("HD", [64, 128])
+def test_dominant_key_in_a_late_split(gpu, HD):
+    """One key far above the rest, sitting in the last split: the log-sum-exp combine must
+    hand that split ~all the weight.  A combine that reuses split 0's statistics for every
+    split (custom_kernels.cu:184,201,209) returns the mean of the splits and fails this."""
+    S = 1500
+
+    def tweak(q, k, v):
+        k[0, 1, S - 10] = q[0, 5, 0] * 4.0   # query head 5 -> kv head 1
+
+    out, ref, _ = _run(gpu, 1, 32, 8, S, HD, seed=3, splits=8, tweak=tweak)
+    q, k, v = make_qkv(1, 32, 8, S, HD, seed=3)
+    got = t2f32(out)[0, 5, 0]
+    assert np.abs(got - t2f32(v)[0, 1, S - 10]).max() < 0.05
+    assert np.abs(ref[0, 5, 0] - t2f32(v)[0, 1, S - 10]).max() < 0.05
+
+
+@pytest.mark.parametrize("HD", [64, 128])
+def test_cache_view_and_dense_layouts_give_identical_bits(gpu, HD):
+    """Same values through three layouts: a slice of a longer cache (batch stride L*KVH*HD,
+    model.py:89,107), the benchmark's token-major tensor (benchmark_kernel.py:165-173) and
+    a head-major contiguous (B, KVH, S, HD) tensor."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, QH, KVH, S = 3, 32, 8, 777
+    q, k, v = make_qkv(B, QH, KVH, S, HD, seed=9, cache_len=1024, device=gpu)
+    a = cke.flash_attention_decode(q, k, v)
+    kt = k.transpose(1, 2).contiguous().transpose(1, 2)
+    vt = v.transpose(1, 2).contiguous().transpose(1, 2)
+    b = cke.flash_attention_decode(q, kt, vt)
+    c = cke.flash_attention_decode(q.contiguous(), k.contiguous(), v.contiguous())
+    torch.cuda.synchronize()
+    assert k.stride() != kt.stride() != k.contiguous().stride()
+    np.testing.assert_array_equal(t2bits(a), t2bits(b))
+    np.testing.assert_array_equal(t2bits(a), t2bits(c))
+
+
+def test_equal_value_rows_return_that_row(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    q, k, v = make_qkv(2, 32, 8, 4096, 128, seed=1, device=gpu)
+    row = randn_bf16((2, 8, 1, 128), 77).to(gpu)
+    v_const = row.expand(2, 8, 4096, 128).transpose(1, 2).contiguous().transpose(1, 2)
+    out = cke.flash_attention_decode(q, k, v_const)
+    torch.cuda.synchronize()
+    want = row.repeat_interleave(4, dim=1)
+    # a convex combination of identical rows: only bf16 rounding of the normalised sum remains
+    assert (out.float() - want.float()).abs().max().item() <= 2.0 ** -7 * want.float().abs().max().item()
+
+
+def test_inputs_are_not_modified_and_errors_are_raised(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    q, k, v = make_qkv(1, 32, 8, 300, 64, seed=2, device=gpu)
+    qb, kb, vb = t2bits(q), t2bits(k), t2bits(v)
+    cke.flash_attention_decode(q, k, v)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(t2bits(q), qb)
+    np.testing.assert_array_equal(t2bits(k), kb)
+    np.testing.assert_array_equal(t2bits(v), vb)
+    with pytest.raises(RuntimeError, match="Unsupported head size"):
+        cke.flash_attention_decode(*make_qkv(1, 8, 2, 16, 96, device=gpu))
+    with pytest.raises(RuntimeError, match="Unsupported QKV head ratio"):
+        cke.flash_attention_decode(*make_qkv(1, 10, 2, 16, 64, device=gpu))
+    with pytest.raises(RuntimeError, match="BFloat16"):
+        cke.flash_attention_decode(q.float(), k, v)
+
+
+def test_runs_on_the_current_stream(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    q, k, v = make_qkv(2, 32, 8, 512, 64, seed=4, device=gpu)
+    ref = cke.flash_attention_decode(q, k, v)
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream(device=gpu)
+    with torch.cuda.stream(s):
+        out = cke.flash_attention_decode(q, k, v)
+    s.synchronize()
+    np.testing.assert_array_equal(t2bits(out), t2bits(ref))
+
+
+# ---- BASELINE.json shapes at full size (oracle in float64, chunked over the batch)
+FULL = {
+    "c1": (1, 32, 8, 256, 64),
+    "c2_s512": (1, 32, 8, 512, 128),
+    "c2_s4096": (1, 32, 8, 4096, 128),
+    "c2_s32768": (1, 32, 8, 32768, 128),
+    "c3a": (256, 32, 8, 256, 64),
+    "c3b": (16, 32, 8, 4096, 64),
+}
+
+
+@pytest.mark.parametrize("name", list(FULL))
+def test_baseline_shapes_full_size(gpu, name):
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, QH, KVH, S, HD = FULL[name]
+    print(f"full-size {name}: B={B} S={S} HD={HD}", flush=True)
+    q, k, v = make_qkv(B, QH, KVH, S, HD, seed=42)
+    qg, kg, vg = make_qkv(B, QH, KVH, S, HD, seed=42, device=gpu)
+    out = cke.flash_attention_decode(qg, kg, vg)
+    torch.cuda.synchronize()
+    out_f = t2f32(out)
+    worst = 0.0
+    for b0 in range(0, B, 32):
+        sl = slice(b0, min(B, b0 + 32))
+        ref = attention_decode_ref(t2f32(q[sl]), t2f32(k[sl]), t2f32(v[sl]))
+        err = np.abs(out_f[sl] - ref)
+        assert np.all(err <= 2e-2 + 1.6e-2 * np.abs(ref)), f"{name}: max err {err.max()}"
+        worst = max(worst, float(err.max()))
+    print(f"  max abs err {worst:.3e}", flush=True)

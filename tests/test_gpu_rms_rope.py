@@ -1,0 +1,150 @@
+"""GPU parity: fused RMSNorm and rotary embedding (through the C ABI) against the float64
+oracle, to within 1 bf16 ulp."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_within_ulps, randn_bf16, t2bits, t2f32, to_device_like
+from oracle import precompute_freqs_cis_ref, rms_norm_ref, rot_embed_ref
+
+pytestmark = pytest.mark.gpu
+
+
+# ------------------------------------------------------------------------------ RMSNorm
+@pytest.mark.parametrize("C", [2048, 4096])
+@pytest.mark.parametrize("shape", [(1, 1), (1, 64), (64, 1), (1, 256), (2, 2048), (1, 1500)])
+def test_rms_norm_config_shapes(gpu, C, shape):
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, T = shape
+    print(f"rms_norm B={B} T={T} C={C}", flush=True)
+    x = randn_bf16((B, T, C), 100 + T)
+    w = randn_bf16((C,), 7, scale=0.02, mean=1.0)
+    out = cke.rms_norm(x.to(gpu), w.to(gpu), 1e-5)
+    torch.cuda.synchronize()
+    assert out.shape == x.shape and out.dtype == torch.bfloat16 and out.is_contiguous()
+    assert_within_ulps(out, rms_norm_ref(t2f32(x), t2f32(w), 1e-5), 1, what=f"rms {B}x{T}x{C}")
+
+
+@pytest.mark.parametrize("C", [8, 64, 100, 136, 2056, 5120, 8192, 8200, 16384])
+@pytest.mark.parametrize("rows", [3, 1100])
+def test_rms_norm_other_widths(gpu, C, rows):
+    """Widths off the fast paths: not a multiple of 8 (2-byte path), wider than the
+    register-resident limit, and tiny."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"rms_norm rows={rows} C={C}", flush=True)
+    x = randn_bf16((1, rows, C), C)
+    w = randn_bf16((C,), 8, scale=0.5, mean=0.0)
+    out = cke.rms_norm(x.to(gpu), w.to(gpu), 1e-5)
+    torch.cuda.synchronize()
+    assert_within_ulps(out, rms_norm_ref(t2f32(x), t2f32(w), 1e-5), 1, what=f"rms rows{rows} C{C}")
+
+
+def test_rms_norm_adversarial_rows(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    C = 4096
+    rows = []
+    g = torch.Generator().manual_seed(0)
+    rows.append(torch.randn(C, generator=g) * torch.logspace(-6, 6, C))          # 12 decades of range
+    rows.append(torch.full((C,), 3.0))                                           # constant
+    rows.append(torch.zeros(C))                                                  # eps only
+    onehot = torch.zeros(C); onehot[123] = -7.0; rows.append(onehot)
+    rows.append(torch.randn(C, generator=g) * 1e-4)                              # eps comparable to mean(x^2)
+    rows.append(torch.randn(C, generator=g) * 1e4)
+    alt = torch.ones(C); alt[::2] = -1.0; rows.append(alt * 255.0)
+    x = torch.stack(rows).to(torch.bfloat16).unsqueeze(0)
+    w = randn_bf16((C,), 9, scale=1.0)
+    out = cke.rms_norm(x.to(gpu), w.to(gpu), 1e-5)
+    torch.cuda.synchronize()
+    assert_within_ulps(out, rms_norm_ref(t2f32(x), t2f32(w), 1e-5), 1, what="adversarial rows")
+    assert torch.all(out[0, 2] == 0)
+    # non-contiguous input is accepted (made contiguous), weight of ones is the identity scaling
+    xt = randn_bf16((4, 2, 2048), 3).to(gpu).transpose(0, 1)
+    o2 = cke.rms_norm(xt, torch.ones(2048, dtype=torch.bfloat16, device=gpu), 1e-5)
+    assert_within_ulps(o2, rms_norm_ref(t2f32(xt), np.ones(2048), 1e-5), 1, what="transposed input")
+    with pytest.raises(RuntimeError):
+        cke.rms_norm(xt, torch.ones(100, dtype=torch.bfloat16, device=gpu), 1e-5)
+
+
+# --------------------------------------------------------------------------------- RoPE
+def _qkv_views(B, T, HD, seed, device=None):
+    """q (32 heads) and k (8 heads) as views into a fused projection output (model.py:95-97)."""
+    buf = randn_bf16((B, T, (32 + 16) * HD), seed)
+    if device is not None:
+        buf = buf.to(device)
+    q, k, _ = buf.split([32 * HD, 8 * HD, 8 * HD], dim=-1)
+    return q.view(B, T, 32, HD), k.view(B, T, 8, HD)
+
+
+@pytest.mark.parametrize("HD", [64, 128])
+@pytest.mark.parametrize("shape", [(1, 1), (64, 1), (1, 64), (1, 256), (2, 2048)])
+def test_rot_embed_config_shapes(gpu, HD, shape):
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, T = shape
+    start = 0 if T > 1 else 4321
+    print(f"rot_embed B={B} T={T} HD={HD} start={start}", flush=True)
+    tab = precompute_freqs_cis_ref(HD, start + T, theta=500000.0, use_scaled=True, scale_factor=32.0)[start:]
+    tab_g = torch.from_numpy(tab).to(gpu)
+    for x, xg in zip(_qkv_views(B, T, HD, 5), _qkv_views(B, T, HD, 5, device=gpu)):
+        assert not xg.is_contiguous() or B * T == 1
+        out = cke.rot_embed(xg, tab_g)
+        torch.cuda.synchronize()
+        assert out.shape == x.shape and out.is_contiguous() and out.dtype == torch.bfloat16
+        assert_within_ulps(out, rot_embed_ref(t2f32(x), tab), 1, what=f"rope {tuple(x.shape)}")
+        # the same values from a contiguous tensor give the same bits
+        out_c = cke.rot_embed(xg.contiguous(), tab_g)
+        np.testing.assert_array_equal(t2bits(out), t2bits(out_c))
+
+
+def test_rot_embed_identity_at_position_zero_and_norms(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    HD = 64
+    x = randn_bf16((2, 3, 8, HD), 11)
+    tab = precompute_freqs_cis_ref(HD, 3, theta=500000.0, use_scaled=True, scale_factor=32.0)
+    out = cke.rot_embed(x.to(gpu), torch.from_numpy(tab).to(gpu))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(t2bits(out[:, 0]), t2bits(x[:, 0]))   # cos 1, sin 0: bit-exact identity
+    o = t2f32(out).astype(np.float64)
+    xi = t2f32(x).astype(np.float64)
+    n_out = o[..., 0::2] ** 2 + o[..., 1::2] ** 2
+    n_in = xi[..., 0::2] ** 2 + xi[..., 1::2] ** 2
+    np.testing.assert_allclose(n_out, n_in, rtol=2.0 ** -6, atol=1e-6)   # rotation keeps pair norms (bf16 rounding)
+
+
+def test_rot_embed_cancellation_stays_within_one_ulp(gpu):
+    """Pairs built so that x0*cos - x1*sin nearly cancels: the float32 evaluation must keep the
+    error relative to the (small) result."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    HD, T = 64, 2048
+    tab = precompute_freqs_cis_ref(HD, T, theta=500000.0, use_scaled=True, scale_factor=32.0)
+    c, s = tab[:, 0::2].astype(np.float64), tab[:, 1::2].astype(np.float64)
+    x = np.zeros((1, T, 1, HD))
+    x[0, :, 0, 0::2] = s          # x0 = sin, x1 = cos  ->  y0 = sin*cos - cos*sin ~ 0 after bf16 rounding of x
+    x[0, :, 0, 1::2] = c
+    xb = torch.from_numpy(x).to(torch.bfloat16)
+    out = cke.rot_embed(xb.to(gpu), torch.from_numpy(tab).to(gpu))
+    torch.cuda.synchronize()
+    assert_within_ulps(out, rot_embed_ref(t2f32(xb), tab), 1, what="cancelling pairs")
+
+
+def test_rot_embed_pair_path_and_errors(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    # head size 6 and a token stride that is not a multiple of 8: the 4-byte path
+    buf = randn_bf16((2, 5, 3 * 6 + 2), 13)
+    x = buf[..., : 3 * 6].view(2, 5, 3, 6)
+    ang = np.random.default_rng(1).uniform(-3, 3, size=(5, 3))
+    tab = np.empty((5, 6), dtype=np.float32); tab[:, 0::2] = np.cos(ang); tab[:, 1::2] = np.sin(ang)
+    out = cke.rot_embed(to_device_like(x, gpu), torch.from_numpy(tab).to(gpu))
+    torch.cuda.synchronize()
+    assert_within_ulps(out, rot_embed_ref(t2f32(x), tab), 1, what="pair path")
+    with pytest.raises(RuntimeError):
+        cke.rot_embed(to_device_like(x, gpu), torch.from_numpy(tab[:4]).to(gpu))
+    with pytest.raises(RuntimeError):
+        cke.rot_embed(to_device_like(x, gpu).float(), torch.from_numpy(tab).to(gpu))
