@@ -33,6 +33,7 @@ for _p in (ROOT, PKG):
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 SEED = 42               # the reference's default seed (benchmark_kernel.py:126)
+FORCE_SPLITS = 0        # --splits
 
 
 def attn_bytes(B, QH, KVH, S, HD):
@@ -60,7 +61,7 @@ class AttnCase:
         self.v = [v.to(dev).transpose(1, 2) for _ in range(slots)]
         self.out = [torch.empty_like(t) for t in self.q]
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
-        self.num_splits = lib.l3_attn_choose_splits(B, KVH, S, HD, cus)
+        self.num_splits = FORCE_SPLITS or lib.l3_attn_choose_splits(B, KVH, S, HD, cus)
         self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.num_splits)
         self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
         self._args = []
@@ -139,6 +140,9 @@ def run_attention(args, torch, lib, l3, dev, name):
     else:
         raise ValueError(name)
 
+    if args.lengths:
+        lengths = [int(x) for x in args.lengths.split(",")]
+        label += f" [lengths overridden: {lengths}]"
     smax = max(lengths)
     g = torch.Generator().manual_seed(SEED)
     q = torch.randn((B, 1, QH, HD), generator=g).to(torch.bfloat16)
@@ -298,8 +302,14 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall time spent on the CPU baseline sample")
     ap.add_argument("--e2e-batch", type=int, default=1)
+    ap.add_argument("--attn-kernel", default="default", choices=["default", "mfma", "fma"],
+                    help="split-KV kernel to measure (default: the library's choice)")
+    ap.add_argument("--splits", type=int, default=0, help="force the split count (0 = the library's choice)")
+    ap.add_argument("--lengths", default="", help="comma-separated KV lengths replacing the workload's own (experiments)")
     args = ap.parse_args()
 
+    global FORCE_SPLITS
+    FORCE_SPLITS = args.splits
     if args.gpus != 1:
         print(f"bench.py: this path runs on one GPU with no sharding; --gpus {args.gpus} is not supported "
               "(every (batch, kv head) pair is independent, see DESIGN.md for how it would shard)", file=sys.stderr)
@@ -315,6 +325,10 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.attn_kernel != "default":
+        lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL,
+                               l3.L3_ATTN_KERNEL_MFMA if args.attn_kernel == "mfma" else l3.L3_ATTN_KERNEL_FMA)
+    attn_opts = {"split_kv_kernel": "mfma" if lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL, -1) else "fma"}
 
     if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):
         res = run_attention(args, torch, lib, l3, dev, args.workload)
@@ -330,6 +344,8 @@ def main():
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": res.pop("dtype"),
             "data": "synthetic", "config": res.pop("config")}
     line.update(res)
+    if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):
+        line["config"].update(attn_opts)
     line["device"] = torch.cuda.get_device_name(0)
     print(json.dumps(line), flush=True)
 

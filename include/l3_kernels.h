@@ -49,11 +49,25 @@ int l3_version(void);
 const char* l3_strerror(int code);
 
 /*
+ * Process-wide choice of the split-KV kernel l3_attn_decode launches: MFMA tiles fed through
+ * LDS (the default, chosen by measurement) or FMA dot products on the vector ALUs.  Both
+ * compute the same thing; the switch exists so that the comparison can be repeated (the
+ * reference has one kernel and no counterpart of this call).  `option` must be
+ * L3_ATTN_OPT_KERNEL; returns the previous value; a `value` other than the two kernels only
+ * queries.  The initial value is MFMA unless the environment variable L3_ATTN_IMPL is "fma".
+ * Split planning depends on the kernel, so choose before sizing workspaces.
+ */
+#define L3_ATTN_OPT_KERNEL 0
+#define L3_ATTN_KERNEL_FMA 0
+#define L3_ATTN_KERNEL_MFMA 1
+int l3_attn_set_option(int option, int value);
+
+/*
  * Split count the attention kernel would pick for this problem on a device with
  * `num_cus` compute units (<= 0: ask the current HIP device, 256 if there is none).
  * Pure integer host logic.  Replaces the fixed rule n_step = ceil(S / 64) of
- * custom_kernels.cu:243,251; the count is chosen so that B*KVH*splits workgroups fill
- * the device while every split keeps enough tokens to amortise its merge.
+ * custom_kernels.cu:243,251; the count is chosen so that the wavefronts fill the device
+ * while every split keeps at least one full tile of tokens.
  * Returns a value in [1, L3_ATTN_MAX_SPLITS], or a negative error code.
  */
 int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus);
@@ -80,7 +94,8 @@ size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int
  *   num_splits : 0 = automatic, otherwise 1..L3_ATTN_MAX_SPLITS (the kernel may use fewer
  *            when S is short); results do not depend on it beyond float32 rounding
  *   workspace : >= l3_attn_decode_workspace_bytes(...) bytes, 256-byte aligned; may be NULL
- *            when that size is 0.  Contents on entry are ignored.
+ *            when that size is 0.  Contents on entry are ignored; calls that share a
+ *            workspace must not overlap in time.
  * Supported: HD in {64, 128}, QH/KVH in {1, 2, 3, 4, 8}, S >= 1.
  */
 int l3_attn_decode(const void* q, const void* k, const void* v, void* out,

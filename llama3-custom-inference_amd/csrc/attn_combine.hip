@@ -1,0 +1,125 @@
+// Log-sum-exp combine of the split-KV partials:
+//   out = sum_i o_i 2^(m_i - M) / sum_i l_i 2^(m_i - M),   M = max_i m_i
+// over the splits i of one (batch, query head).  Takes the place of
+// custom_flash_attention_combine_kernel (custom_kernels.cu:179-223), which is meant to do
+// this but reads split 0's (max, sum) for every split (:184,201,209) and so returns the plain
+// mean of the per-split outputs; here every split contributes its own statistics.
+//
+// One workgroup of eight wavefronts per (batch, query head).  The kernel is short and
+// latency-bound, so it is built around a single round trip to memory: a wavefront issues the
+// loads of its (max, sum) pairs AND of its partial rows back to back, before it knows any
+// weight, and only then reduces.  Each wavefront merges up to 32 splits per pass with its own
+// local maximum; the eight local results are merged through LDS.
+#include "attn_common.hpp"
+
+namespace l3 {
+
+namespace {
+
+constexpr int kCombineWaves = 8;
+constexpr int kCombineRows = 32;  // splits a wavefront merges per pass (their loads are all in flight at once)
+
+template <int HD>
+__global__ void __launch_bounds__(kCombineWaves * kWaveSize)
+attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
+                    uint16_t* __restrict__ out, int QH, int n, int64_t o_sb, int64_t o_sh) {
+    constexpr int TPR = HD / 4;             // lanes covering one partial row with float4 loads
+    constexpr int RPL = kWaveSize / TPR;    // rows per wavefront-wide load (2 or 4)
+    constexpr int NLD = kCombineRows / RPL; // row loads per pass
+
+    __shared__ float s_m[kCombineWaves];
+    __shared__ float s_l[kCombineWaves];
+    __shared__ float4 s_acc[kCombineWaves][TPR];
+
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int wave = threadIdx.x / kWaveSize;
+    const int bq = blockIdx.x;
+    const float2* ml = part_ml + int64_t(bq) * n;
+    const float4* po = reinterpret_cast<const float4*>(part_o + int64_t(bq) * n * HD);
+    const int dq = lane % TPR;
+    const int sub = lane / TPR;
+
+    float m_w = kMaskedScore, l_w = 0.f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    // splits are dealt to the wavefronts in blocks of kCombineRows
+    for (int r0 = wave * kCombineRows; r0 < n; r0 += kCombineWaves * kCombineRows) {
+        // all loads of the pass first: statistics (lane j < 32 holds split r0 + j) and rows
+        float2 st = make_float2(kMaskedScore, 0.f);
+        if (lane < kCombineRows && r0 + lane < n) st = ml[r0 + lane];
+        float4 x[NLD];
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            const int r = min(r0 + u * RPL + sub, n - 1);  // rows past the end get weight 0 below
+            x[u] = po[int64_t(r) * TPR + dq];
+        }
+        const float m_new = fmaxf(m_w, wave_max(st.x));
+        const float alpha = fast_exp2(m_w - m_new);
+        const float wgt = fast_exp2(st.x - m_new);  // absent splits: 2^(-1e30 - m) = 0
+        l_w = fmaf(l_w, alpha, wave_sum(st.y * wgt));
+        acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
+        m_w = m_new;
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            const float w = __shfl(wgt, u * RPL + sub, kWaveSize);
+            acc.x = fmaf(w, x[u].x, acc.x);
+            acc.y = fmaf(w, x[u].y, acc.y);
+            acc.z = fmaf(w, x[u].z, acc.z);
+            acc.w = fmaf(w, x[u].w, acc.w);
+        }
+    }
+#pragma unroll
+    for (int off = TPR; off < kWaveSize; off <<= 1) {
+        acc.x += __shfl_xor(acc.x, off, kWaveSize);
+        acc.y += __shfl_xor(acc.y, off, kWaveSize);
+        acc.z += __shfl_xor(acc.z, off, kWaveSize);
+        acc.w += __shfl_xor(acc.w, off, kWaveSize);
+    }
+    if (lane < TPR) s_acc[wave][lane] = acc;
+    if (lane == 0) {
+        s_m[wave] = m_w;
+        s_l[wave] = l_w;
+    }
+    __syncthreads();
+
+    if (threadIdx.x < TPR) {
+        float M = s_m[0];
+#pragma unroll
+        for (int w = 1; w < kCombineWaves; ++w) M = fmaxf(M, s_m[w]);
+        float L = 0.f;
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int w = 0; w < kCombineWaves; ++w) {
+            const float e = fast_exp2(s_m[w] - M);  // idle wavefronts: 0
+            const float4 a = s_acc[w][threadIdx.x];
+            L = fmaf(s_l[w], e, L);
+            t.x = fmaf(a.x, e, t.x);
+            t.y = fmaf(a.y, e, t.y);
+            t.z = fmaf(a.z, e, t.z);
+            t.w = fmaf(a.w, e, t.w);
+        }
+        const float inv = 1.0f / L;
+        uint2 packed;
+        packed.x = pack_bf16x2(t.x * inv, t.y * inv);
+        packed.y = pack_bf16x2(t.z * inv, t.w * inv);
+        const int b = bq / QH;
+        const int qh = bq % QH;
+        *reinterpret_cast<uint2*>(out + b * o_sb + int64_t(qh) * o_sh + threadIdx.x * 4) = packed;
+    }
+}
+
+}  // namespace
+
+int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream) {
+    const dim3 grid(unsigned(p.B) * unsigned(p.QH));
+    const dim3 block(kCombineWaves * kWaveSize);
+    if (HD == 64) {
+        hipLaunchKernelGGL((attn_combine_kernel<64>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
+                           p.num_splits, p.o_sb, p.o_sh);
+    } else {
+        hipLaunchKernelGGL((attn_combine_kernel<128>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
+                           p.num_splits, p.o_sb, p.o_sh);
+    }
+    return int(hipGetLastError());
+}
+
+}  // namespace l3

@@ -1,8 +1,9 @@
-// Split-KV decode attention for gfx950 (wave64) and its log-sum-exp combine.
+// Split-KV decode attention for gfx950 (wave64) with FMA dot products on the vector ALUs.
+// This is the comparison kernel: the MFMA kernel (attn_mfma.hip) is the default because it
+// measured faster; this one stays selectable so that the comparison can be repeated.
 //
-// Takes the place of custom_flash_attention_splitkv_kernel (custom_kernels.cu:13-177)
-// and custom_flash_attention_combine_kernel (custom_kernels.cu:179-223).  What differs
-// from those, by design:
+// Takes the place of custom_flash_attention_splitkv_kernel (custom_kernels.cu:13-177).
+// What differs from it, by design:
 //   * one workgroup (4 wavefronts) owns a (batch, kv head, token range) whose length the
 //     host picks from the problem and the device, not a fixed 64 tokens;
 //   * inside a workgroup every wavefront streams its own tiles with 16-byte loads, each
@@ -11,29 +12,35 @@
 //     in registers, so each K/V byte leaves HBM once per GQA group;
 //   * each group of HD/8 lanes keeps a private online softmax (running max, sum and
 //     output slice); the groups, then the wavefronts, are merged once at the end;
-//   * partials handed to the combine are float32 and unnormalised, and the combine reads
-//     every split's own (max, sum) -- the reference reads split 0's for all of them
-//     (custom_kernels.cu:184,201,209) and rounds partials to bf16 (:163).
-#include "l3_device.hpp"
-#include "l3_host.hpp"
+//   * partials handed to the combine are float32 and unnormalised (the reference rounds
+//     them to bf16, custom_kernels.cu:163).
+#include "attn_common.hpp"
 
 namespace l3 {
 
 namespace {
 
-constexpr float kMaskedScore = -1.0e30f;  // finite stand-in for -inf (exp2 of a difference stays defined)
 constexpr int kAttnWaves = 4;
 constexpr int kAttnUnroll = 4;            // 16-byte loads of K (and of V) in flight per lane and tile
 
+// LDS hand-over between the wavefronts of a workgroup: per wave and query head of the group,
+// the running maximum (log2 units), the sum of exp2 and the unnormalised output row.
+template <int HD, int R>
+struct AttnMergeBuffers {
+    float m[kAttnWaves][R];
+    float l[kAttnWaves][R];
+    alignas(16) float o[kAttnWaves][R][HD];
+};
+
 template <int HD, int R>
 __global__ void __launch_bounds__(kAttnWaves * kWaveSize)
-attn_splitkv_kernel(const AttnParams p) {
+attn_splitkv_fma_kernel(const AttnParams p) {
     constexpr int U = kAttnUnroll;
     constexpr int LPR = HD / 8;          // lanes covering one token row
     constexpr int G = kWaveSize / LPR;   // token rows per wavefront-wide load
     constexpr int WT = U * G;            // tokens per wavefront tile
     constexpr int STEP = kAttnWaves * WT;
-    static_assert(STEP == attn_block_tile_tokens(HD), "host plan and kernel tile disagree");
+    static_assert(STEP == attn_tile_tokens(HD, kAttnImplFma), "host plan and kernel tile disagree");
 
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int wave = threadIdx.x / kWaveSize;
@@ -165,123 +172,54 @@ attn_splitkv_kernel(const AttnParams p) {
     }
 
     // ---- merge the wavefronts through LDS
-    __shared__ float s_m[kAttnWaves][R];
-    __shared__ float s_l[kAttnWaves][R];
-    __shared__ float s_o[kAttnWaves][R][HD];
+    __shared__ AttnMergeBuffers<HD, R> s_merge;
     if (g == 0) {
 #pragma unroll
         for (int h = 0; h < R; ++h) {
-            float4* dst = reinterpret_cast<float4*>(&s_o[wave][h][c * 8]);
+            float4* dst = reinterpret_cast<float4*>(&s_merge.o[wave][h][c * 8]);
             dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
             dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
         }
         if (c == 0) {
 #pragma unroll
             for (int h = 0; h < R; ++h) {
-                s_m[wave][h] = m[h];
-                s_l[wave][h] = l[h];
+                s_merge.m[wave][h] = m[h];
+                s_merge.l[wave][h] = l[h];
             }
         }
     }
     __syncthreads();
 
-    const int QHn = p.QH;
+    // Single split: the normalised bf16 output row; otherwise the unnormalised float32 partial
+    // and its (max, sum) for the combine kernel.
     for (int idx = threadIdx.x; idx < R * HD; idx += kAttnWaves * kWaveSize) {
         const int h = idx / HD;
         const int d = idx % HD;
-        float M = s_m[0][h];
+        float M = s_merge.m[0][h];
 #pragma unroll
-        for (int w = 1; w < kAttnWaves; ++w) M = fmaxf(M, s_m[w][h]);
+        for (int w = 1; w < kAttnWaves; ++w) M = fmaxf(M, s_merge.m[w][h]);
         float L = 0.f, o = 0.f;
 #pragma unroll
         for (int w = 0; w < kAttnWaves; ++w) {
-            const float e = fast_exp2(s_m[w][h] - M);
-            L = fmaf(s_l[w][h], e, L);
-            o = fmaf(s_o[w][h][d], e, o);
+            const float e = fast_exp2(s_merge.m[w][h] - M);
+            L = fmaf(s_merge.l[w][h], e, L);
+            o = fmaf(s_merge.o[w][h][d], e, o);
         }
         const int qh = kvh * R + h;
         if (p.num_splits == 1) {
             p.out[b * p.o_sb + int64_t(qh) * p.o_sh + d] = uint16_t(f32_to_bf16_bits(o / L));
         } else {
-            const int64_t row = (int64_t(b) * QHn + qh) * p.num_splits + split;
+            const int64_t row = attn_partial_row(p, b, qh, split);
             p.part_o[row * HD + d] = o;
             if (d == 0) p.part_ml[row] = make_float2(M, L);
         }
     }
 }
 
-// out = sum_i o_i 2^(m_i - M) / sum_i l_i 2^(m_i - M) over the splits of one (batch, query head).
-template <int HD>
-__global__ void __launch_bounds__(256)
-attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
-                    uint16_t* __restrict__ out, int QH, int n, int64_t o_sb, int64_t o_sh) {
-    constexpr int TPR = HD / 4;     // threads covering one partial row with float4 loads
-    constexpr int NSG = 256 / TPR;  // split groups working side by side
-    __shared__ float s_w[L3_ATTN_MAX_SPLITS];
-    __shared__ float s_red[4];
-    __shared__ float4 s_acc[NSG][TPR];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWaveSize - 1);
-    const int wave = tid / kWaveSize;
-    const int bq = blockIdx.x;
-    const int b = bq / QH;
-    const int qh = bq % QH;
-    const float2* ml = part_ml + int64_t(bq) * n;
-
-    float mx = kMaskedScore;
-    for (int i = tid; i < n; i += 256) mx = fmaxf(mx, ml[i].x);
-    mx = wave_max(mx);
-    if (lane == 0) s_red[wave] = mx;
-    __syncthreads();
-    const float M = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    __syncthreads();
-
-    float sum = 0.f;
-    for (int i = tid; i < n; i += 256) {
-        const float2 v = ml[i];
-        const float w = fast_exp2(v.x - M);
-        s_w[i] = w;
-        sum = fmaf(v.y, w, sum);
-    }
-    sum = wave_sum(sum);
-    if (lane == 0) s_red[wave] = sum;
-    __syncthreads();
-    const float L = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
-
-    const int dq = tid % TPR;
-    const int sg = tid / TPR;
-    const float4* po = reinterpret_cast<const float4*>(part_o + int64_t(bq) * n * HD) + dq;
-    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int i = sg; i < n; i += NSG) {
-        const float w = s_w[i];
-        const float4 x = po[int64_t(i) * TPR];
-        a.x = fmaf(w, x.x, a.x);
-        a.y = fmaf(w, x.y, a.y);
-        a.z = fmaf(w, x.z, a.z);
-        a.w = fmaf(w, x.w, a.w);
-    }
-    s_acc[sg][dq] = a;
-    __syncthreads();
-    if (tid < TPR) {
-        float4 t = s_acc[0][tid];
-#pragma unroll
-        for (int j = 1; j < NSG; ++j) {
-            const float4 x = s_acc[j][tid];
-            t.x += x.x; t.y += x.y; t.z += x.z; t.w += x.w;
-        }
-        const float inv = 1.0f / L;
-        uint2 packed;
-        packed.x = pack_bf16x2(t.x * inv, t.y * inv);
-        packed.y = pack_bf16x2(t.z * inv, t.w * inv);
-        *reinterpret_cast<uint2*>(out + b * o_sb + int64_t(qh) * o_sh + tid * 4) = packed;
-    }
-}
-
 template <int HD, int R>
 int launch_split(const AttnParams& p, hipStream_t stream) {
     const dim3 grid(unsigned(p.B) * unsigned(p.KVH) * unsigned(p.num_splits));
-    hipLaunchKernelGGL((attn_splitkv_kernel<HD, R>), grid, dim3(kAttnWaves * kWaveSize), 0, stream, p);
+    hipLaunchKernelGGL((attn_splitkv_fma_kernel<HD, R>), grid, dim3(kAttnWaves * kWaveSize), 0, stream, p);
     return int(hipGetLastError());
 }
 
@@ -299,18 +237,8 @@ int launch_for_ratio(const AttnParams& p, int R, hipStream_t stream) {
 
 }  // namespace
 
-int launch_attn_decode(const AttnParams& p, int HD, int R, hipStream_t stream) {
-    int err = (HD == 64) ? launch_for_ratio<64>(p, R, stream) : launch_for_ratio<128>(p, R, stream);
-    if (err != 0 || p.num_splits == 1) return err;
-    const dim3 grid(unsigned(p.B) * unsigned(p.QH));
-    if (HD == 64) {
-        hipLaunchKernelGGL((attn_combine_kernel<64>), grid, dim3(256), 0, stream, p.part_o, p.part_ml, p.out,
-                           p.QH, p.num_splits, p.o_sb, p.o_sh);
-    } else {
-        hipLaunchKernelGGL((attn_combine_kernel<128>), grid, dim3(256), 0, stream, p.part_o, p.part_ml, p.out,
-                           p.QH, p.num_splits, p.o_sb, p.o_sh);
-    }
-    return int(hipGetLastError());
+int launch_attn_splitkv_fma(const AttnParams& p, int HD, int R, hipStream_t stream) {
+    return (HD == 64) ? launch_for_ratio<64>(p, R, stream) : launch_for_ratio<128>(p, R, stream);
 }
 
 }  // namespace l3

@@ -3,7 +3,10 @@
 // Takes the place of the host launchers flash_attention_decode / rms_norm / rot_embed
 // (custom_kernels.cu:233-338, 369-389, 418-442) and of the pybind table in main.cpp:5-9.
 #include <math.h>
+#include <stdlib.h>
+#include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "l3_host.hpp"
@@ -56,18 +59,36 @@ int current_device_cus() {
     return cus;
 }
 
-AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus) {
-    const int tile = attn_block_tile_tokens(HD);
-    const int max_by_len = ceil_div(S, tile);  // a split shorter than one tile leaves waves idle
+namespace {
+std::atomic<int> g_attn_kernel{-1};  // -1: not chosen yet
+}  // namespace
+
+int attn_kernel_option() {
+    int v = g_attn_kernel.load(std::memory_order_relaxed);
+    if (v >= 0) return v;
+    const char* e = getenv("L3_ATTN_IMPL");
+    v = (e && strcmp(e, "fma") == 0) ? kAttnImplFma : kAttnImplMfma;
+    g_attn_kernel.store(v, std::memory_order_relaxed);
+    return v;
+}
+
+AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl) {
+    const int tile = attn_tile_tokens(HD, impl);
+    const int max_by_len = ceil_div(S, tile);  // a split shorter than one tile leaves lanes idle
     int splits;
     if (requested > 0) {
         splits = requested;
+    } else if (impl == kAttnImplMfma) {
+        // One 8-wave workgroup per compute unit (its loads in flight already saturate HBM); a
+        // workgroup covers heads_per_wg kv heads x (8 / heads_per_wg) splits of one batch row.
+        const int hpw = attn_mfma_heads_per_wg(KVH);
+        const int64_t wgs_per_split_group = int64_t(B) * (KVH / hpw);
+        const int64_t groups = (int64_t(num_cus) + wgs_per_split_group - 1) / wgs_per_split_group;
+        splits = int(groups * (kMfmaWaves / hpw));
     } else {
-        // Two 4-wave workgroups per compute unit keep 128 KiB of K/V in flight per CU; more
-        // splits than that only add partials for the combine to re-read.
+        // Two 4-wave workgroups per compute unit; more splits than that only add partials.
         const int64_t units = int64_t(B) * KVH;
-        const int64_t target = int64_t(num_cus) * 2;
-        splits = int((target + units - 1) / units);
+        splits = int((int64_t(num_cus) * 2 + units - 1) / units);
     }
     if (splits > max_by_len) splits = max_by_len;
     if (splits > L3_ATTN_MAX_SPLITS) splits = L3_ATTN_MAX_SPLITS;
@@ -103,18 +124,25 @@ const char* l3_strerror(int code) {
     }
 }
 
+int l3_attn_set_option(int option, int value) {
+    if (option != L3_ATTN_OPT_KERNEL) return L3_ERR_SHAPE;
+    const int prev = attn_kernel_option();
+    if (value == L3_ATTN_KERNEL_FMA || value == L3_ATTN_KERNEL_MFMA) g_attn_kernel.store(value, std::memory_order_relaxed);
+    return prev;
+}
+
 int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus) {
     if (HD != 64 && HD != 128) return L3_ERR_HEAD_SIZE;
     if (B <= 0 || KVH <= 0 || S <= 0) return L3_ERR_SHAPE;
     if (num_cus <= 0) num_cus = current_device_cus();
-    return attn_make_plan(B, KVH, S, HD, 0, num_cus).num_splits;
+    return attn_make_plan(B, KVH, S, HD, 0, num_cus, attn_kernel_option()).num_splits;
 }
 
 size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int num_splits) {
     if (check_attn_shape(B, QH, KVH, S, HD) != L3_OK) return 0;
     if (num_splits < 0 || num_splits > L3_ATTN_MAX_SPLITS) return 0;
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
-    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus);
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, attn_kernel_option());
     return attn_workspace_bytes(B, QH, HD, plan.num_splits);
 }
 
@@ -141,7 +169,8 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void*
     if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 16)) return L3_ERR_ALIGNMENT;
 
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
-    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus);
+    const int impl = attn_kernel_option();
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
     const size_t need = attn_workspace_bytes(B, QH, HD, plan.num_splits);
     if (need > 0) {
         if (!workspace || workspace_bytes < need) return L3_ERR_WORKSPACE;
@@ -154,9 +183,9 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void*
     p.v = static_cast<const uint16_t*>(v);
     p.out = static_cast<uint16_t*>(out);
     const size_t rows = size_t(B) * size_t(QH) * size_t(plan.num_splits);
-    p.part_o = static_cast<float*>(workspace);
-    p.part_ml = reinterpret_cast<float2*>(static_cast<char*>(workspace) +
-                                          round_up(rows * HD * sizeof(float), kWorkspaceAlign));
+    char* ws = static_cast<char*>(workspace);
+    p.part_o = reinterpret_cast<float*>(ws);
+    p.part_ml = reinterpret_cast<float2*>(ws + round_up(rows * HD * sizeof(float), kWorkspaceAlign));
     p.B = B; p.QH = QH; p.KVH = KVH; p.S = S;
     p.num_splits = plan.num_splits;
     p.tokens_per_split = plan.tokens_per_split;
@@ -165,7 +194,11 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void*
     p.v_sb = v_strides[0]; p.v_sh = v_strides[1]; p.v_st = v_strides[2];
     p.o_sb = out_strides[0]; p.o_sh = out_strides[1];
     p.scale_log2e = scale * 1.4426950408889634f;
-    return launch_attn_decode(p, HD, QH / KVH, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int err = (impl == kAttnImplMfma) ? launch_attn_splitkv_mfma(p, HD, QH / KVH, st)
+                                      : launch_attn_splitkv_fma(p, HD, QH / KVH, st);
+    if (err == 0 && plan.num_splits > 1) err = launch_attn_combine(p, HD, st);
+    return err == 0 ? L3_OK : L3_ERR_HIP;
 }
 
 int l3_rms_norm(const void* x, const void* w, void* y, int64_t rows, int C, float eps, void* stream) {

@@ -24,8 +24,12 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     r = (f != f) ? 0x7fc00000u : r;
     return r >> 16;
 }
+// Two f32 -> packed bf16x2 with the gfx950 v_cvt_pk_bf16_f32 (round-to-nearest-even).
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // Unpack the 8 bf16 values of a 16-byte vector into f32.

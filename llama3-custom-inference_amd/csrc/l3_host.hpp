@@ -9,18 +9,33 @@
 
 namespace l3 {
 
-// How one decode-attention call is cut into workgroups.  The reference fixes 64 tokens per
-// workgroup (custom_kernels.cu:243,251); here the cut depends on the problem and device.
+// How one decode-attention call is cut up.  The reference fixes 64 tokens per workgroup
+// (custom_kernels.cu:243,251); here the cut depends on the problem and the device.
 struct AttnPlan {
-    int num_splits;        // workgroups per (batch, kv head)
-    int tokens_per_split;  // multiple of the workgroup tile, except that the last split is shorter
+    int num_splits;        // token ranges per (batch, kv head); each yields one partial per query head
+    int tokens_per_split;  // multiple of the kernel's tile, except that the last split is shorter
 };
 
-// Tokens one workgroup consumes per main-loop trip (4 waves x 8 KiB of K+V each).
-constexpr int attn_block_tile_tokens(int HD) { return HD == 128 ? 64 : 128; }
+// The two split-KV kernels: FMA dot products on the vector ALUs, or MFMA tiles fed through LDS.
+constexpr int kAttnImplFma = 0;
+constexpr int kAttnImplMfma = 1;
+
+constexpr int kMfmaWaves = 8;  // wavefronts per workgroup of the MFMA kernel
+
+// Granularity of a split in tokens.  FMA kernel: one main-loop trip of its 4-wave workgroup
+// (4 x 8 KiB of K+V).  MFMA kernel: one tile of a wavefront (16 KiB of K+V).
+constexpr int attn_tile_tokens(int HD, int impl) {
+    return impl == kAttnImplMfma ? (HD == 128 ? 32 : 64) : (HD == 128 ? 64 : 128);
+}
+
+// Adjacent kv heads that share a workgroup of the MFMA kernel (largest power of two <= 8 dividing KVH).
+int attn_mfma_heads_per_wg(int KVH);
+
+// Which kernel l3_attn_decode uses (see l3_attn_set_option in the C ABI).
+int attn_kernel_option();
 
 // Pure integer logic (no HIP): the plan for `requested` splits (0 = automatic).
-AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus);
+AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl);
 
 // Compute units of the current device, 256 when no device can be queried.
 int current_device_cus();
@@ -42,7 +57,9 @@ struct AttnParams {
 };
 
 // Launchers: return a hipError_t cast to int (0 = success).
-int launch_attn_decode(const AttnParams& p, int HD, int R, hipStream_t stream);
+int launch_attn_splitkv_fma(const AttnParams& p, int HD, int R, hipStream_t stream);
+int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, hipStream_t stream);
+int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream);
 int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
                     bool vec_ok, hipStream_t stream);
 int launch_rot_embed(const uint16_t* x, const float* freq, uint16_t* y, int B, int T, int NH, int HD,

@@ -20,12 +20,16 @@ L3_ERR_WORKSPACE = -7
 L3_ERR_SPLITS = -8
 L3_ERR_HIP = -9
 L3_ATTN_MAX_SPLITS = 512
+L3_ATTN_OPT_KERNEL = 0
+L3_ATTN_KERNEL_FMA = 0
+L3_ATTN_KERNEL_MFMA = 1
 
 # name -> (restype, argtypes); mirrors include/l3_kernels.h line by line
 _c_i64p = ctypes.POINTER(ctypes.c_int64)
 SIGNATURES = {
     "l3_version": (ctypes.c_int, []),
     "l3_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "l3_attn_set_option": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     "l3_attn_choose_splits": (ctypes.c_int, [ctypes.c_int] * 5),
     "l3_attn_decode_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 6),
     "l3_attn_decode": (

@@ -21,6 +21,7 @@ from . import _l3lib
 __all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits"]
 
 _cu_count = {}
+_workspaces = {}  # (device index, stream handle) -> uint8 tensor
 
 
 def _fail(code: int, detail: str = ""):
@@ -49,6 +50,18 @@ def _cus(device) -> int:
         n = torch.cuda.get_device_properties(idx).multi_processor_count
         _cu_count[idx] = n
     return n
+
+
+def _workspace(device, stream_ptr: int, nbytes: int):
+    """Attention workspace (float32 partials), kept per (device, stream) and grown on demand so
+    that a decode step does not allocate.  Calls on one stream are ordered and can share it;
+    another stream gets its own."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
 
 
 def attention_num_splits(B: int, KVH: int, S: int, HD: int, num_cus: int = 256) -> int:
@@ -97,7 +110,8 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0):
             if num_splits < 0:
                 _fail(num_splits)
         ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, num_splits)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=query.device) if ws_bytes else None
+        stream_ptr = _stream_ptr(query.device)
+        ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None
         rc = lib.l3_attn_decode(
             query.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr(),
             ws.data_ptr() if ws is not None else None, ws_bytes,
@@ -106,7 +120,7 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0):
             _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
             _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
             _l3lib.i64_array((out.stride(0), out.stride(1))),
-            1.0 / math.sqrt(HD), num_splits, _stream_ptr(query.device))
+            1.0 / math.sqrt(HD), num_splits, stream_ptr)
     if rc != 0:
         _fail(rc, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
     return out

@@ -30,3 +30,15 @@ def gpu():
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     _l3lib.load()  # raises if libl3kernels.so is missing: no fallback is allowed
     return torch.device("cuda:0")
+
+
+@pytest.fixture(params=["mfma", "fma"])
+def attn_kernel(request):
+    """Run an attention test once per split-KV kernel (MFMA tiles / FMA dot products)."""
+    from custom_kernels import _l3lib as l3
+
+    lib = l3.load()
+    prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL,
+                                  l3.L3_ATTN_KERNEL_FMA if request.param == "fma" else l3.L3_ATTN_KERNEL_MFMA)
+    yield request.param
+    lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL, prev)

@@ -86,7 +86,7 @@ def test_rms_norm_and_rot_embed_argument_checks():
 
 def test_split_planning():
     lib = _l3lib.load()
-    for HD, tile in ((64, 128), (128, 64)):
+    for HD, tile in ((64, 64), (128, 32)):
         prev = 0
         for S in (1, 63, 64, 65, 256, 512, 1000, 4096, 32768, 131072):
             n = lib.l3_attn_choose_splits(1, 8, S, HD, 256)

@@ -64,11 +64,11 @@ def test_freq_table_golden(name):
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", list(cases.ATTN_CASES))
 @pytest.mark.parametrize("splits", [0, 1, 3])
-def test_gpu_attention_golden(gpu, name, splits):
+def test_gpu_attention_golden(gpu, attn_kernel, name, splits):
     from custom_kernels import custom_kernels_extension as cke
 
     q, k, v = cases.attn_inputs(name)
-    print(f"attention golden {name} splits={splits} shapes q{tuple(q.shape)} k{tuple(k.shape)}", flush=True)
+    print(f"attention golden {attn_kernel} {name} splits={splits} shapes q{tuple(q.shape)} k{tuple(k.shape)}", flush=True)
     qg, kg, vg = (to_device_like(t, gpu) for t in (q, k, v))
     assert kg.stride() == k.stride()
     out = cke.flash_attention_decode(qg, kg, vg, splits)

@@ -9,7 +9,7 @@ import torch
 from helpers import assert_attn_close, make_qkv, randn_bf16, t2bits, t2f32
 from oracle import attention_decode_ref
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("attn_kernel")]
 
 
 def _run(gpu, B, QH, KVH, S, HD, seed=42, cache_len=None, splits=0, tweak=None):
