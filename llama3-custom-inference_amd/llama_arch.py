@@ -1,0 +1,256 @@
+"""Llama-3 architecture harness around the three custom operators, for the end-to-end
+measurement (random-init weights, synthetic prompts, greedy decode).
+
+It reproduces how the reference's model.py drives the operators -- the four call sites with
+the same tensor layouts and views -- without its checkpoint loading:
+
+  RMSNorm.forward                model.py:70-72     -> ops.rms_norm(x, weight, eps)
+  CausalSelfAttention.forward    model.py:92-122    -> ops.rot_embed(q|k views of the fused qkv
+                                                       projection, freqs), static KV cache
+                                                       (maxB, L, KVH, HD) sliced and transposed,
+                                                       ops.flash_attention_decode(q, k, v) when T == 1,
+                                                       torch SDPA (causal, GQA) for the prefill
+  LLaMA3.forward                 model.py:203-232   -> embedding, blocks, final norm, tied lm_head
+                                                       on the last position, float32 logits
+  LLaMA3.generate                model.py:313-396   -> prompt mask keep, argmax when temperature is 0,
+                                                       stop-token bookkeeping with one device-side .all()
+                                                       (the reference iterates the tensor in Python, :380)
+
+GEMMs, SwiGLU, embedding and sampling stay stock PyTorch, as in the reference.  `ops` is the
+module that provides the three operators: custom_kernels.custom_kernels_extension on the GPU,
+or any object with the same three functions (the CPU baseline passes torch restatements).
+"""
+
+import math
+import time
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+
+from custom_kernels import precompute_freqs_cis
+
+
+@dataclass
+class LlamaConfig:
+    """Hyper-parameters with the reference's names and Llama-3.2-1B defaults (model.py:153-166)."""
+    block_size: int = 8192
+    vocab_size: int = 128256
+    n_layer: int = 16
+    n_head: int = 32
+    n_kv_head: int = 8
+    n_embd: int = 2048
+    hidden_dim: int = 8192
+    norm_eps: float = 1e-5
+    rope_theta: float = 500000.0
+    use_scaled_rope: bool = True
+    rope_scale_factor: float = 32.0   # model.py:29 hard-codes 8 (Llama-3.1); Llama-3.2 uses 32
+    max_model_len: int = 256
+    max_gen_batch_size: int = 256
+
+    def __post_init__(self):
+        assert self.n_kv_head <= self.n_head and self.n_head % self.n_kv_head == 0
+        assert self.n_embd % self.n_head == 0
+
+
+class _Tokenizer:
+    """Stand-in carrying what generate() reads from the HF tokenizer (model.py:307-308)."""
+    pad_id = 128004
+    stop_tokens = (128001,)
+
+
+class LlamaDecoder:
+    def __init__(self, config: LlamaConfig, ops, device, dtype=torch.bfloat16, seed: int = 42):
+        self.config, self.ops, self.device, self.dtype = config, ops, torch.device(device), dtype
+        self.tokenizer = _Tokenizer()
+        c = config
+        hd = c.n_embd // c.n_head
+        self.hd = hd
+        g = torch.Generator().manual_seed(seed)
+
+        def w(*shape):
+            return (torch.randn(shape, generator=g, dtype=torch.float32) * 0.02).to(dtype).to(self.device)
+
+        self.wte = w(c.vocab_size, c.n_embd)          # tied with the lm_head (model.py:190)
+        self.layers = []
+        for _ in range(c.n_layer):
+            self.layers.append(dict(
+                ln_1=torch.ones(c.n_embd, dtype=dtype, device=self.device),
+                c_attn=w((c.n_head + 2 * c.n_kv_head) * hd, c.n_embd),
+                c_proj=w(c.n_embd, c.n_embd),
+                ln_2=torch.ones(c.n_embd, dtype=dtype, device=self.device),
+                c_fc=w(c.hidden_dim, c.n_embd),
+                c_fc2=w(c.hidden_dim, c.n_embd),
+                mlp_proj=w(c.n_embd, c.hidden_dim),
+                cache_k=torch.zeros((c.max_gen_batch_size, c.max_model_len, c.n_kv_head, hd), dtype=dtype,
+                                    device=self.device),
+                cache_v=torch.zeros((c.max_gen_batch_size, c.max_model_len, c.n_kv_head, hd), dtype=dtype,
+                                    device=self.device),
+            ))
+        self.ln_f = torch.ones(c.n_embd, dtype=dtype, device=self.device)
+        self.freqs_cis = precompute_freqs_cis(hd, c.block_size * 2, c.rope_theta, c.use_scaled_rope,
+                                              scale_factor=c.rope_scale_factor, device=self.device)
+        self.prefill_backend = "unset"
+
+    # ------------------------------------------------------------------ attention block
+    def _attention(self, L, x, freqs_cis, start_pos):
+        c = self.config
+        B, T, C = x.shape
+        hd = self.hd
+        qkv = F.linear(x, L["c_attn"])
+        q, k, v = qkv.split([c.n_head * hd, c.n_kv_head * hd, c.n_kv_head * hd], dim=-1)
+        q, k, v = (t.view(B, T, -1, hd) for t in (q, k, v))        # strided views into qkv
+        q = self.ops.rot_embed(q, freqs_cis)
+        k = self.ops.rot_embed(k, freqs_cis)
+        L["cache_k"][:B, start_pos:start_pos + T] = k
+        L["cache_v"][:B, start_pos:start_pos + T] = v
+        k = L["cache_k"][:B, :start_pos + T]
+        v = L["cache_v"][:B, :start_pos + T]
+        q, k, v = (t.transpose(1, 2) for t in (q, k, v))           # (B, H, T|S, HD) views
+        if T > 1:
+            y = self._prefill_attention(q, k, v)
+        else:
+            y = self.ops.flash_attention_decode(q, k, v)
+        y = y.transpose(1, 2).contiguous().view(B, T, C)
+        return F.linear(y, L["c_proj"])
+
+    def _prefill_attention(self, q, k, v):
+        """Causal GQA attention for T > 1: stock PyTorch, as in the reference (model.py:114-116),
+        which pins the FLASH backend; here whichever fused backend this build offers is used."""
+        y = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+        self.prefill_backend = "torch.sdpa(default backend selection)"
+        return y
+
+    def forward(self, idx, start_pos=0):
+        """idx (B, T) token ids -> float32 logits (B, 1, vocab) of the last position."""
+        c = self.config
+        B, T = idx.shape
+        assert T <= c.block_size
+        x = F.embedding(idx, self.wte)
+        freqs_cis = self.freqs_cis[start_pos:start_pos + T]
+        for L in self.layers:
+            x = x + self._attention(L, self.ops.rms_norm(x, L["ln_1"], c.norm_eps), freqs_cis, start_pos)
+            h = self.ops.rms_norm(x, L["ln_2"], c.norm_eps)
+            x = x + F.linear(F.silu(F.linear(h, L["c_fc2"])) * F.linear(h, L["c_fc"]), L["mlp_proj"])
+        x = self.ops.rms_norm(x, self.ln_f, c.norm_eps)
+        return F.linear(x[:, [-1], :], self.wte).float()
+
+    # ------------------------------------------------------------------------- generate
+    @torch.inference_mode()
+    def generate(self, prompt_tokens, max_gen_len, temperature=0.0, echo=False, ignore_eos=False):
+        """Greedy (temperature 0) generation with the reference's bookkeeping (model.py:340-396);
+        sampling is out of scope here and raises."""
+        if temperature > 0:
+            raise NotImplementedError("the harness measures greedy decode (temperature 0)")
+        c = self.config
+        bsz = len(prompt_tokens)
+        assert bsz <= c.max_gen_batch_size
+        min_prompt_len = min(len(t) for t in prompt_tokens)
+        max_prompt_len = max(len(t) for t in prompt_tokens)
+        assert max_prompt_len <= c.block_size
+        total_len = min(c.block_size, max_gen_len + max_prompt_len)
+        assert total_len <= c.max_model_len, "KV cache too short for prompt + generation"
+        pad_id = self.tokenizer.pad_id
+        tokens = torch.full((bsz, total_len), pad_id, dtype=torch.long, device=self.device)
+        for i, t in enumerate(prompt_tokens):
+            tokens[i, :len(t)] = torch.tensor(t, dtype=torch.long, device=self.device)
+        input_text_mask = tokens != pad_id
+        stop_tokens = torch.tensor(list(self.tokenizer.stop_tokens), device=self.device)
+        eos_reached = torch.zeros(bsz, dtype=torch.bool, device=self.device)
+        prev_pos = 0
+        for cur_pos in range(min_prompt_len, total_len):
+            logits = self.forward(tokens[:, prev_pos:cur_pos], start_pos=prev_pos)
+            next_token = torch.argmax(logits[:, -1], dim=-1).reshape(-1)
+            next_token = torch.where(input_text_mask[:, cur_pos], tokens[:, cur_pos], next_token)
+            tokens[:, cur_pos] = next_token
+            eos_reached |= ~input_text_mask[:, cur_pos] & torch.isin(next_token, stop_tokens)
+            prev_pos = cur_pos
+            if not ignore_eos and bool(eos_reached.all()):
+                break
+        out = []
+        for i, toks in enumerate(tokens.tolist()):
+            start = 0 if echo else len(prompt_tokens[i])
+            toks = toks[start:len(prompt_tokens[i]) + max_gen_len]
+            for s in self.tokenizer.stop_tokens:
+                if s in toks and not ignore_eos:
+                    toks = toks[:toks.index(s)]
+            out.append(toks)
+        return out
+
+
+def random_prompts(batch, length, vocab_size, seed, exclude=(128004, 128001)):
+    """Uniform random token ids from a seeded generator, avoiding the pad and stop ids
+    (benchmark_model.py:17-43 draws from the tokenizer's vocabulary and avoids EOS)."""
+    g = torch.Generator().manual_seed(seed)
+    ids = torch.randint(0, vocab_size, (batch, length), generator=g)
+    for e in exclude:
+        ids = torch.where(ids == e, (ids + 1) % vocab_size, ids)
+    return ids.tolist()
+
+
+def timed_generate(model, batch, input_len, gen_len, seed=42, sync=None):
+    """tokens/s = gen_len * batch / wall time of generate(), prefill included (benchmark_model.py:76-82)."""
+    prompts = random_prompts(batch, input_len, model.config.vocab_size, seed)
+    if sync:
+        sync()
+    t0 = time.perf_counter()
+    out = model.generate(prompts, max_gen_len=gen_len, temperature=0.0, ignore_eos=True)
+    if sync:
+        sync()
+    dt = time.perf_counter() - t0
+    return gen_len * batch / dt, dt, out
+
+
+def bench_e2e(args, torch_mod, dev):
+    """bench.py --workload e2e: BASELINE config 5 (16 layers, hidden 2048, 32/8 heads, head_dim 64,
+    FFN 8192, vocab 128256 tied, N(0, 0.02) weights, 128 random prompt ids + 128 greedy tokens) at
+    batch 1 and 64, every RMSNorm / rotary / decode-attention call going through the HIP operators."""
+    import os
+
+    from custom_kernels import custom_kernels_extension as cke
+
+    input_len, gen_len = 128, 128
+    results = {}
+    for batch in (1, 64):
+        cfg = LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=batch)
+        model = LlamaDecoder(cfg, cke, dev)
+        model.generate(random_prompts(batch, 8, cfg.vocab_size, 1), max_gen_len=2)   # warm-up (llama3_inference.py:31-36)
+        best = None
+        for _ in range(max(1, args.steps if args.steps < 10 else 3)):
+            tps, dt, _ = timed_generate(model, batch, input_len, gen_len, sync=torch_mod.cuda.synchronize)
+            best = max(best or 0.0, tps)
+        results[batch] = {"tok_per_s": round(best, 1), "seconds": round(gen_len * batch / best, 4),
+                          "prefill": model.prefill_backend}
+        del model
+        torch_mod.cuda.empty_cache()
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import cpu_baseline
+
+        class _CpuOps:
+            rms_norm = staticmethod(cpu_baseline.rms_norm_cpu)
+            rot_embed = staticmethod(cpu_baseline.rot_embed_cpu)
+            flash_attention_decode = staticmethod(cpu_baseline.attention_cpu)
+
+        cfg = LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=1)
+        cpu_model = LlamaDecoder(cfg, _CpuOps, "cpu")
+        short = 16
+        tps, dt, _ = timed_generate(cpu_model, 1, input_len, short)
+        cpu = {"value": round(tps, 2), "unit": "tokens/s", "cores": torch_mod.get_num_threads(), "kind": "port",
+               "host_cpus": os.cpu_count(),
+               "sample": f"same architecture and prompts on the CPU with torch ops, batch 1, 128 prompt ids + "
+                         f"{short} greedy tokens in {dt:.1f} s (shortened generation)"}
+
+    v = results[1]["tok_per_s"]
+    return {
+        "metric": "e2e_greedy_decode_tokens_per_s_bs1", "value": v, "unit": "tokens/s", "steps": args.steps,
+        "ms_per_step": round(1e3 / v, 4), "dtype": "bf16",
+        "config": {"workload": "Llama-3.2-1B architecture, random init, 128 prompt ids + 128 greedy tokens, batch 1 "
+                               "(batch 64 alongside); a step is one generated token", "seed": 42},
+        "roofline": {"bound": "hbm", "achieved": round(2471628800 * v / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                     "frac": round(2471628800 * v / 1e9 / 8000.0, 4), "traffic": None,
+                     "note": "bf16 weight bytes streamed per generated token x tokens/s; launch-bound at batch 1"},
+        "cpu_baseline": cpu,
+        "e2e": {"bs1": results[1], "bs64": results[64]},
+    }

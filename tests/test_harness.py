@@ -1,0 +1,88 @@
+"""The Llama-architecture harness (llama_arch.py) that drives the operators the way the
+reference's model.py does.  CPU: cache/position logic with torch restatements of the three
+operators.  GPU: the same model with the HIP operators against the CPU run, at logits level
+(greedy token streams of a random-init model are near ties and are not compared alone)."""
+
+import numpy as np
+import pytest
+import torch
+
+import llama_arch as la
+from oracle import cpu_baseline
+
+
+class CpuOps:
+    rms_norm = staticmethod(cpu_baseline.rms_norm_cpu)
+    rot_embed = staticmethod(cpu_baseline.rot_embed_cpu)
+    flash_attention_decode = staticmethod(cpu_baseline.attention_cpu)
+
+
+def tiny_config(**kw):
+    base = dict(n_layer=2, vocab_size=1000, n_embd=256, n_head=4, n_kv_head=2, hidden_dim=512, max_model_len=48,
+                max_gen_batch_size=3, block_size=64)
+    base.update(kw)
+    return la.LlamaConfig(**base)
+
+
+def test_incremental_decode_matches_full_forward_cpu():
+    """Prefill + single-token steps through the KV cache give the logits of one causal pass:
+    pins the cache slice views, the start_pos rows of the rotary table and the T == 1 branch."""
+    torch.manual_seed(0)
+    cfg = tiny_config()
+    m = la.LlamaDecoder(cfg, CpuOps, "cpu", dtype=torch.float32)
+    ids = torch.tensor(la.random_prompts(3, 12, 900, 5))
+    with torch.inference_mode():
+        inc = [m.forward(ids[:, :8], start_pos=0)]
+        for p in range(8, 12):
+            inc.append(m.forward(ids[:, p:p + 1], start_pos=p))
+        for n, got in zip(range(8, 13), inc):
+            full = la.LlamaDecoder(cfg, CpuOps, "cpu", dtype=torch.float32).forward(ids[:, :n], start_pos=0)
+            np.testing.assert_allclose(got.numpy(), full.numpy(), rtol=2e-4, atol=2e-5)
+
+
+def test_generate_bookkeeping_cpu():
+    cfg = tiny_config()
+    m = la.LlamaDecoder(cfg, CpuOps, "cpu", dtype=torch.float32)
+    m.tokenizer.pad_id, m.tokenizer.stop_tokens = 999, (998,)
+    prompts = [[5, 6, 7, 8], [9, 10]]        # ragged: the shorter row starts generating first
+    out = m.generate(prompts, max_gen_len=5, ignore_eos=True)
+    assert [len(o) for o in out] == [5, 5]
+    echoed = m.generate(prompts, max_gen_len=5, echo=True, ignore_eos=True)
+    assert echoed[0][:4] == prompts[0] and echoed[1][:2] == prompts[1]
+    assert echoed[0][4:] == out[0][:len(echoed[0]) - 4]
+    # greedy == argmax of the logits the forward pass returns
+    with torch.inference_mode():
+        m2 = la.LlamaDecoder(cfg, CpuOps, "cpu", dtype=torch.float32)
+        lg = m2.forward(torch.tensor([prompts[1]]), start_pos=0)
+    assert out[1][0] == int(lg[0, -1].argmax())
+    tps, dt, toks = la.timed_generate(m, 2, 6, 4)
+    assert tps > 0 and len(toks) == 2 and all(len(t) == 4 for t in toks)
+    with pytest.raises(NotImplementedError):
+        m.generate(prompts, max_gen_len=2, temperature=0.6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_kv_head,n_head", [(2, 4), (1, 4), (2, 16)])
+def test_hip_operators_in_the_model_match_cpu_logits(gpu, n_kv_head, n_head):
+    from custom_kernels import custom_kernels_extension as cke
+
+    cfg = tiny_config(n_head=n_head, n_kv_head=n_kv_head, n_embd=64 * n_head)
+    print(f"harness logits: heads {n_head}/{n_kv_head}", flush=True)
+    ref = la.LlamaDecoder(cfg, CpuOps, "cpu", dtype=torch.float32, seed=7)
+    dut = la.LlamaDecoder(cfg, cke, gpu, dtype=torch.bfloat16, seed=7)
+    # same weights: the reference model holds the bf16-rounded values in float32
+    ref.wte = dut.wte.float().cpu()
+    for Lr, Ld in zip(ref.layers, dut.layers):
+        for key in ("c_attn", "c_proj", "c_fc", "c_fc2", "mlp_proj"):
+            Lr[key] = Ld[key].float().cpu()
+    ids = torch.tensor(la.random_prompts(3, 20, 900, 11))
+    with torch.inference_mode():
+        worst = 0.0
+        for (lo, hi, sp) in [(0, 16, 0), (16, 17, 16), (17, 18, 17), (18, 19, 18), (19, 20, 19)]:
+            a = ref.forward(ids[:, lo:hi], start_pos=sp)
+            b = dut.forward(ids[:, lo:hi].to(gpu), start_pos=sp).cpu()
+            scale = a.abs().max().item()
+            err = (a - b).abs().max().item()
+            worst = max(worst, err / scale)
+            assert err <= 0.04 * scale, f"step at {sp}: logits differ by {err} (scale {scale})"
+    print(f"  worst relative logit error {worst:.4f}", flush=True)
