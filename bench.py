@@ -36,6 +36,19 @@ SEED = 42               # the reference's default seed (benchmark_kernel.py:126)
 FORCE_SPLITS = 0        # --splits
 
 
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file (summaries and the copy-kernel calibration are in profiles/); keyed by (workload, kernel).
+MEASURED_TRAFFIC = {
+    # profiles/attn_splitkv_mfma_c2_sweep_hbm_traffic.md: 38.22 MB fetched + 2.51 MB written per launch
+    ("c2", "attn_splitkv_mfma_kernel"): 40730000,
+}
+
+
+def attn_kernel_name(lib):
+    from custom_kernels import _l3lib as l3
+    return "mfma" if lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL, -1) == l3.L3_ATTN_KERNEL_MFMA else "fma"
+
+
 def attn_bytes(B, QH, KVH, S, HD):
     """K+V+Q read, O written, bf16 (the reference counts K+V only: benchmark_kernel.py:48)."""
     return 2 * B * KVH * S * HD * 2 + 2 * B * QH * HD * 2
@@ -64,6 +77,7 @@ class AttnCase:
         self.num_splits = FORCE_SPLITS or lib.l3_attn_choose_splits(B, KVH, S, HD, cus)
         self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.num_splits)
         self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
+        self.part_o = self.part_ml = None
         self._args = []
         for i in range(slots):
             qt, kt, vt, ot = self.q[i], self.k[i], self.v[i], self.out[i]
@@ -78,6 +92,19 @@ class AttnCase:
         rc = self.lib.l3_attn_decode(*self._args[slot % self.slots], stream_ptr)
         if rc != 0:
             raise RuntimeError(f"l3_attn_decode failed: {rc}")
+
+    def launch_split_stage(self, slot, stream_ptr):
+        """The split-KV kernel alone (l3_attn_split), for pricing it against the roofline."""
+        a = self._args[slot % self.slots]
+        if self.part_o is None:
+            n = max(self.num_splits, 1)
+            self.part_o = self.torch.empty((self.B, self.QH, n, self.HD), dtype=self.torch.float32, device=self.ws.device)
+            self.part_ml = self.torch.empty((self.B, self.QH, n, 2), dtype=self.torch.float32, device=self.ws.device)
+        rc = self.lib.l3_attn_split(a[0], a[1], a[2], self.part_o.data_ptr(), self.part_ml.data_ptr(),
+                                    self.B, self.QH, self.KVH, self.S, self.HD, a[11], a[12], a[13], a[15],
+                                    self.num_splits, stream_ptr)
+        if rc < 0:
+            raise RuntimeError(f"l3_attn_split failed: {rc}")
 
 
 def capture_graph(torch, fn):
@@ -178,7 +205,21 @@ def run_attention(args, torch, lib, l3, dev, name):
 
     # HIP-event timing of the same replays (events on the stream the kernels run on)
     ev_ms = event_time_ms(torch, graph.replay, max(1, steps // passes_per_graph)) / passes_per_graph
-    achieved = pass_bytes / (ev_ms * 1e-3) / 1e9
+    op_gbps = pass_bytes / (ev_ms * 1e-3) / 1e9
+
+    # The dominant kernel on its own: the split-KV stage of every length, same rotation, graph-replayed.
+    def split_pass(slot):
+        sp = torch.cuda.current_stream().cuda_stream
+        for c in cases:
+            c.launch_split_stage(slot, sp)
+
+    split_pass(0)
+    sgraph = capture_graph(torch, lambda: [split_pass(s) for s in range(passes_per_graph)])
+    sgraph.replay()
+    split_ms = event_time_ms(torch, sgraph.replay, max(1, steps // passes_per_graph)) / passes_per_graph
+    achieved = pass_bytes / (split_ms * 1e-3) / 1e9
+    split_kernel = "attn_splitkv_mfma_kernel" if attn_kernel_name(lib) == "mfma" else "attn_splitkv_fma_kernel"
+    del sgraph
 
     # per-length detail: each length alone, rotating over its copies, graph-replayed
     detail = []
@@ -212,9 +253,13 @@ def run_attention(args, torch, lib, l3, dev, name):
         "config": {"workload": label, "kv_copies_per_length": slots, "accumulate": "f32", "launch": "hip graph",
                    "seed": SEED},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "attn_splitkv_kernel (+ attn_combine_kernel), per pass of the workload",
-                     "algorithmic_bytes_per_pass": pass_bytes},
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((name, split_kernel)),
+                     "kernel": split_kernel, "launches_per_pass": len(cases),
+                     "avg_launch_us": round(split_ms * 1e3 / len(cases), 3),
+                     "algorithmic_bytes_per_launch": pass_bytes // len(cases),
+                     "split_plus_combine_GBps": round(op_gbps, 1),
+                     "split_plus_combine_frac": round(op_gbps / HBM_PEAK_GBPS, 4)},
         "cpu_baseline": cpu, "per_length": detail,
     }
 
@@ -293,12 +338,35 @@ def run_rows(args, torch, lib, l3, dev, name):
     }
 
 
+def run_copy(args, torch, dev):
+    """A plain device copy of known size (torch's copy kernel): the yardstick that the FETCH_SIZE /
+    WRITE_SIZE counters are scaled by, and the practical rate of a read+write stream."""
+    nbytes = 256 << 20
+    copies = 4
+    src = [torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(i) for i in range(copies)]
+    dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(copies)]
+    gph = capture_graph(torch, lambda: [d.copy_(s_) for s_, d in zip(src, dst)])
+    gph.replay()
+    ms = event_time_ms(torch, gph.replay, 10) / copies
+    gbps = 2 * nbytes / ms / 1e6
+    return {
+        "metric": "device_copy_hbm_GBps", "value": round(gbps, 1), "unit": "GB/s",
+        "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "steps": 10 * copies, "ms_per_step": round(ms, 5),
+        "dtype": "u8", "config": {"workload": f"torch device copy, {nbytes} bytes read and {nbytes} bytes written "
+                                              "per launch (counter calibration)"},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": 2 * nbytes},
+        "cpu_baseline": None,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "e2e"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "e2e", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall time spent on the CPU baseline sample")
     ap.add_argument("--e2e-batch", type=int, default=1)
@@ -328,12 +396,14 @@ def main():
     if args.attn_kernel != "default":
         lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL,
                                l3.L3_ATTN_KERNEL_MFMA if args.attn_kernel == "mfma" else l3.L3_ATTN_KERNEL_FMA)
-    attn_opts = {"split_kv_kernel": "mfma" if lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL, -1) else "fma"}
+    attn_opts = {"split_kv_kernel": attn_kernel_name(lib)}
 
     if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):
         res = run_attention(args, torch, lib, l3, dev, args.workload)
     elif args.workload in ("rms", "rope"):
         res = run_rows(args, torch, lib, l3, dev, args.workload)
+    elif args.workload == "copy":
+        res = run_copy(args, torch, dev)
     else:
         import llama_arch
 

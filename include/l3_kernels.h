@@ -106,6 +106,32 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out,
                    float scale, int num_splits, void* stream);
 
 /*
+ * The two stages of l3_attn_decode on their own, for callers that hold one sequence's KV
+ * cache in several pieces (e.g. token ranges on different GPUs): every piece runs the split
+ * stage on its range, the partials are concatenated along the split axis, and one combine
+ * finishes the row.  Together they replace the reference's two kernels one to one
+ * (custom_kernels.cu:13-177 and :179-223); the reference has no host entry that runs them
+ * separately.
+ *
+ * l3_attn_split: same inputs as l3_attn_decode; ALWAYS writes partials, even for one split:
+ *   part_o  : (B, QH, n, HD) float32, sum_j 2^(s_j - m) v_j over the split's tokens, where
+ *             s_j = scale * log2(e) * q.k_j  (scores in log2 units) and m = max_j s_j
+ *   part_ml : (B, QH, n, 2) float32, the pair (m, sum_j 2^(s_j - m))
+ *   Returns n >= 1, the number of splits actually used (<= the requested count; the caller
+ *   sizes both buffers for the requested count, or for l3_attn_choose_splits when 0), or a
+ *   negative error code.
+ * l3_attn_combine: out[b, h, :] = sum_i part_o_i 2^(m_i - M) / sum_i l_i 2^(m_i - M),
+ *   M = max_i m_i, over i < n; out is (B, QH, 1, HD) bf16 with {batch, head} strides.
+ *   1 <= n <= L3_ATTN_MAX_SPLITS.
+ */
+int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, float* part_ml,
+                  int B, int QH, int KVH, int S, int HD,
+                  const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
+                  float scale, int num_splits, void* stream);
+int l3_attn_combine(const float* part_o, const float* part_ml, void* out, int B, int QH, int HD, int n,
+                    const int64_t out_strides[2], void* stream);
+
+/*
  * y[r, :] = bf16( x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * w[:] ), float32 inside, one rounding.
  *
  * Replaces rms_norm(input, weight, eps), custom_kernels.cu:369-389 (kernel :340-367,

@@ -206,7 +206,7 @@ attn_splitkv_fma_kernel(const AttnParams p) {
             o = fmaf(s_merge.o[w][h][d], e, o);
         }
         const int qh = kvh * R + h;
-        if (p.num_splits == 1) {
+        if (p.part_o == nullptr) {  // single split: the final output row
             p.out[b * p.o_sb + int64_t(qh) * p.o_sh + d] = uint16_t(f32_to_bf16_bits(o / L));
         } else {
             const int64_t row = attn_partial_row(p, b, qh, split);

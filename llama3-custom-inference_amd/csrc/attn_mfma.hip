@@ -226,7 +226,7 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     l_part += __shfl_xor(l_part, 32, kWaveSize);
     if (fn < R) {
         const int qh = kvh * R + fn;
-        if (p.num_splits == 1) {
+        if (p.part_o == nullptr) {  // single split: the final output row
             const float inv = 1.0f / l_part;
             uint16_t* orow = p.out + b * p.o_sb + int64_t(qh) * p.o_sh + fg * 4;
 #pragma unroll

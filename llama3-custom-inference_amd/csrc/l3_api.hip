@@ -146,12 +146,14 @@ size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int
     return attn_workspace_bytes(B, QH, HD, plan.num_splits);
 }
 
-int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void* workspace,
-                   size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
-                   const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
-                   const int64_t out_strides[2], float scale, int num_splits, void* stream) {
-    if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !out_strides)
-        return L3_ERR_NULL_POINTER;
+namespace {
+
+// Argument checks shared by l3_attn_decode and l3_attn_split (out may be absent for the latter).
+int check_attn_args(const void* q, const void* k, const void* v, const void* out, int B, int QH, int KVH, int S,
+                    int HD, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                    const int64_t* out_strides, int num_splits, bool need_out) {
+    if (!q || !k || !v || !q_strides || !k_strides || !v_strides) return L3_ERR_NULL_POINTER;
+    if (need_out && (!out || !out_strides)) return L3_ERR_NULL_POINTER;
     if (int rc = check_attn_shape(B, QH, KVH, S, HD); rc != L3_OK) return rc;
     if (num_splits < 0 || num_splits > L3_ATTN_MAX_SPLITS) return L3_ERR_SPLITS;
     // 16-byte vector loads: every row must start on a 16-byte boundary.
@@ -159,46 +161,113 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void*
     const int q_dims[2] = {B, QH};
     for (int i = 0; i < 2; ++i) {
         if (q_dims[i] == 1) continue;
-        if (q_strides[i] < 0 || out_strides[i] < 0 || q_strides[i] % 8 || out_strides[i] % 8) return L3_ERR_STRIDE;
+        if (q_strides[i] < 0 || q_strides[i] % 8) return L3_ERR_STRIDE;
+        if (need_out && (out_strides[i] < 0 || out_strides[i] % 8)) return L3_ERR_STRIDE;
     }
     const int kv_dims[3] = {B, KVH, S};
     for (int i = 0; i < 3; ++i) {
         if (kv_dims[i] == 1) continue;
         if (k_strides[i] < 0 || v_strides[i] < 0 || k_strides[i] % 8 || v_strides[i] % 8) return L3_ERR_STRIDE;
     }
-    if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 16)) return L3_ERR_ALIGNMENT;
+    if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || (need_out && !aligned(out, 16)))
+        return L3_ERR_ALIGNMENT;
+    return L3_OK;
+}
 
-    const int cus = (num_splits == 0) ? current_device_cus() : 0;
-    const int impl = attn_kernel_option();
-    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
-    const size_t need = attn_workspace_bytes(B, QH, HD, plan.num_splits);
-    if (need > 0) {
-        if (!workspace || workspace_bytes < need) return L3_ERR_WORKSPACE;
-        if (!aligned(workspace, kWorkspaceAlign)) return L3_ERR_ALIGNMENT;
-    }
-
-    AttnParams p;
+void fill_attn_params(AttnParams& p, const void* q, const void* k, const void* v, void* out, int B, int QH,
+                      int KVH, int S, const int64_t* q_strides, const int64_t* k_strides,
+                      const int64_t* v_strides, const int64_t* out_strides, float scale, const AttnPlan& plan) {
     p.q = static_cast<const uint16_t*>(q);
     p.k = static_cast<const uint16_t*>(k);
     p.v = static_cast<const uint16_t*>(v);
     p.out = static_cast<uint16_t*>(out);
-    const size_t rows = size_t(B) * size_t(QH) * size_t(plan.num_splits);
-    char* ws = static_cast<char*>(workspace);
-    p.part_o = reinterpret_cast<float*>(ws);
-    p.part_ml = reinterpret_cast<float2*>(ws + round_up(rows * HD * sizeof(float), kWorkspaceAlign));
+    p.part_o = nullptr;
+    p.part_ml = nullptr;
     p.B = B; p.QH = QH; p.KVH = KVH; p.S = S;
     p.num_splits = plan.num_splits;
     p.tokens_per_split = plan.tokens_per_split;
     p.q_sb = q_strides[0]; p.q_sh = q_strides[1];
     p.k_sb = k_strides[0]; p.k_sh = k_strides[1]; p.k_st = k_strides[2];
     p.v_sb = v_strides[0]; p.v_sh = v_strides[1]; p.v_st = v_strides[2];
-    p.o_sb = out_strides[0]; p.o_sh = out_strides[1];
+    p.o_sb = out_strides ? out_strides[0] : 0;
+    p.o_sh = out_strides ? out_strides[1] : 0;
     p.scale_log2e = scale * 1.4426950408889634f;
+}
+
+int launch_split_stage(const AttnParams& p, int HD, int R, int impl, hipStream_t st) {
+    return (impl == kAttnImplMfma) ? launch_attn_splitkv_mfma(p, HD, R, st) : launch_attn_splitkv_fma(p, HD, R, st);
+}
+
+}  // namespace
+
+int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void* workspace,
+                   size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
+                   const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
+                   const int64_t out_strides[2], float scale, int num_splits, void* stream) {
+    if (int rc = check_attn_args(q, k, v, out, B, QH, KVH, S, HD, q_strides, k_strides, v_strides, out_strides,
+                                 num_splits, true); rc != L3_OK)
+        return rc;
+    const int impl = attn_kernel_option();
+    const int cus = (num_splits == 0) ? current_device_cus() : 0;
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
+    const size_t need = attn_workspace_bytes(B, QH, HD, plan.num_splits);
+    if (need > 0) {
+        if (!workspace || workspace_bytes < need) return L3_ERR_WORKSPACE;
+        if (!aligned(workspace, kWorkspaceAlign)) return L3_ERR_ALIGNMENT;
+    }
+    AttnParams p;
+    fill_attn_params(p, q, k, v, out, B, QH, KVH, S, q_strides, k_strides, v_strides, out_strides, scale, plan);
+    if (plan.num_splits > 1) {
+        const size_t rows = size_t(B) * size_t(QH) * size_t(plan.num_splits);
+        char* ws = static_cast<char*>(workspace);
+        p.part_o = reinterpret_cast<float*>(ws);
+        p.part_ml = reinterpret_cast<float2*>(ws + round_up(rows * HD * sizeof(float), kWorkspaceAlign));
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int err = (impl == kAttnImplMfma) ? launch_attn_splitkv_mfma(p, HD, QH / KVH, st)
-                                      : launch_attn_splitkv_fma(p, HD, QH / KVH, st);
+    int err = launch_split_stage(p, HD, QH / KVH, impl, st);
     if (err == 0 && plan.num_splits > 1) err = launch_attn_combine(p, HD, st);
     return err == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, float* part_ml,
+                  int B, int QH, int KVH, int S, int HD,
+                  const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
+                  float scale, int num_splits, void* stream) {
+    if (!part_o || !part_ml) return L3_ERR_NULL_POINTER;
+    if (int rc = check_attn_args(q, k, v, nullptr, B, QH, KVH, S, HD, q_strides, k_strides, v_strides, nullptr,
+                                 num_splits, false); rc != L3_OK)
+        return rc;
+    if (!aligned(part_o, 16) || !aligned(part_ml, 8)) return L3_ERR_ALIGNMENT;
+    const int impl = attn_kernel_option();
+    const int cus = (num_splits == 0) ? current_device_cus() : 0;
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
+    AttnParams p;
+    fill_attn_params(p, q, k, v, nullptr, B, QH, KVH, S, q_strides, k_strides, v_strides, nullptr, scale, plan);
+    p.part_o = part_o;
+    p.part_ml = reinterpret_cast<float2*>(part_ml);
+    const int err = launch_split_stage(p, HD, QH / KVH, impl, static_cast<hipStream_t>(stream));
+    return err == 0 ? plan.num_splits : L3_ERR_HIP;
+}
+
+int l3_attn_combine(const float* part_o, const float* part_ml, void* out, int B, int QH, int HD, int n,
+                    const int64_t out_strides[2], void* stream) {
+    if (!part_o || !part_ml || !out || !out_strides) return L3_ERR_NULL_POINTER;
+    if (HD != 64 && HD != 128) return L3_ERR_HEAD_SIZE;
+    if (B <= 0 || QH <= 0 || int64_t(B) * QH >= (int64_t(1) << 31)) return L3_ERR_SHAPE;
+    if (n < 1 || n > L3_ATTN_MAX_SPLITS) return L3_ERR_SPLITS;
+    const int dims[2] = {B, QH};
+    for (int i = 0; i < 2; ++i) {
+        if (dims[i] != 1 && (out_strides[i] < 0 || out_strides[i] % 8)) return L3_ERR_STRIDE;
+    }
+    if (!aligned(part_o, 16) || !aligned(part_ml, 8) || !aligned(out, 16)) return L3_ERR_ALIGNMENT;
+    AttnParams p = {};
+    p.out = static_cast<uint16_t*>(out);
+    p.part_o = const_cast<float*>(part_o);
+    p.part_ml = reinterpret_cast<float2*>(const_cast<float*>(part_ml));
+    p.B = B; p.QH = QH;
+    p.num_splits = n;
+    p.o_sb = out_strides[0]; p.o_sh = out_strides[1];
+    return launch_attn_combine(p, HD, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 
 int l3_rms_norm(const void* x, const void* w, void* y, int64_t rows, int C, float eps, void* stream) {

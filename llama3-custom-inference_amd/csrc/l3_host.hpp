@@ -45,7 +45,7 @@ struct AttnParams {
     const uint16_t* k;
     const uint16_t* v;
     uint16_t* out;
-    float* part_o;    // [B][QH][num_splits][HD] unnormalised partial outputs
+    float* part_o;    // [B][QH][num_splits][HD] unnormalised partial outputs; null = write `out` directly
     float2* part_ml;  // [B][QH][num_splits] (max in log2 units, sum of exp2)
     int B, QH, KVH, S;
     int num_splits, tokens_per_split;

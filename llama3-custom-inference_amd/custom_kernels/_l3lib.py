@@ -40,6 +40,17 @@ SIGNATURES = {
          _c_i64p, _c_i64p, _c_i64p, _c_i64p,                                  # strides
          ctypes.c_float, ctypes.c_int, ctypes.c_void_p],                      # scale splits stream
     ),
+    "l3_attn_split": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v part_o part_ml
+         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,                   # B QH KVH S HD
+         _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_int, ctypes.c_void_p],
+    ),
+    "l3_attn_combine": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         _c_i64p, ctypes.c_void_p],
+    ),
     "l3_rms_norm": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float,

@@ -18,7 +18,8 @@ import torch
 
 from . import _l3lib
 
-__all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits"]
+__all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits",
+           "flash_attention_split", "flash_attention_combine"]
 
 _cu_count = {}
 _workspaces = {}  # (device index, stream handle) -> uint8 tensor
@@ -79,20 +80,9 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0):
     signature is the three tensors.
     """
     lib = _l3lib.load()
-    _require_gpu_bf16("query", query)
-    _require_gpu_bf16("keys", keys)
-    _require_gpu_bf16("values", values)
-    if query.dim() != 4 or keys.dim() != 4 or values.dim() != 4:
-        raise RuntimeError("flash_attention_decode expects 4-D query, keys and values")
+    B, QH, KVH, S, HD = _check_qkv(query, keys, values)
     if keys.device != query.device or values.device != query.device:
         raise RuntimeError("query, keys and values must be on the same device")
-    B, KVH, S, HD = keys.shape
-    QH = query.size(1)
-    if query.size(0) != B or query.size(2) != 1 or query.size(3) != HD or tuple(values.shape) != tuple(keys.shape):
-        raise RuntimeError(
-            f"shape mismatch: query {tuple(query.shape)}, keys {tuple(keys.shape)}, values {tuple(values.shape)}")
-    if query.stride(3) != 1 or keys.stride(3) != 1 or values.stride(3) != 1:
-        raise RuntimeError("the head dimension of query, keys and values must be contiguous")
     if HD not in (64, 128):
         _fail(_l3lib.L3_ERR_HEAD_SIZE, str(HD))
     if KVH == 0 or QH % KVH != 0 or (QH // KVH) not in (1, 2, 3, 4, 8):
@@ -123,6 +113,71 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0):
             1.0 / math.sqrt(HD), num_splits, stream_ptr)
     if rc != 0:
         _fail(rc, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
+    return out
+
+
+def _check_qkv(query, keys, values):
+    _require_gpu_bf16("query", query)
+    _require_gpu_bf16("keys", keys)
+    _require_gpu_bf16("values", values)
+    if query.dim() != 4 or keys.dim() != 4 or values.dim() != 4:
+        raise RuntimeError("expected 4-D query, keys and values")
+    B, KVH, S, HD = keys.shape
+    QH = query.size(1)
+    if query.size(0) != B or query.size(2) != 1 or query.size(3) != HD or tuple(values.shape) != tuple(keys.shape):
+        raise RuntimeError(
+            f"shape mismatch: query {tuple(query.shape)}, keys {tuple(keys.shape)}, values {tuple(values.shape)}")
+    if query.stride(3) != 1 or keys.stride(3) != 1 or values.stride(3) != 1:
+        raise RuntimeError("the head dimension of query, keys and values must be contiguous")
+    return B, QH, KVH, S, HD
+
+
+def flash_attention_split(query, keys, values, num_splits: int = 0):
+    """First stage of flash_attention_decode on its own (an extension; the reference runs its two
+    kernels only together, custom_kernels.cu:274-275).  Returns float32 partials
+    ``(part_o (B, QH, n, HD), part_ml (B, QH, n, 2))``: unnormalised outputs and (max, sum) per
+    split, scores in log2 units.  Partials of several token ranges of one sequence can be
+    concatenated along dim 2 and finished by flash_attention_combine."""
+    lib = _l3lib.load()
+    B, QH, KVH, S, HD = _check_qkv(query, keys, values)
+    with torch.cuda.device(query.device):
+        n_req = num_splits if num_splits > 0 else lib.l3_attn_choose_splits(B, KVH, S, HD, _cus(query.device))
+        if n_req < 0:
+            _fail(n_req)
+        part_o = torch.empty((B, QH, n_req, HD), dtype=torch.float32, device=query.device)
+        part_ml = torch.empty((B, QH, n_req, 2), dtype=torch.float32, device=query.device)
+        n = lib.l3_attn_split(
+            query.data_ptr(), keys.data_ptr(), values.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(),
+            B, QH, KVH, S, HD,
+            _l3lib.i64_array((query.stride(0), query.stride(1))),
+            _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
+            _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
+            1.0 / math.sqrt(HD), n_req, _stream_ptr(query.device))
+    if n < 0:
+        _fail(n, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
+    if n != n_req:  # the kernel laid its rows out for n splits: re-view the front of the buffers
+        part_o = part_o.flatten()[: B * QH * n * HD].view(B, QH, n, HD)
+        part_ml = part_ml.flatten()[: B * QH * n * 2].view(B, QH, n, 2)
+    return part_o, part_ml
+
+
+def flash_attention_combine(part_o, part_ml, dtype=torch.bfloat16):
+    """Second stage on its own: log-sum-exp merge of (B, QH, n, HD) / (B, QH, n, 2) float32
+    partials into a (B, QH, 1, HD) bf16 tensor laid out like empty_like of the model's query view."""
+    lib = _l3lib.load()
+    if not part_o.is_cuda or part_o.dtype != torch.float32 or part_ml.dtype != torch.float32:
+        raise RuntimeError("partials must be float32 GPU tensors")
+    B, QH, n, HD = part_o.shape
+    if tuple(part_ml.shape) != (B, QH, n, 2):
+        raise RuntimeError(f"part_ml is {tuple(part_ml.shape)}, expected {(B, QH, n, 2)}")
+    po = part_o if part_o.is_contiguous() else part_o.contiguous()
+    pm = part_ml if part_ml.is_contiguous() else part_ml.contiguous()
+    out = torch.empty((B, 1, QH, HD), dtype=dtype, device=part_o.device).transpose(1, 2)
+    with torch.cuda.device(part_o.device):
+        rc = lib.l3_attn_combine(po.data_ptr(), pm.data_ptr(), out.data_ptr(), B, QH, HD, n,
+                                 _l3lib.i64_array((out.stride(0), out.stride(1))), _stream_ptr(part_o.device))
+    if rc != 0:
+        _fail(rc, f"B={B} QH={QH} HD={HD} n={n}")
     return out
 
 

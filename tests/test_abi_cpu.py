@@ -130,3 +130,21 @@ def test_missing_library_raises(monkeypatch, tmp_path):
     monkeypatch.setattr(_l3lib, "_lib", None)
     with pytest.raises(ImportError, match="no fallback"):
         _l3lib.load()
+
+
+def test_stage_entry_points_argument_checks():
+    lib = _l3lib.load()
+    qs, ks = _l3lib.i64_array((2048, 64)), _l3lib.i64_array((131072, 64, 512))
+    assert lib.l3_attn_split(FAKE, FAKE, FAKE, None, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, None) \
+        == _l3lib.L3_ERR_NULL_POINTER
+    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 32, 8, 256, 80, qs, ks, ks, 0.125, 1, None) \
+        == _l3lib.L3_ERR_HEAD_SIZE
+    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE + 4, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, None) \
+        == _l3lib.L3_ERR_ALIGNMENT
+    assert lib.l3_attn_combine(FAKE, FAKE, None, 1, 32, 64, 4, qs, None) == _l3lib.L3_ERR_NULL_POINTER
+    assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 1, 32, 96, 4, qs, None) == _l3lib.L3_ERR_HEAD_SIZE
+    assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 1, 32, 64, 0, qs, None) == _l3lib.L3_ERR_SPLITS
+    assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 1, 32, 64, 513, qs, None) == _l3lib.L3_ERR_SPLITS
+    assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 0, 32, 64, 4, qs, None) == _l3lib.L3_ERR_SHAPE
+    assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 2, 32, 64, 4, _l3lib.i64_array((2049, 64)), None) \
+        == _l3lib.L3_ERR_STRIDE

@@ -163,3 +163,46 @@ def test_baseline_shapes_full_size(gpu, name):
         assert np.all(err <= 2e-2 + 1.6e-2 * np.abs(ref)), f"{name}: max err {err.max()}"
         worst = max(worst, float(err.max()))
     print(f"  max abs err {worst:.3e}", flush=True)
+
+
+# ---- the two stages on their own (sequence held in several pieces)
+@pytest.mark.parametrize("HD", [64, 128])
+def test_split_stage_partials_match_oracle(gpu, HD):
+    from custom_kernels import custom_kernels_extension as cke
+    from oracle import attention_split_partials_ref
+
+    B, QH, KVH, S = 2, 8, 2, 150
+    q, k, v = make_qkv(B, QH, KVH, S, HD, seed=21)
+    qg, kg, vg = make_qkv(B, QH, KVH, S, HD, seed=21, device=gpu)
+    po, pml = cke.flash_attention_split(qg, kg, vg, 1)
+    torch.cuda.synchronize()
+    assert po.shape == (B, QH, 1, HD) and pml.shape == (B, QH, 1, 2)
+    o, m, l = attention_split_partials_ref(t2f32(q), t2f32(k), t2f32(v), [0, S])
+    LOG2E = 1.4426950408889634
+    np.testing.assert_allclose(pml[:, :, 0, 0].cpu().numpy(), m[0] * LOG2E, rtol=1e-5, atol=1e-4)
+    # P is rounded to bf16 before the second product on the MFMA path: 2^-8 relative per term
+    np.testing.assert_allclose(pml[:, :, 0, 1].cpu().numpy(), l[0], rtol=2e-5)
+    np.testing.assert_allclose(po[:, :, 0].cpu().numpy(), o[0], rtol=0, atol=8e-3 * np.abs(o[0]).max())
+
+
+@pytest.mark.parametrize("HD", [64, 128])
+def test_pieces_of_a_sequence_combine_to_the_whole(gpu, HD):
+    """Token ranges processed separately (as if on different devices), partials concatenated
+    along the split axis, one combine: equals attention over the whole sequence."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, QH, KVH, S = 2, 32, 8, 1000
+    q, k, v = make_qkv(B, QH, KVH, S, HD, seed=31)
+    k[0, 3, 900] = q[0, 13, 0] * 4.0          # a dominant key in the last piece
+    qg, kg, vg = make_qkv(B, QH, KVH, S, HD, seed=31, device=gpu)
+    kg[0, 3, 900] = qg[0, 13, 0] * 4.0
+    pieces = [(0, 333), (333, 400), (400, 1000)]
+    parts = [cke.flash_attention_split(qg, kg[:, :, a:b], vg[:, :, a:b], ns) for (a, b), ns in zip(pieces, (0, 1, 5))]
+    po = torch.cat([p[0] for p in parts], dim=2)
+    pml = torch.cat([p[1] for p in parts], dim=2)
+    out = cke.flash_attention_combine(po, pml)
+    torch.cuda.synchronize()
+    assert out.shape == (B, QH, 1, HD) and out.stride() == qg.stride()
+    assert_attn_close(out, attention_decode_ref(t2f32(q), t2f32(k), t2f32(v)), what="pieces")
+    whole = cke.flash_attention_decode(qg, kg, vg)
+    assert (out.float() - whole.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, whole.float().abs().max().item())
