@@ -106,6 +106,21 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out,
                    float scale, int num_splits, void* stream);
 
 /*
+ * l3_attn_decode with the KV length read from device memory at run time (*kv_len_dev, clamped to
+ * max_S), so that one recorded launch -- a HIP graph node -- serves every step of a decode loop
+ * whose cache grows by a token per step.  `k`/`v` are views of the whole cache row range
+ * [0, max_S) with the usual {batch, head, token} strides; the split plan and the workspace are
+ * sized for max_S.  No counterpart in the reference, whose KV length is the tensor shape
+ * (custom_kernels.cu:246) and therefore fixed per launch.
+ */
+int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out,
+                          void* workspace, size_t workspace_bytes,
+                          int B, int QH, int KVH, int max_S, int HD,
+                          const int64_t q_strides[2], const int64_t k_strides[3],
+                          const int64_t v_strides[3], const int64_t out_strides[2],
+                          float scale, int num_splits, const int32_t* kv_len_dev, void* stream);
+
+/*
  * The two stages of l3_attn_decode on their own, for callers that hold one sequence's KV
  * cache in several pieces (e.g. token ranges on different GPUs): every piece runs the split
  * stage on its range, the partials are concatenated along the split axis, and one combine
@@ -156,6 +171,24 @@ int l3_rms_norm(const void* x, const void* w, void* y, int64_t rows, int C, floa
  */
 int l3_rot_embed(const void* x, const float* freq, void* y, int B, int T, int NH, int HD,
                  const int64_t x_strides[3], void* stream);
+
+/*
+ * Decode-step fusion of the two rot_embed calls and the two KV-cache slice assignments of
+ * model.py:100-106 for ONE new token per sequence, with the position read from device memory
+ * (*pos_dev) so that the launch can be replayed from a HIP graph:
+ *   q_out[b, 0, h, :]            = rope(qkv[b, h*HD : (h+1)*HD], freq_table[pos])            h < NH
+ *   cache_k[b, pos, h, :]        = rope(qkv[b, (NH+h)*HD : ...], freq_table[pos])            h < KVH
+ *   cache_v[b, pos, h, :]        = qkv[b, (NH+KVH+h)*HD : ...]                               h < KVH
+ * qkv is the fused projection output (B, 1, (NH+2*KVH)*HD) bf16 in the q|k|v order of
+ * model.py:96 with `qkv_batch_stride` elements between rows; freq_table is the whole
+ * (table_rows, HD) float32 cos/sin table; q_out is contiguous (B, 1, NH, HD); the caches are
+ * (maxB, cache_len, KVH, HD) with cache_strides = {batch, token} strides.  HD % 8 == 0, 16-byte
+ * aligned rows.  A position outside [0, min(cache_len, table_rows)) writes nothing.
+ * The rotation arithmetic is that of l3_rot_embed.  No counterpart in the reference.
+ */
+int l3_rot_embed_append(const void* qkv, const float* freq_table, void* q_out, void* cache_k, void* cache_v,
+                        const int32_t* pos_dev, int B, int NH, int KVH, int HD, int64_t qkv_batch_stride,
+                        const int64_t cache_strides[2], int cache_len, int table_rows, void* stream);
 
 #ifdef __cplusplus
 }

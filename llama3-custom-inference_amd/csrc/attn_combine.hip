@@ -22,7 +22,8 @@ constexpr int kCombineRows = 32;  // splits a wavefront merges per pass (their l
 template <int HD>
 __global__ void __launch_bounds__(kCombineWaves * kWaveSize)
 attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
-                    uint16_t* __restrict__ out, int QH, int n, int64_t o_sb, int64_t o_sh) {
+                    uint16_t* __restrict__ out, int QH, int n_rows, int64_t o_sb, int64_t o_sh,
+                    const int* __restrict__ seqlen_dev, int tokens_per_split) {
     constexpr int TPR = HD / 4;             // lanes covering one partial row with float4 loads
     constexpr int RPL = kWaveSize / TPR;    // rows per wavefront-wide load (2 or 4)
     constexpr int NLD = kCombineRows / RPL; // row loads per pass
@@ -34,8 +35,11 @@ attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int wave = threadIdx.x / kWaveSize;
     const int bq = blockIdx.x;
-    const float2* ml = part_ml + int64_t(bq) * n;
-    const float4* po = reinterpret_cast<const float4*>(part_o + int64_t(bq) * n * HD);
+    // rows are laid out for n_rows splits; with a device-side KV length only the first n hold data
+    int n = n_rows;
+    if (seqlen_dev) n = min(n_rows, max(1, (*seqlen_dev + tokens_per_split - 1) / tokens_per_split));
+    const float2* ml = part_ml + int64_t(bq) * n_rows;
+    const float4* po = reinterpret_cast<const float4*>(part_o + int64_t(bq) * n_rows * HD);
     const int dq = lane % TPR;
     const int sub = lane / TPR;
 
@@ -114,10 +118,10 @@ int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream) {
     const dim3 block(kCombineWaves * kWaveSize);
     if (HD == 64) {
         hipLaunchKernelGGL((attn_combine_kernel<64>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
-                           p.num_splits, p.o_sb, p.o_sh);
+                           p.num_splits, p.o_sb, p.o_sh, p.seqlen_dev, p.tokens_per_split);
     } else {
         hipLaunchKernelGGL((attn_combine_kernel<128>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
-                           p.num_splits, p.o_sb, p.o_sh);
+                           p.num_splits, p.o_sb, p.o_sh, p.seqlen_dev, p.tokens_per_split);
     }
     return int(hipGetLastError());
 }

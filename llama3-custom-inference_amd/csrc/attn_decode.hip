@@ -53,7 +53,9 @@ attn_splitkv_fma_kernel(const AttnParams p) {
     const int b = bid % p.B;
     const int split = bid / p.B;
     const int t_begin = split * p.tokens_per_split;
-    const int t_end = min(p.S, t_begin + p.tokens_per_split);
+    const int S = p.seqlen_dev ? min(*p.seqlen_dev, p.S) : p.S;  // wave-uniform
+    if (t_begin >= S) return;  // whole workgroup: split beyond a device-side KV length, the combine skips it
+    const int t_end = min(S, t_begin + p.tokens_per_split);
 
     // Query slices for the R heads of this group, pre-multiplied by scale*log2(e).
     float qf[R][8];

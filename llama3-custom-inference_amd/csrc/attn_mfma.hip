@@ -79,7 +79,9 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     const int split = sg * splits_per_wg + wave / heads_per_wg;
     if (split >= p.num_splits) return;  // whole wavefront; no barrier follows
     const int t_begin = split * p.tokens_per_split;
-    const int t_end = min(p.S, t_begin + p.tokens_per_split);
+    const int S = p.seqlen_dev ? min(*p.seqlen_dev, p.S) : p.S;  // wave-uniform
+    if (t_begin >= S) return;           // split beyond a device-side KV length: the combine skips it
+    const int t_end = min(S, t_begin + p.tokens_per_split);
     const float c = p.scale_log2e;
 
     // B operand of the first product: lane (head fn, k group fg) holds q[head][(m*4+fg)*8 .. +8].

@@ -184,6 +184,7 @@ void fill_attn_params(AttnParams& p, const void* q, const void* k, const void* v
     p.part_o = nullptr;
     p.part_ml = nullptr;
     p.B = B; p.QH = QH; p.KVH = KVH; p.S = S;
+    p.seqlen_dev = nullptr;
     p.num_splits = plan.num_splits;
     p.tokens_per_split = plan.tokens_per_split;
     p.q_sb = q_strides[0]; p.q_sh = q_strides[1];
@@ -200,10 +201,12 @@ int launch_split_stage(const AttnParams& p, int HD, int R, int impl, hipStream_t
 
 }  // namespace
 
-int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void* workspace,
-                   size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
-                   const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
-                   const int64_t out_strides[2], float scale, int num_splits, void* stream) {
+namespace {
+int attn_decode_impl(const void* q, const void* k, const void* v, void* out, void* workspace,
+                     size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
+                     const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
+                     const int64_t out_strides[2], float scale, int num_splits, const int* seqlen_dev,
+                     void* stream) {
     if (int rc = check_attn_args(q, k, v, out, B, QH, KVH, S, HD, q_strides, k_strides, v_strides, out_strides,
                                  num_splits, true); rc != L3_OK)
         return rc;
@@ -217,6 +220,7 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void*
     }
     AttnParams p;
     fill_attn_params(p, q, k, v, out, B, QH, KVH, S, q_strides, k_strides, v_strides, out_strides, scale, plan);
+    p.seqlen_dev = seqlen_dev;
     if (plan.num_splits > 1) {
         const size_t rows = size_t(B) * size_t(QH) * size_t(plan.num_splits);
         char* ws = static_cast<char*>(workspace);
@@ -227,6 +231,26 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void*
     int err = launch_split_stage(p, HD, QH / KVH, impl, st);
     if (err == 0 && plan.num_splits > 1) err = launch_attn_combine(p, HD, st);
     return err == 0 ? L3_OK : L3_ERR_HIP;
+}
+}  // namespace
+
+int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void* workspace,
+                   size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
+                   const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
+                   const int64_t out_strides[2], float scale, int num_splits, void* stream) {
+    return attn_decode_impl(q, k, v, out, workspace, workspace_bytes, B, QH, KVH, S, HD, q_strides, k_strides,
+                            v_strides, out_strides, scale, num_splits, nullptr, stream);
+}
+
+int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out, void* workspace,
+                          size_t workspace_bytes, int B, int QH, int KVH, int max_S, int HD,
+                          const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
+                          const int64_t out_strides[2], float scale, int num_splits, const int32_t* kv_len_dev,
+                          void* stream) {
+    if (!kv_len_dev) return L3_ERR_NULL_POINTER;
+    if (!aligned(kv_len_dev, 4)) return L3_ERR_ALIGNMENT;
+    return attn_decode_impl(q, k, v, out, workspace, workspace_bytes, B, QH, KVH, max_S, HD, q_strides, k_strides,
+                            v_strides, out_strides, scale, num_splits, kv_len_dev, stream);
 }
 
 int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, float* part_ml,
@@ -297,6 +321,26 @@ int l3_rot_embed(const void* x, const float* freq, void* y, int B, int T, int NH
     return launch_rot_embed(static_cast<const uint16_t*>(x), freq, static_cast<uint16_t*>(y), B, T, NH, HD,
                             x_strides[0], x_strides[1], x_strides[2], vec_ok,
                             static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_rot_embed_append(const void* qkv, const float* freq_table, void* q_out, void* cache_k, void* cache_v,
+                        const int32_t* pos_dev, int B, int NH, int KVH, int HD, int64_t qkv_batch_stride,
+                        const int64_t cache_strides[2], int cache_len, int table_rows, void* stream) {
+    if (!qkv || !freq_table || !q_out || !cache_k || !cache_v || !pos_dev || !cache_strides)
+        return L3_ERR_NULL_POINTER;
+    if (B <= 0 || NH <= 0 || KVH <= 0 || HD <= 0 || HD % 8 != 0 || cache_len <= 0 || table_rows <= 0)
+        return L3_ERR_SHAPE;
+    if (int64_t(B) * (NH + 2 * KVH) * (HD / 8) >= (int64_t(1) << 31)) return L3_ERR_SHAPE;
+    if (qkv_batch_stride < 0 || (B > 1 && qkv_batch_stride % 8)) return L3_ERR_STRIDE;
+    if (cache_strides[0] < 0 || cache_strides[1] < 0 || cache_strides[1] % 8 || (B > 1 && cache_strides[0] % 8))
+        return L3_ERR_STRIDE;
+    if (!aligned(qkv, 16) || !aligned(q_out, 16) || !aligned(cache_k, 16) || !aligned(cache_v, 16) ||
+        !aligned(freq_table, 16) || !aligned(pos_dev, 4))
+        return L3_ERR_ALIGNMENT;
+    return launch_rot_embed_append(static_cast<const uint16_t*>(qkv), freq_table, static_cast<uint16_t*>(q_out),
+                                   static_cast<uint16_t*>(cache_k), static_cast<uint16_t*>(cache_v), pos_dev, B, NH,
+                                   KVH, HD, qkv_batch_stride, cache_strides[0], cache_strides[1], cache_len,
+                                   table_rows, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 
 }  // extern "C"

@@ -48,6 +48,7 @@ struct AttnParams {
     float* part_o;    // [B][QH][num_splits][HD] unnormalised partial outputs; null = write `out` directly
     float2* part_ml;  // [B][QH][num_splits] (max in log2 units, sum of exp2)
     int B, QH, KVH, S;
+    const int* seqlen_dev;  // when set, the KV length is read from here (<= S, which then only bounds the plan)
     int num_splits, tokens_per_split;
     int64_t q_sb, q_sh;
     int64_t k_sb, k_sh, k_st;
@@ -64,5 +65,8 @@ int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t r
                     bool vec_ok, hipStream_t stream);
 int launch_rot_embed(const uint16_t* x, const float* freq, uint16_t* y, int B, int T, int NH, int HD,
                      int64_t sb, int64_t st, int64_t sh, bool vec_ok, hipStream_t stream);
+int launch_rot_embed_append(const uint16_t* qkv, const float* table, uint16_t* q_out, uint16_t* cache_k,
+                            uint16_t* cache_v, const int* pos_dev, int B, int NH, int KVH, int HD, int64_t qkv_sb,
+                            int64_t c_sb, int64_t c_st, int cache_len, int table_rows, hipStream_t stream);
 
 }  // namespace l3

@@ -73,7 +73,57 @@ rot_embed_pair_kernel(const uint16_t* __restrict__ x, const float* __restrict__ 
     *reinterpret_cast<uint32_t*>(y + item * 2) = rotate_pair(xw, f.x, f.y);
 }
 
+// Decode step (one new token per sequence): rotate the query and key heads of the fused qkv
+// projection at the position held in device memory, write the rotated keys and the values
+// straight into the KV cache row of that position, and return the rotated queries.  One launch
+// in place of two rot_embed calls plus the two cache slice assignments of model.py:100-106;
+// because the position is read on the device the launch can be replayed from a HIP graph.
+// One 16-byte item per thread over (batch, q|k|v head slot, chunk).
+__global__ void __launch_bounds__(kRopeThreads)
+rot_embed_append_kernel(const uint16_t* __restrict__ qkv, const float* __restrict__ table, uint16_t* __restrict__ q_out,
+                        uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
+                        const int* __restrict__ pos_dev, int total_items, int NH, int KVH, int HD, int64_t qkv_sb,
+                        int64_t c_sb, int64_t c_st, int cache_len, int table_rows) {
+    const int item = blockIdx.x * kRopeThreads + threadIdx.x;
+    if (item >= total_items) return;
+    const int pos = *pos_dev;
+    if (pos < 0 || pos >= cache_len || pos >= table_rows) return;  // never write outside the cache
+    const int vpr = HD / 8;
+    const int slots = NH + 2 * KVH;
+    const int c = item % vpr;
+    const int slot = (item / vpr) % slots;
+    const int b = item / (vpr * slots);
+    const uint4 xv = load16(qkv + b * qkv_sb + slot * HD + c * 8);
+    if (slot >= NH + KVH) {  // value head: plain copy into the cache
+        store16(cache_v + b * c_sb + pos * c_st + (slot - NH - KVH) * HD + c * 8, xv);
+        return;
+    }
+    const float4* fp = reinterpret_cast<const float4*>(table + int64_t(pos) * HD + c * 8);
+    const float4 f0 = fp[0];
+    const float4 f1 = fp[1];
+    uint4 o;
+    o.x = rotate_pair(xv.x, f0.x, f0.y);
+    o.y = rotate_pair(xv.y, f0.z, f0.w);
+    o.z = rotate_pair(xv.z, f1.x, f1.y);
+    o.w = rotate_pair(xv.w, f1.z, f1.w);
+    if (slot < NH) {
+        store16(q_out + (int64_t(b) * NH + slot) * HD + c * 8, o);
+    } else {
+        store16(cache_k + b * c_sb + pos * c_st + (slot - NH) * HD + c * 8, o);
+    }
+}
+
 }  // namespace
+
+int launch_rot_embed_append(const uint16_t* qkv, const float* table, uint16_t* q_out, uint16_t* cache_k,
+                            uint16_t* cache_v, const int* pos_dev, int B, int NH, int KVH, int HD, int64_t qkv_sb,
+                            int64_t c_sb, int64_t c_st, int cache_len, int table_rows, hipStream_t stream) {
+    const int items = B * (NH + 2 * KVH) * (HD / 8);
+    const unsigned blocks = unsigned((items + kRopeThreads - 1) / kRopeThreads);
+    hipLaunchKernelGGL(rot_embed_append_kernel, dim3(blocks), dim3(kRopeThreads), 0, stream, qkv, table, q_out,
+                       cache_k, cache_v, pos_dev, items, NH, KVH, HD, qkv_sb, c_sb, c_st, cache_len, table_rows);
+    return int(hipGetLastError());
+}
 
 int launch_rot_embed(const uint16_t* x, const float* freq, uint16_t* y, int B, int T, int NH, int HD,
                      int64_t sb, int64_t st, int64_t sh, bool vec_ok, hipStream_t stream) {

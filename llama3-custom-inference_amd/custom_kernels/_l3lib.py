@@ -40,6 +40,18 @@ SIGNATURES = {
          _c_i64p, _c_i64p, _c_i64p, _c_i64p,                                  # strides
          ctypes.c_float, ctypes.c_int, ctypes.c_void_p],                      # scale splits stream
     ),
+    "l3_attn_decode_devlen": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         _c_i64p, _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p],
+    ),
+    "l3_rot_embed_append": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64, _c_i64p, ctypes.c_int, ctypes.c_int,
+         ctypes.c_void_p],
+    ),
     "l3_attn_split": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v part_o part_ml

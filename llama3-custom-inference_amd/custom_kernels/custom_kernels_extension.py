@@ -19,7 +19,8 @@ import torch
 from . import _l3lib
 
 __all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits",
-           "flash_attention_split", "flash_attention_combine"]
+           "flash_attention_split", "flash_attention_combine", "flash_attention_decode_devlen",
+           "rot_embed_append"]
 
 _cu_count = {}
 _workspaces = {}  # (device index, stream handle) -> uint8 tensor
@@ -178,6 +179,78 @@ def flash_attention_combine(part_o, part_ml, dtype=torch.bfloat16):
                                  _l3lib.i64_array((out.stride(0), out.stride(1))), _stream_ptr(part_o.device))
     if rc != 0:
         _fail(rc, f"B={B} QH={QH} HD={HD} n={n}")
+    return out
+
+
+def flash_attention_decode_devlen(query, keys, values, kv_len, num_splits: int = 0, out=None):
+    """flash_attention_decode whose KV length is the int32 GPU scalar ``kv_len`` instead of the
+    tensor shape: ``keys`` / ``values`` are (B, KVH, L, HD) views of the whole cache and only the
+    first ``kv_len`` tokens are attended.  The launch does not depend on the length, so it can be
+    captured once in a HIP graph and replayed while the cache grows (an extension; the reference
+    takes the length from keys.size(2), custom_kernels.cu:246).  ``out`` may be supplied to keep
+    the call allocation-free under capture."""
+    lib = _l3lib.load()
+    B, QH, KVH, L, HD = _check_qkv(query, keys, values)
+    if not kv_len.is_cuda or kv_len.dtype != torch.int32 or kv_len.numel() != 1:
+        raise RuntimeError("kv_len must be a one-element int32 GPU tensor")
+    if out is None:
+        out = torch.empty_like(query)
+    with torch.cuda.device(query.device):
+        if num_splits == 0:
+            num_splits = lib.l3_attn_choose_splits(B, KVH, L, HD, _cus(query.device))
+            if num_splits < 0:
+                _fail(num_splits)
+        ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, L, HD, num_splits)
+        stream_ptr = _stream_ptr(query.device)
+        ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None
+        rc = lib.l3_attn_decode_devlen(
+            query.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws_bytes, B, QH, KVH, L, HD,
+            _l3lib.i64_array((query.stride(0), query.stride(1))),
+            _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
+            _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
+            _l3lib.i64_array((out.stride(0), out.stride(1))),
+            1.0 / math.sqrt(HD), num_splits, kv_len.data_ptr(), stream_ptr)
+    if rc != 0:
+        _fail(rc, f"B={B} QH={QH} KVH={KVH} L={L} HD={HD}")
+    return out
+
+
+def rot_embed_append(qkv, freq_table, cache_k, cache_v, pos, n_head: int, out=None):
+    """Decode-step fusion of model.py:100-106 for one new token per sequence: rotates the query
+    and key heads of ``qkv`` (B, 1, (n_head + 2*KVH)*HD, the fused projection in q|k|v order) with
+    row ``pos`` of ``freq_table`` ((rows, HD) float32), writes the rotated keys and the values
+    into ``cache_k`` / ``cache_v`` ((maxB, L, KVH, HD)) at token ``pos`` and returns the rotated
+    queries (B, 1, n_head, HD).  ``pos`` is a one-element int32 GPU tensor read by the kernel, so
+    the launch can be replayed from a HIP graph.  An extension of the reference's operator set."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("qkv", qkv)
+    _require_gpu_bf16("cache_k", cache_k)
+    _require_gpu_bf16("cache_v", cache_v)
+    if qkv.dim() != 3 or qkv.size(1) != 1 or qkv.stride(2) != 1:
+        raise RuntimeError("qkv must be (B, 1, (n_head + 2*KVH)*HD) with a contiguous last dimension")
+    if cache_k.dim() != 4 or cache_k.shape != cache_v.shape or cache_k.stride() != cache_v.stride():
+        raise RuntimeError("cache_k and cache_v must be (maxB, L, KVH, HD) tensors of the same layout")
+    maxB, L, KVH, HD = cache_k.shape
+    B = qkv.size(0)
+    if qkv.size(2) != (n_head + 2 * KVH) * HD or B > maxB:
+        raise RuntimeError(f"qkv {tuple(qkv.shape)} does not match n_head={n_head}, cache {tuple(cache_k.shape)}")
+    if cache_k.stride(3) != 1 or cache_k.stride(2) != HD:
+        raise RuntimeError("the (KVH, HD) dimensions of the cache must be contiguous")
+    if not freq_table.is_cuda or freq_table.dtype != torch.float32 or freq_table.dim() != 2 \
+            or freq_table.size(1) != HD or not freq_table.is_contiguous():
+        raise RuntimeError("freq_table must be a contiguous (rows, HD) float32 GPU tensor")
+    if not pos.is_cuda or pos.dtype != torch.int32 or pos.numel() != 1:
+        raise RuntimeError("pos must be a one-element int32 GPU tensor")
+    if out is None:
+        out = torch.empty((B, 1, n_head, HD), dtype=qkv.dtype, device=qkv.device)
+    with torch.cuda.device(qkv.device):
+        rc = lib.l3_rot_embed_append(qkv.data_ptr(), freq_table.data_ptr(), out.data_ptr(), cache_k.data_ptr(),
+                                     cache_v.data_ptr(), pos.data_ptr(), B, n_head, KVH, HD, qkv.stride(0),
+                                     _l3lib.i64_array((cache_k.stride(0), cache_k.stride(1))), L,
+                                     freq_table.size(0), _stream_ptr(qkv.device))
+    if rc != 0:
+        _fail(rc, f"B={B} NH={n_head} KVH={KVH} HD={HD}")
     return out
 
 

@@ -91,6 +91,7 @@ class LlamaDecoder:
         self.freqs_cis = precompute_freqs_cis(hd, c.block_size * 2, c.rope_theta, c.use_scaled_rope,
                                               scale_factor=c.rope_scale_factor, device=self.device)
         self.prefill_backend = "unset"
+        self._graphs = {}
 
     # ------------------------------------------------------------------ attention block
     def _attention(self, L, x, freqs_cis, start_pos):
@@ -137,6 +138,56 @@ class LlamaDecoder:
 
     # ------------------------------------------------------------------------- generate
     @torch.inference_mode()
+    def generate_graphed(self, prompt_tokens, max_gen_len, echo=False, ignore_eos=False):
+        """generate() with the per-token loop replayed from a HIP graph: prefill of the common
+        prompt prefix runs eagerly (model.py:365 with T = min_prompt_len), every later position is
+        one graph replay.  Needs ops with rot_embed_append / flash_attention_decode_devlen."""
+        c = self.config
+        bsz = len(prompt_tokens)
+        min_prompt_len = min(len(t) for t in prompt_tokens)
+        max_prompt_len = max(len(t) for t in prompt_tokens)
+        total_len = min(c.block_size, max_gen_len + max_prompt_len)
+        assert bsz <= c.max_gen_batch_size and total_len <= c.max_model_len
+        key = (bsz, total_len)
+        loop = self._graphs.get(key)
+        if loop is None:
+            loop = GraphedDecodeLoop(self, bsz, total_len)
+            self._graphs[key] = loop
+        pad_id = self.tokenizer.pad_id
+        host = torch.full((bsz, total_len), pad_id, dtype=torch.long)
+        for i, t in enumerate(prompt_tokens):
+            host[i, :len(t)] = torch.tensor(t, dtype=torch.long)
+        loop.tokens.copy_(host)
+        loop.text_mask.copy_(host != pad_id)
+        loop.eos.zero_()
+        # position min_prompt_len: eager prefill + the usual bookkeeping
+        logits = self.forward(loop.tokens[:, :min_prompt_len], start_pos=0)
+        nxt = torch.argmax(logits[:, -1], dim=-1)
+        if min_prompt_len < total_len:
+            keep = loop.text_mask[:, min_prompt_len]
+            nxt = torch.where(keep, loop.tokens[:, min_prompt_len], nxt)
+            loop.tokens[:, min_prompt_len] = nxt
+            loop.eos |= ~keep & torch.isin(nxt, loop.stop)
+        loop.tok.copy_(nxt.unsqueeze(1))
+        loop.pos.fill_(min_prompt_len)
+        loop.kv_len.fill_(min_prompt_len + 1)
+        if loop.graph is None:
+            loop.capture()
+        for cur_pos in range(min_prompt_len + 1, total_len):
+            loop.graph.replay()
+            if not ignore_eos and (cur_pos - min_prompt_len) % 16 == 0 and bool(loop.eos.all()):
+                break
+        out = []
+        for i, toks in enumerate(loop.tokens.tolist()):
+            start = 0 if echo else len(prompt_tokens[i])
+            toks = toks[start:len(prompt_tokens[i]) + max_gen_len]
+            for s_ in self.tokenizer.stop_tokens:
+                if s_ in toks and not ignore_eos:
+                    toks = toks[:toks.index(s_)]
+            out.append(toks)
+        return out
+
+    @torch.inference_mode()
     def generate(self, prompt_tokens, max_gen_len, temperature=0.0, echo=False, ignore_eos=False):
         """Greedy (temperature 0) generation with the reference's bookkeeping (model.py:340-396);
         sampling is out of scope here and raises."""
@@ -178,6 +229,75 @@ class LlamaDecoder:
         return out
 
 
+class GraphedDecodeLoop:
+    """The single-token decode step of LlamaDecoder recorded once as a HIP graph and replayed per
+    generated token (the reference's loop, model.py:363-381, launches ~450 kernels per token from
+    Python; at batch 1 that, not the GPU, sets the pace).
+
+    What makes the step replayable: the token position lives in device memory.  The fused
+    rot_embed_append operator writes K/V at that position, flash_attention_decode_devlen reads the
+    KV length from it, and the bookkeeping of generate() (prompt-mask keep, token store, stop
+    flags, position increment) is expressed with fixed-shape torch ops on device tensors.
+    """
+
+    def __init__(self, model: "LlamaDecoder", batch: int, total_len: int):
+        import torch as _t
+
+        self.m, self.B, self.total_len = model, batch, total_len
+        dev = model.device
+        self.tokens = _t.zeros((batch, total_len), dtype=_t.long, device=dev)
+        self.text_mask = _t.zeros((batch, total_len), dtype=_t.bool, device=dev)
+        self.tok = _t.zeros((batch, 1), dtype=_t.long, device=dev)     # token fed to this step
+        self.pos = _t.zeros(1, dtype=_t.int32, device=dev)             # its position = cache row written
+        self.kv_len = _t.ones(1, dtype=_t.int32, device=dev)           # pos + 1
+        self.eos = _t.zeros(batch, dtype=_t.bool, device=dev)
+        self.stop = _t.tensor(list(model.tokenizer.stop_tokens), device=dev)
+        self.graph = None
+
+    def step(self):
+        m, c, B = self.m, self.m.config, self.B
+        ops = m.ops
+        x = F.embedding(self.tok, m.wte)
+        for L in m.layers:
+            h = ops.rms_norm(x, L["ln_1"], c.norm_eps)
+            qkv = F.linear(h, L["c_attn"])
+            q = ops.rot_embed_append(qkv, m.freqs_cis, L["cache_k"], L["cache_v"], self.pos, c.n_head)
+            y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
+                                                  L["cache_v"][:B].transpose(1, 2), self.kv_len)
+            x = x + F.linear(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"])
+            h = ops.rms_norm(x, L["ln_2"], c.norm_eps)
+            x = x + F.linear(F.silu(F.linear(h, L["c_fc2"])) * F.linear(h, L["c_fc"]), L["mlp_proj"])
+        x = ops.rms_norm(x, m.ln_f, c.norm_eps)
+        logits = F.linear(x[:, -1], m.wte).float()
+        nxt = torch.argmax(logits, dim=-1)
+        # generate() bookkeeping (model.py:373-378) at position pos + 1, all on the device
+        cur = (self.pos + 1).long().clamp_(max=self.total_len - 1)
+        keep = self.text_mask.index_select(1, cur).squeeze(1)
+        nxt = torch.where(keep, self.tokens.index_select(1, cur).squeeze(1), nxt)
+        self.tokens.index_copy_(1, cur, nxt.unsqueeze(1))
+        self.eos |= ~keep & torch.isin(nxt, self.stop)
+        self.tok.copy_(nxt.unsqueeze(1))
+        self.pos += 1
+        self.kv_len += 1
+
+    def capture(self):
+        side = torch.cuda.Stream(device=self.m.device)
+        saved = [t.clone() for t in (self.tokens, self.tok, self.pos, self.kv_len, self.eos)]
+        side.wait_stream(torch.cuda.current_stream(self.m.device))
+        with torch.cuda.stream(side):
+            self.step()   # warm-up outside capture: workspaces, hipBLASLt handles, allocator
+        torch.cuda.current_stream(self.m.device).wait_stream(side)
+        torch.cuda.synchronize(self.m.device)
+        for t, s in zip((self.tokens, self.tok, self.pos, self.kv_len, self.eos), saved):
+            t.copy_(s)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.step()
+        for t, s in zip((self.tokens, self.tok, self.pos, self.kv_len, self.eos), saved):
+            t.copy_(s)   # capture does not execute, but keep the state explicit
+        torch.cuda.synchronize(self.m.device)
+
+
 def random_prompts(batch, length, vocab_size, seed, exclude=(128004, 128001)):
     """Uniform random token ids from a seeded generator, avoiding the pad and stop ids
     (benchmark_model.py:17-43 draws from the tokenizer's vocabulary and avoids EOS)."""
@@ -188,13 +308,16 @@ def random_prompts(batch, length, vocab_size, seed, exclude=(128004, 128001)):
     return ids.tolist()
 
 
-def timed_generate(model, batch, input_len, gen_len, seed=42, sync=None):
+def timed_generate(model, batch, input_len, gen_len, seed=42, sync=None, graphed=False):
     """tokens/s = gen_len * batch / wall time of generate(), prefill included (benchmark_model.py:76-82)."""
     prompts = random_prompts(batch, input_len, model.config.vocab_size, seed)
     if sync:
         sync()
     t0 = time.perf_counter()
-    out = model.generate(prompts, max_gen_len=gen_len, temperature=0.0, ignore_eos=True)
+    if graphed:
+        out = model.generate_graphed(prompts, max_gen_len=gen_len, ignore_eos=True)
+    else:
+        out = model.generate(prompts, max_gen_len=gen_len, temperature=0.0, ignore_eos=True)
     if sync:
         sync()
     dt = time.perf_counter() - t0
@@ -214,13 +337,23 @@ def bench_e2e(args, torch_mod, dev):
     for batch in (1, 64):
         cfg = LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=batch)
         model = LlamaDecoder(cfg, cke, dev)
-        model.generate(random_prompts(batch, 8, cfg.vocab_size, 1), max_gen_len=2)   # warm-up (llama3_inference.py:31-36)
-        best = None
-        for _ in range(max(1, args.steps if args.steps < 10 else 3)):
-            tps, dt, _ = timed_generate(model, batch, input_len, gen_len, sync=torch_mod.cuda.synchronize)
-            best = max(best or 0.0, tps)
-        results[batch] = {"tok_per_s": round(best, 1), "seconds": round(gen_len * batch / best, 4),
-                          "prefill": model.prefill_backend}
+        rec = {}
+        for mode in ("eager", "graphed"):
+            graphed = mode == "graphed"
+            # warm-up generate, as llama3_inference.py:31-36 does (for the graphed loop it also records the graph)
+            timed_generate(model, batch, input_len, gen_len if graphed else 2, seed=1, graphed=graphed)
+            best, toks = 0.0, None
+            for _ in range(3):
+                tps, dt, out = timed_generate(model, batch, input_len, gen_len, sync=torch_mod.cuda.synchronize,
+                                              graphed=graphed)
+                if tps > best:
+                    best, toks = tps, out
+            rec[mode] = {"tok_per_s": round(best, 1), "seconds": round(gen_len * batch / best, 4)}
+            rec[mode + "_tokens"] = toks
+        same = sum(a == b for ra, rb in zip(rec.pop("eager_tokens"), rec.pop("graphed_tokens")) for a, b in zip(ra, rb))
+        rec["graphed_vs_eager_same_tokens"] = f"{same}/{batch * gen_len}"
+        rec["prefill"] = model.prefill_backend
+        results[batch] = rec
         del model
         torch_mod.cuda.empty_cache()
 
@@ -242,12 +375,13 @@ def bench_e2e(args, torch_mod, dev):
                "sample": f"same architecture and prompts on the CPU with torch ops, batch 1, 128 prompt ids + "
                          f"{short} greedy tokens in {dt:.1f} s (shortened generation)"}
 
-    v = results[1]["tok_per_s"]
+    v = results[1]["graphed"]["tok_per_s"]
     return {
         "metric": "e2e_greedy_decode_tokens_per_s_bs1", "value": v, "unit": "tokens/s", "steps": args.steps,
         "ms_per_step": round(1e3 / v, 4), "dtype": "bf16",
         "config": {"workload": "Llama-3.2-1B architecture, random init, 128 prompt ids + 128 greedy tokens, batch 1 "
-                               "(batch 64 alongside); a step is one generated token", "seed": 42},
+                               "(batch 64 alongside); a step is one generated token; decode loop replayed from a "
+                               "HIP graph (the eager loop is reported next to it)", "seed": 42},
         "roofline": {"bound": "hbm", "achieved": round(2471628800 * v / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
                      "frac": round(2471628800 * v / 1e9 / 8000.0, 4), "traffic": None,
                      "note": "bf16 weight bytes streamed per generated token x tokens/s; launch-bound at batch 1"},

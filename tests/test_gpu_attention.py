@@ -206,3 +206,23 @@ def test_pieces_of_a_sequence_combine_to_the_whole(gpu, HD):
     assert_attn_close(out, attention_decode_ref(t2f32(q), t2f32(k), t2f32(v)), what="pieces")
     whole = cke.flash_attention_decode(qg, kg, vg)
     assert (out.float() - whole.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, whole.float().abs().max().item())
+
+
+# ---- KV length read from device memory (one recorded launch serves a growing cache)
+@pytest.mark.parametrize("HD,B,L", [(64, 1, 256), (64, 3, 300), (128, 2, 1024), (64, 64, 256)])
+def test_device_side_kv_length(gpu, HD, B, L):
+    from custom_kernels import custom_kernels_extension as cke
+
+    QH, KVH = 32, 8
+    q, k, v = make_qkv(B, QH, KVH, L, HD, seed=41)
+    qg, kg, vg = make_qkv(B, QH, KVH, L, HD, seed=41, device=gpu)
+    kv_len = torch.zeros(1, dtype=torch.int32, device=gpu)
+    for S in (1, 2, 63, 64, 65, 129, L - 1, L):
+        kv_len.fill_(S)
+        out = cke.flash_attention_decode_devlen(qg, kg, vg, kv_len)
+        torch.cuda.synchronize()
+        ref = attention_decode_ref(t2f32(q), t2f32(k[:, :, :S]), t2f32(v[:, :, :S]))
+        assert_attn_close(out, ref, what=f"devlen S={S} of L={L}")
+        # same bits as the shape-driven call planned for the same cache length
+        splits = cke.attention_num_splits(B, KVH, L, HD, torch.cuda.get_device_properties(gpu).multi_processor_count)
+        np.testing.assert_array_equal(t2bits(out), t2bits(cke.flash_attention_decode_devlen(qg, kg, vg, kv_len, splits)))

@@ -148,3 +148,41 @@ def test_rot_embed_pair_path_and_errors(gpu):
         cke.rot_embed(to_device_like(x, gpu), torch.from_numpy(tab[:4]).to(gpu))
     with pytest.raises(RuntimeError):
         cke.rot_embed(to_device_like(x, gpu).float(), torch.from_numpy(tab).to(gpu))
+
+
+@pytest.mark.parametrize("HD,NH,KVH", [(64, 32, 8), (128, 32, 8), (64, 4, 4)])
+def test_rot_embed_append_fuses_rope_and_cache_write(gpu, HD, NH, KVH):
+    """Against the unfused sequence of model.py:100-106: rot_embed(q), rot_embed(k), two cache
+    slice assignments -- q, the cache row at `pos`, and every other cache row (untouched)."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, maxB, L = 3, 4, 40
+    tab = precompute_freqs_cis_ref(HD, 64, theta=500000.0, use_scaled=True, scale_factor=32.0)
+    tab_g = torch.from_numpy(tab).to(gpu)
+    qkv = randn_bf16((B, 1, (NH + 2 * KVH) * HD), 17)
+    ck0 = randn_bf16((maxB, L, KVH, HD), 18)
+    cv0 = randn_bf16((maxB, L, KVH, HD), 19)
+    pos = torch.zeros(1, dtype=torch.int32, device=gpu)
+    for p in (0, 7, L - 1):
+        ck, cv = ck0.to(gpu), cv0.to(gpu)
+        pos.fill_(p)
+        q_out = cke.rot_embed_append(qkv.to(gpu), tab_g, ck, cv, pos, NH)
+        torch.cuda.synchronize()
+        q, k, v = qkv.split([NH * HD, KVH * HD, KVH * HD], dim=-1)
+        q, k, v = (t.view(B, 1, -1, HD) for t in (q, k, v))
+        assert q_out.shape == (B, 1, NH, HD) and q_out.is_contiguous()
+        assert_within_ulps(q_out, rot_embed_ref(t2f32(q), tab[p:p + 1]), 1, what="q")
+        assert_within_ulps(ck[:B, p:p + 1].contiguous(), rot_embed_ref(t2f32(k), tab[p:p + 1]), 1, what="k row")
+        np.testing.assert_array_equal(t2bits(cv[:B, p]), t2bits(v[:, 0]))
+        # bit-identical to the unfused operator
+        np.testing.assert_array_equal(t2bits(q_out), t2bits(cke.rot_embed(q.to(gpu), tab_g[p:p + 1])))
+        keep = [i for i in range(L) if i != p]
+        np.testing.assert_array_equal(t2bits(ck[:, keep]), t2bits(ck0[:, keep]))
+        np.testing.assert_array_equal(t2bits(cv[:, keep]), t2bits(cv0[:, keep]))
+        np.testing.assert_array_equal(t2bits(ck[B:]), t2bits(ck0[B:]))
+    # a position outside the cache writes nothing
+    ck, cv = ck0.to(gpu), cv0.to(gpu)
+    pos.fill_(L)
+    cke.rot_embed_append(qkv.to(gpu), tab_g, ck, cv, pos, NH)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(t2bits(ck), t2bits(ck0))
