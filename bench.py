@@ -73,9 +73,10 @@ class AttnCase:
         self.k = [k.to(dev).transpose(1, 2) for _ in range(slots)]
         self.v = [v.to(dev).transpose(1, 2) for _ in range(slots)]
         self.out = [torch.empty_like(t) for t in self.q]
-        cus = torch.cuda.get_device_properties(dev).multi_processor_count
-        self.num_splits = FORCE_SPLITS or lib.l3_attn_choose_splits(B, KVH, S, HD, cus)
-        self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.num_splits)
+        # 0 = the library plans for the current device (split count and kernel form)
+        self.req_splits = FORCE_SPLITS
+        self.num_splits = FORCE_SPLITS or lib.l3_attn_choose_splits(B, KVH, S, HD, 0)
+        self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.req_splits)
         self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
         self.part_o = self.part_ml = None
         self._args = []
@@ -86,7 +87,7 @@ class AttnCase:
                 B, QH, KVH, S, HD,
                 l3.i64_array((qt.stride(0), qt.stride(1))), l3.i64_array((kt.stride(0), kt.stride(1), kt.stride(2))),
                 l3.i64_array((vt.stride(0), vt.stride(1), vt.stride(2))), l3.i64_array((ot.stride(0), ot.stride(1))),
-                1.0 / math.sqrt(HD), self.num_splits))
+                1.0 / math.sqrt(HD), self.req_splits))
 
     def launch(self, slot, stream_ptr):
         rc = self.lib.l3_attn_decode(*self._args[slot % self.slots], stream_ptr)
@@ -102,7 +103,7 @@ class AttnCase:
             self.part_ml = self.torch.empty((self.B, self.QH, n, 2), dtype=self.torch.float32, device=self.ws.device)
         rc = self.lib.l3_attn_split(a[0], a[1], a[2], self.part_o.data_ptr(), self.part_ml.data_ptr(),
                                     self.B, self.QH, self.KVH, self.S, self.HD, a[11], a[12], a[13], a[15],
-                                    self.num_splits, stream_ptr)
+                                    self.req_splits, stream_ptr)
         if rc < 0:
             raise RuntimeError(f"l3_attn_split failed: {rc}")
 

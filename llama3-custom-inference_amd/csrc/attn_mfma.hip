@@ -41,7 +41,13 @@ typedef __attribute__((ext_vector_type(8))) short s16x8_t;
 // hardware already executes one wavefront's LDS accesses in order).
 __device__ __forceinline__ void lds_phase_fence() { asm volatile("" ::: "memory"); }
 
-template <int HD>
+// COOP = false: the streaming form described above (a wavefront per head and token range).
+// COOP = true: the short-sequence form.  All eight wavefronts of a workgroup work on ONE
+// (batch, kv head, token range), taking its tiles in turn, and merge their softmax states
+// through LDS at the end; with a single split per head the workgroup writes the final output and
+// no combine kernel runs.  It trades the contiguous-row access of the streaming form for eight
+// times the parallelism per head, which is what a latency-bound call (a few tiles per head) needs.
+template <int HD, bool COOP>
 __global__ void __launch_bounds__(kMfmaWaves * kWaveSize, 2)
 attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg) {
     constexpr int LPR = HD / 8;            // lanes per token row in a global load
@@ -55,6 +61,7 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     constexpr int KPITCH = HD * 2 + 16;    // slab row pitch while it holds K
     constexpr int VPITCH = HD * 2 + 32;    // slab row pitch while it holds V
     constexpr int SLAB = WT * VPITCH;
+    constexpr int STEP = COOP ? kMfmaWaves * WT : WT;  // token stride between a wavefront's tiles
     static_assert(WT == attn_tile_tokens(HD, kAttnImplMfma), "host plan and kernel tile disagree");
 
     __shared__ __align__(16) unsigned char s_slab[kMfmaWaves][SLAB];
@@ -66,21 +73,31 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     const int fn = lane & 15;        // role in an MFMA operand: row/column index ...
     const int fg = lane >> 4;        // ... and k group
 
-    // Workgroup -> (batch, group of heads_per_wg adjacent kv heads, group of splits); its eight
-    // wavefronts -> heads_per_wg heads x (8 / heads_per_wg) consecutive splits.
-    const int head_groups = p.KVH / heads_per_wg;
-    const int splits_per_wg = kMfmaWaves / heads_per_wg;
-    int bid = blockIdx.x;
-    const int hg = bid % head_groups;
-    bid /= head_groups;
-    const int b = bid % p.B;
-    const int sg = bid / p.B;
-    const int kvh = hg * heads_per_wg + wave % heads_per_wg;
-    const int split = sg * splits_per_wg + wave / heads_per_wg;
-    if (split >= p.num_splits) return;  // whole wavefront; no barrier follows
+    int b, kvh, split;
+    if constexpr (COOP) {
+        // workgroup -> (batch, kv head, split), kv head fastest
+        int bid = blockIdx.x;
+        kvh = bid % p.KVH;
+        bid /= p.KVH;
+        b = bid % p.B;
+        split = bid / p.B;
+    } else {
+        // workgroup -> (batch, group of heads_per_wg adjacent kv heads, group of splits); its eight
+        // wavefronts -> heads_per_wg heads x (8 / heads_per_wg) consecutive splits
+        const int head_groups = p.KVH / heads_per_wg;
+        const int splits_per_wg = kMfmaWaves / heads_per_wg;
+        int bid = blockIdx.x;
+        const int hg = bid % head_groups;
+        bid /= head_groups;
+        b = bid % p.B;
+        const int sg = bid / p.B;
+        kvh = hg * heads_per_wg + wave % heads_per_wg;
+        split = sg * splits_per_wg + wave / heads_per_wg;
+        if (split >= p.num_splits) return;  // whole wavefront; no barrier follows
+    }
     const int t_begin = split * p.tokens_per_split;
     const int S = p.seqlen_dev ? min(*p.seqlen_dev, p.S) : p.S;  // wave-uniform
-    if (t_begin >= S) return;           // split beyond a device-side KV length: the combine skips it
+    if (t_begin >= S) return;  // split beyond a device-side KV length (whole workgroup when COOP): the combine skips it
     const int t_end = min(S, t_begin + p.tokens_per_split);
     const float c = p.scale_log2e;
 
@@ -125,11 +142,11 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
         }
     };
 
-    int t0 = t_begin;
+    int t0 = t_begin + (COOP ? wave * WT : 0);
     issue_k(t0);
     issue_v(t0);
-    for (; t0 < t_end; t0 += WT) {
-        const int tn = t0 + WT;
+    for (; t0 < t_end; t0 += STEP) {
+        const int tn = t0 + STEP;
 
         // ---- K tile -> slab; its registers are free again, so the next K tile starts loading
 #pragma unroll
@@ -226,7 +243,51 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     //      denominator is still spread over the four k groups.
     l_part += __shfl_xor(l_part, 16, kWaveSize);
     l_part += __shfl_xor(l_part, 32, kWaveSize);
-    if (fn < R) {
+    const float m_log2 = (m_run == kMaskedScore) ? kMaskedScore : m_run * c;  // a COOP wave may have had no tile
+
+    if constexpr (COOP) {
+        // merge the eight wavefronts through LDS, then write like the streaming form
+        __shared__ float s_m[kMfmaWaves][kAttnMaxRatio];
+        __shared__ float s_l[kMfmaWaves][kAttnMaxRatio];
+        __shared__ __align__(16) float s_o[kMfmaWaves][kAttnMaxRatio][HD];
+        if (fn < R) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                *reinterpret_cast<float4*>(&s_o[wave][fn][nb * 16 + fg * 4]) =
+                    make_float4(O[nb][0], O[nb][1], O[nb][2], O[nb][3]);
+            }
+            if (fg == 0) {
+                s_m[wave][fn] = m_log2;
+                s_l[wave][fn] = l_part;
+            }
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < R * (HD / 2); idx += kMfmaWaves * kWaveSize) {
+            const int h = idx / (HD / 2);
+            const int d = (idx % (HD / 2)) * 2;
+            float M = s_m[0][h];
+#pragma unroll
+            for (int w = 1; w < kMfmaWaves; ++w) M = fmaxf(M, s_m[w][h]);
+            float L = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+            for (int w = 0; w < kMfmaWaves; ++w) {
+                const float e = fast_exp2(s_m[w][h] - M);  // wavefronts without a tile: 0
+                L = fmaf(s_l[w][h], e, L);
+                o0 = fmaf(s_o[w][h][d], e, o0);
+                o1 = fmaf(s_o[w][h][d + 1], e, o1);
+            }
+            const int qh = kvh * R + h;
+            if (p.part_o == nullptr) {
+                const float inv = 1.0f / L;
+                *reinterpret_cast<uint32_t*>(p.out + b * p.o_sb + int64_t(qh) * p.o_sh + d) =
+                    pack_bf16x2(o0 * inv, o1 * inv);
+            } else {
+                const int64_t row = attn_partial_row(p, b, qh, split);
+                *reinterpret_cast<float2*>(p.part_o + row * HD + d) = make_float2(o0, o1);
+                if (d == 0) p.part_ml[row] = make_float2(M, L);
+            }
+        }
+    } else if (fn < R) {
         const int qh = kvh * R + fn;
         if (p.part_o == nullptr) {  // single split: the final output row
             const float inv = 1.0f / l_part;
@@ -246,7 +307,7 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
             for (int nb = 0; nb < NB; ++nb) {
                 *reinterpret_cast<float4*>(prow + nb * 16) = make_float4(O[nb][0], O[nb][1], O[nb][2], O[nb][3]);
             }
-            if (fg == 0) p.part_ml[row] = make_float2(m_run * c, l_part);
+            if (fg == 0) p.part_ml[row] = make_float2(m_log2, l_part);
         }
     }
 }
@@ -260,16 +321,25 @@ int attn_mfma_heads_per_wg(int KVH) {
     return 1;
 }
 
-int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, hipStream_t stream) {
+int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipStream_t stream) {
     if (R < 1 || R > kAttnMaxRatio) return int(hipErrorInvalidValue);
+    const dim3 block(kMfmaWaves * kWaveSize);
+    if (coop) {
+        const dim3 grid(unsigned(p.B) * unsigned(p.KVH) * unsigned(p.num_splits));
+        if (HD == 64) {
+            hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, true>), grid, block, 0, stream, p, R, 1);
+        } else {
+            hipLaunchKernelGGL((attn_splitkv_mfma_kernel<128, true>), grid, block, 0, stream, p, R, 1);
+        }
+        return int(hipGetLastError());
+    }
     const int hpw = attn_mfma_heads_per_wg(p.KVH);
     const int spw = kMfmaWaves / hpw;
     const dim3 grid(unsigned(p.B) * unsigned(p.KVH / hpw) * unsigned((p.num_splits + spw - 1) / spw));
-    const dim3 block(kMfmaWaves * kWaveSize);
     if (HD == 64) {
-        hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64>), grid, block, 0, stream, p, R, hpw);
+        hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, false>), grid, block, 0, stream, p, R, hpw);
     } else {
-        hipLaunchKernelGGL((attn_splitkv_mfma_kernel<128>), grid, block, 0, stream, p, R, hpw);
+        hipLaunchKernelGGL((attn_splitkv_mfma_kernel<128, false>), grid, block, 0, stream, p, R, hpw);
     }
     return int(hipGetLastError());
 }

@@ -74,13 +74,25 @@ int attn_kernel_option() {
 
 AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl) {
     const int tile = attn_tile_tokens(HD, impl);
-    const int max_by_len = ceil_div(S, tile);  // a split shorter than one tile leaves lanes idle
+    const int tiles = ceil_div(S, tile);
+    AttnPlan plan;
+    plan.coop = false;
     int splits;
     if (requested > 0) {
         splits = requested;
     } else if (impl == kAttnImplMfma) {
-        // One 8-wave workgroup per compute unit (its loads in flight already saturate HBM); a
-        // workgroup covers heads_per_wg kv heads x (8 / heads_per_wg) splits of one batch row.
+        // Short sequences are latency-bound: when a (batch, kv head) has at most two tiles per
+        // wavefront of a workgroup, and there are not already enough heads to fill the device
+        // twice over, one cooperative workgroup per head finishes the row in a single launch.
+        const int64_t units = int64_t(B) * KVH;
+        if (tiles <= 2 * kMfmaWaves && units <= 2 * int64_t(num_cus)) {
+            plan.coop = true;
+            plan.num_splits = 1;
+            plan.tokens_per_split = tiles * tile;
+            return plan;
+        }
+        // Streaming form: one 8-wave workgroup per compute unit (its loads in flight already
+        // saturate HBM); a workgroup covers heads_per_wg kv heads x (8 / heads_per_wg) splits.
         const int hpw = attn_mfma_heads_per_wg(KVH);
         const int64_t wgs_per_split_group = int64_t(B) * (KVH / hpw);
         const int64_t groups = (int64_t(num_cus) + wgs_per_split_group - 1) / wgs_per_split_group;
@@ -90,11 +102,10 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
         const int64_t units = int64_t(B) * KVH;
         splits = int((int64_t(num_cus) * 2 + units - 1) / units);
     }
-    if (splits > max_by_len) splits = max_by_len;
+    if (splits > tiles) splits = tiles;  // a split shorter than one tile leaves lanes idle
     if (splits > L3_ATTN_MAX_SPLITS) splits = L3_ATTN_MAX_SPLITS;
     if (splits < 1) splits = 1;
-    int tps = ceil_div(ceil_div(S, splits), tile) * tile;
-    AttnPlan plan;
+    const int tps = ceil_div(ceil_div(S, splits), tile) * tile;
     plan.tokens_per_split = tps;
     plan.num_splits = ceil_div(S, tps);  // every split is non-empty
     return plan;
@@ -195,8 +206,9 @@ void fill_attn_params(AttnParams& p, const void* q, const void* k, const void* v
     p.scale_log2e = scale * 1.4426950408889634f;
 }
 
-int launch_split_stage(const AttnParams& p, int HD, int R, int impl, hipStream_t st) {
-    return (impl == kAttnImplMfma) ? launch_attn_splitkv_mfma(p, HD, R, st) : launch_attn_splitkv_fma(p, HD, R, st);
+int launch_split_stage(const AttnParams& p, int HD, int R, int impl, bool coop, hipStream_t st) {
+    return (impl == kAttnImplMfma) ? launch_attn_splitkv_mfma(p, HD, R, coop, st)
+                                   : launch_attn_splitkv_fma(p, HD, R, st);
 }
 
 }  // namespace
@@ -228,7 +240,7 @@ int attn_decode_impl(const void* q, const void* k, const void* v, void* out, voi
         p.part_ml = reinterpret_cast<float2*>(ws + round_up(rows * HD * sizeof(float), kWorkspaceAlign));
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int err = launch_split_stage(p, HD, QH / KVH, impl, st);
+    int err = launch_split_stage(p, HD, QH / KVH, impl, plan.coop, st);
     if (err == 0 && plan.num_splits > 1) err = launch_attn_combine(p, HD, st);
     return err == 0 ? L3_OK : L3_ERR_HIP;
 }
@@ -269,7 +281,7 @@ int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, fl
     fill_attn_params(p, q, k, v, nullptr, B, QH, KVH, S, q_strides, k_strides, v_strides, nullptr, scale, plan);
     p.part_o = part_o;
     p.part_ml = reinterpret_cast<float2*>(part_ml);
-    const int err = launch_split_stage(p, HD, QH / KVH, impl, static_cast<hipStream_t>(stream));
+    const int err = launch_split_stage(p, HD, QH / KVH, impl, plan.coop, static_cast<hipStream_t>(stream));
     return err == 0 ? plan.num_splits : L3_ERR_HIP;
 }
 

@@ -14,6 +14,7 @@ namespace l3 {
 struct AttnPlan {
     int num_splits;        // token ranges per (batch, kv head); each yields one partial per query head
     int tokens_per_split;  // multiple of the kernel's tile, except that the last split is shorter
+    bool coop;             // MFMA kernel only: whole workgroup on one (batch, kv head, split) -- short sequences
 };
 
 // The two split-KV kernels: FMA dot products on the vector ALUs, or MFMA tiles fed through LDS.
@@ -59,7 +60,7 @@ struct AttnParams {
 
 // Launchers: return a hipError_t cast to int (0 = success).
 int launch_attn_splitkv_fma(const AttnParams& p, int HD, int R, hipStream_t stream);
-int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, hipStream_t stream);
+int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipStream_t stream);
 int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream);
 int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
                     bool vec_ok, hipStream_t stream);

@@ -96,10 +96,7 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0):
         raise RuntimeError("flash_attention_decode needs at least one sequence and one cached token")
 
     with torch.cuda.device(query.device):
-        if num_splits == 0:
-            num_splits = lib.l3_attn_choose_splits(B, KVH, S, HD, _cus(query.device))
-            if num_splits < 0:
-                _fail(num_splits)
+        # num_splits == 0 lets the library plan for the current device (split count and kernel form)
         ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, num_splits)
         stream_ptr = _stream_ptr(query.device)
         ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None
@@ -142,7 +139,7 @@ def flash_attention_split(query, keys, values, num_splits: int = 0):
     lib = _l3lib.load()
     B, QH, KVH, S, HD = _check_qkv(query, keys, values)
     with torch.cuda.device(query.device):
-        n_req = num_splits if num_splits > 0 else lib.l3_attn_choose_splits(B, KVH, S, HD, _cus(query.device))
+        n_req = num_splits if num_splits > 0 else lib.l3_attn_choose_splits(B, KVH, S, HD, 0)
         if n_req < 0:
             _fail(n_req)
         part_o = torch.empty((B, QH, n_req, HD), dtype=torch.float32, device=query.device)
@@ -153,7 +150,7 @@ def flash_attention_split(query, keys, values, num_splits: int = 0):
             _l3lib.i64_array((query.stride(0), query.stride(1))),
             _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
             _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
-            1.0 / math.sqrt(HD), n_req, _stream_ptr(query.device))
+            1.0 / math.sqrt(HD), num_splits, _stream_ptr(query.device))
     if n < 0:
         _fail(n, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
     if n != n_req:  # the kernel laid its rows out for n splits: re-view the front of the buffers
@@ -196,10 +193,6 @@ def flash_attention_decode_devlen(query, keys, values, kv_len, num_splits: int =
     if out is None:
         out = torch.empty_like(query)
     with torch.cuda.device(query.device):
-        if num_splits == 0:
-            num_splits = lib.l3_attn_choose_splits(B, KVH, L, HD, _cus(query.device))
-            if num_splits < 0:
-                _fail(num_splits)
         ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, L, HD, num_splits)
         stream_ptr = _stream_ptr(query.device)
         ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None

@@ -223,6 +223,6 @@ def test_device_side_kv_length(gpu, HD, B, L):
         torch.cuda.synchronize()
         ref = attention_decode_ref(t2f32(q), t2f32(k[:, :, :S]), t2f32(v[:, :, :S]))
         assert_attn_close(out, ref, what=f"devlen S={S} of L={L}")
-        # same bits as the shape-driven call planned for the same cache length
-        splits = cke.attention_num_splits(B, KVH, L, HD, torch.cuda.get_device_properties(gpu).multi_processor_count)
-        np.testing.assert_array_equal(t2bits(out), t2bits(cke.flash_attention_decode_devlen(qg, kg, vg, kv_len, splits)))
+        # a forced split count (streaming form of the kernel) agrees to bf16 rounding
+        forced = cke.flash_attention_decode_devlen(qg, kg, vg, kv_len, 3)
+        assert (out.float() - forced.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, np.abs(ref).max())
