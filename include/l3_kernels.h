@@ -157,6 +157,20 @@ int l3_attn_combine(const float* part_o, const float* part_ml, void* out, int B,
 int l3_rms_norm(const void* x, const void* w, void* y, int64_t rows, int C, float eps, void* stream);
 
 /*
+ * Residual addition fused with the RMSNorm that follows it in a transformer block
+ * (model.py:147-148: x = x + attn(...), then ln_2(x); likewise before the next block's ln_1 and
+ * before ln_f):
+ *   sum_out[r, :] = bf16( x[r, :] + residual[r, :] )
+ *   y[r, :]       = rms_norm(sum_out[r, :], w, eps)          (of the rounded sum)
+ * so that (sum_out, y) carry the same bits as a bf16 tensor addition followed by l3_rms_norm.
+ * Layout and fast-path rules as for l3_rms_norm; sum_out may alias x or residual, y must not.
+ * One launch and one pass over the row instead of two launches and three passes.  The
+ * reference has no counterpart (it adds with a separate torch kernel).
+ */
+int l3_add_rms_norm(const void* x, const void* residual, const void* w, void* sum_out, void* y, int64_t rows,
+                    int C, float eps, void* stream);
+
+/*
  * Rotary embedding on adjacent pairs:
  *   y[b,t,h,2i]   = bf16( x[b,t,h,2i] * freq[t,2i] - x[b,t,h,2i+1] * freq[t,2i+1] )
  *   y[b,t,h,2i+1] = bf16( x[b,t,h,2i] * freq[t,2i+1] + x[b,t,h,2i+1] * freq[t,2i] )

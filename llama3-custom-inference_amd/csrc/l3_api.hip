@@ -316,6 +316,20 @@ int l3_rms_norm(const void* x, const void* w, void* y, int64_t rows, int C, floa
                            static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 
+int l3_add_rms_norm(const void* x, const void* residual, const void* w, void* sum_out, void* y, int64_t rows,
+                    int C, float eps, void* stream) {
+    if (!x || !residual || !w || !sum_out || !y) return L3_ERR_NULL_POINTER;
+    if (rows <= 0 || C <= 0 || rows >= (int64_t(1) << 31)) return L3_ERR_SHAPE;
+    if (!aligned(x, 2) || !aligned(residual, 2) || !aligned(w, 2) || !aligned(sum_out, 2) || !aligned(y, 2))
+        return L3_ERR_ALIGNMENT;
+    const bool vec_ok = (C % 8 == 0) && aligned(x, 16) && aligned(residual, 16) && aligned(w, 16) &&
+                        aligned(sum_out, 16) && aligned(y, 16);
+    return launch_add_rms_norm(static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(residual),
+                               static_cast<const uint16_t*>(w), static_cast<uint16_t*>(sum_out),
+                               static_cast<uint16_t*>(y), rows, C, eps, vec_ok,
+                               static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
 int l3_rot_embed(const void* x, const float* freq, void* y, int B, int T, int NH, int HD,
                  const int64_t x_strides[3], void* stream) {
     if (!x || !freq || !y || !x_strides) return L3_ERR_NULL_POINTER;

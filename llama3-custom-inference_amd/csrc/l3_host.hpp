@@ -64,6 +64,8 @@ int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipS
 int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream);
 int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
                     bool vec_ok, hipStream_t stream);
+int launch_add_rms_norm(const uint16_t* x, const uint16_t* res, const uint16_t* w, uint16_t* sum_out, uint16_t* y,
+                        int64_t rows, int C, float eps, bool vec_ok, hipStream_t stream);
 int launch_rot_embed(const uint16_t* x, const float* freq, uint16_t* y, int B, int T, int NH, int HD,
                      int64_t sb, int64_t st, int64_t sh, bool vec_ok, hipStream_t stream);
 int launch_rot_embed_append(const uint16_t* qkv, const float* table, uint16_t* q_out, uint16_t* cache_k,

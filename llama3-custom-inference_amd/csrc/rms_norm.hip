@@ -16,9 +16,15 @@ constexpr int kRmsThreads = 256;
 // One row per group of LANES threads (64: a wavefront per row, four rows per workgroup;
 // 256: the whole workgroup on one row).  A thread keeps up to MAXV 16-byte vectors of its
 // row in registers; requires C % 8 == 0 and C / 8 <= LANES * MAXV.
-template <int LANES, int MAXV>
+//
+// ADD = true fuses the residual addition that precedes every RMSNorm but the first in a
+// transformer block (model.py:147-148: x = x + attn(...); ...ln_2(x)): s = bf16(x + res) is
+// written to `sum_out` and the norm is taken of the ROUNDED s, so the pair of outputs is
+// bit-identical to torch's bf16 add followed by the unfused kernel.
+template <int LANES, int MAXV, bool ADD>
 __global__ void __launch_bounds__(kRmsThreads)
-rms_norm_rows_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, uint16_t* __restrict__ y,
+rms_norm_rows_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ res,
+                     const uint16_t* __restrict__ w, uint16_t* __restrict__ sum_out, uint16_t* __restrict__ y,
                      int64_t rows, int C, float eps) {
     constexpr int ROWS_PER_BLOCK = kRmsThreads / LANES;
     const int tid = threadIdx.x;
@@ -38,6 +44,16 @@ rms_norm_rows_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
             xv[j] = load16(xr + vi * 8);
             float f[8];
             unpack8(xv[j], f);
+            if constexpr (ADD) {
+                float r[8];
+                unpack8(load16(res + (live ? row : 0) * int64_t(C) + vi * 8), r);
+                xv[j].x = pack_bf16x2(f[0] + r[0], f[1] + r[1]);
+                xv[j].y = pack_bf16x2(f[2] + r[2], f[3] + r[3]);
+                xv[j].z = pack_bf16x2(f[4] + r[4], f[5] + r[5]);
+                xv[j].w = pack_bf16x2(f[6] + r[6], f[7] + r[7]);
+                if (live) store16(sum_out + row * int64_t(C) + vi * 8, xv[j]);
+                unpack8(xv[j], f);
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
         }
@@ -71,13 +87,24 @@ rms_norm_rows_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
 }
 
 // Any C, any alignment: one workgroup per row, 2-byte accesses, the row is read twice.
+template <bool ADD>
 __global__ void __launch_bounds__(kRmsThreads)
-rms_norm_generic_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, uint16_t* __restrict__ y,
+rms_norm_generic_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ res,
+                        const uint16_t* __restrict__ w, uint16_t* __restrict__ sum_out, uint16_t* __restrict__ y,
                         int C, float eps) {
     const int tid = threadIdx.x;
     const uint16_t* xr = x + int64_t(blockIdx.x) * C;
     uint16_t* yr = y + int64_t(blockIdx.x) * C;
     float ss = 0.f;
+    if constexpr (ADD) {
+        // first pass writes the rounded sum; the passes below then read it back as the input row
+        const uint16_t* rr = res + int64_t(blockIdx.x) * C;
+        uint16_t* sr = sum_out + int64_t(blockIdx.x) * C;
+        for (int i = tid; i < C; i += kRmsThreads) {
+            sr[i] = uint16_t(f32_to_bf16_bits(bf16_to_f32(xr[i]) + bf16_to_f32(rr[i])));
+        }
+        xr = sr;  // each thread re-reads only what it wrote itself
+    }
     for (int i = tid; i < C; i += kRmsThreads) {
         const float f = bf16_to_f32(xr[i]);
         ss = fmaf(f, f, ss);
@@ -95,36 +122,53 @@ rms_norm_generic_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
 
 }  // namespace
 
-int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
-                    bool vec_ok, hipStream_t stream) {
+namespace {
+
+template <bool ADD>
+int launch_rms_norm_impl(const uint16_t* x, const uint16_t* res, const uint16_t* w, uint16_t* sum_out, uint16_t* y,
+                         int64_t rows, int C, float eps, bool vec_ok, hipStream_t stream) {
     const int nvec = C / 8;
+    const dim3 block(kRmsThreads);
     if (vec_ok && rows >= 1024 && nvec <= 64 * 8) {
         // plenty of rows: a wavefront per row, no workgroup barrier
-        const unsigned blocks = unsigned((rows + 3) / 4);
+        const dim3 grid(unsigned((rows + 3) / 4));
         if (nvec <= 64 * 4) {
-            hipLaunchKernelGGL((rms_norm_rows_kernel<64, 4>), dim3(blocks), dim3(kRmsThreads), 0, stream, x, w, y,
-                               rows, C, eps);
+            hipLaunchKernelGGL((rms_norm_rows_kernel<64, 4, ADD>), grid, block, 0, stream, x, res, w, sum_out, y, rows,
+                               C, eps);
         } else {
-            hipLaunchKernelGGL((rms_norm_rows_kernel<64, 8>), dim3(blocks), dim3(kRmsThreads), 0, stream, x, w, y,
-                               rows, C, eps);
+            hipLaunchKernelGGL((rms_norm_rows_kernel<64, 8, ADD>), grid, block, 0, stream, x, res, w, sum_out, y, rows,
+                               C, eps);
         }
     } else if (vec_ok && nvec <= 256 * 4) {
         // few rows (decode): the whole workgroup on one row keeps the latency short
+        const dim3 grid{unsigned(rows)};
         if (nvec <= 256) {
-            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 1>), dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x,
-                               w, y, rows, C, eps);
+            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 1, ADD>), grid, block, 0, stream, x, res, w, sum_out, y,
+                               rows, C, eps);
         } else if (nvec <= 512) {
-            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 2>), dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x,
-                               w, y, rows, C, eps);
+            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 2, ADD>), grid, block, 0, stream, x, res, w, sum_out, y,
+                               rows, C, eps);
         } else {
-            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 4>), dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x,
-                               w, y, rows, C, eps);
+            hipLaunchKernelGGL((rms_norm_rows_kernel<256, 4, ADD>), grid, block, 0, stream, x, res, w, sum_out, y,
+                               rows, C, eps);
         }
     } else {
-        hipLaunchKernelGGL(rms_norm_generic_kernel, dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x, w, y, C,
-                           eps);
+        hipLaunchKernelGGL((rms_norm_generic_kernel<ADD>), dim3(unsigned(rows)), block, 0, stream, x, res, w, sum_out,
+                           y, C, eps);
     }
     return int(hipGetLastError());
+}
+
+}  // namespace
+
+int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
+                    bool vec_ok, hipStream_t stream) {
+    return launch_rms_norm_impl<false>(x, nullptr, w, nullptr, y, rows, C, eps, vec_ok, stream);
+}
+
+int launch_add_rms_norm(const uint16_t* x, const uint16_t* res, const uint16_t* w, uint16_t* sum_out, uint16_t* y,
+                        int64_t rows, int C, float eps, bool vec_ok, hipStream_t stream) {
+    return launch_rms_norm_impl<true>(x, res, w, sum_out, y, rows, C, eps, vec_ok, stream);
 }
 
 }  // namespace l3

@@ -20,7 +20,7 @@ from . import _l3lib
 
 __all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits",
            "flash_attention_split", "flash_attention_combine", "flash_attention_decode_devlen",
-           "rot_embed_append"]
+           "rot_embed_append", "add_rms_norm"]
 
 _cu_count = {}
 _workspaces = {}  # (device index, stream handle) -> uint8 tensor
@@ -269,6 +269,36 @@ def rms_norm(input, weight, eps):
     if rc != 0:
         _fail(rc, f"rows={rows} C={C}")
     return out
+
+
+def add_rms_norm(input, residual, weight, eps):
+    """(input + residual, rms_norm(input + residual, weight, eps)) in one launch: the residual
+    addition of model.py:147-148 fused with the norm that follows it.  Both outputs carry the same
+    bits as ``s = input + residual`` (bf16) followed by ``rms_norm(s, weight, eps)``.  An extension
+    of the reference's operator set."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("input", input)
+    _require_gpu_bf16("residual", residual)
+    _require_gpu_bf16("weight", weight)
+    if input.dim() != 3 or tuple(residual.shape) != tuple(input.shape):
+        raise RuntimeError("add_rms_norm expects two (B, T, C) tensors of the same shape")
+    C = input.size(2)
+    if weight.numel() != C:
+        raise RuntimeError(f"weight has {weight.numel()} elements, expected {C}")
+    x = input if input.is_contiguous() else input.contiguous()
+    r = residual if residual.is_contiguous() else residual.contiguous()
+    w = weight if weight.is_contiguous() else weight.contiguous()
+    s = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    rows = x.size(0) * x.size(1)
+    if rows == 0:
+        return s, y
+    with torch.cuda.device(x.device):
+        rc = lib.l3_add_rms_norm(x.data_ptr(), r.data_ptr(), w.data_ptr(), s.data_ptr(), y.data_ptr(), rows, C,
+                                 float(eps), _stream_ptr(x.device))
+    if rc != 0:
+        _fail(rc, f"rows={rows} C={C}")
+    return s, y
 
 
 def rot_embed(input, freq):

@@ -236,7 +236,7 @@ class GraphedDecodeLoop:
 
     What makes the step replayable: the token position lives in device memory.  The fused
     rot_embed_append operator writes K/V at that position, flash_attention_decode_devlen reads the
-    KV length from it, and the bookkeeping of generate() (prompt-mask keep, token store, stop
+    KV length from it, residual additions ride along with the norms (add_rms_norm), and the bookkeeping of generate() (prompt-mask keep, token store, stop
     flags, position increment) is expressed with fixed-shape torch ops on device tensors.
     """
 
@@ -258,17 +258,19 @@ class GraphedDecodeLoop:
         m, c, B = self.m, self.m.config, self.B
         ops = m.ops
         x = F.embedding(self.tok, m.wte)
-        for L in m.layers:
-            h = ops.rms_norm(x, L["ln_1"], c.norm_eps)
+        h = ops.rms_norm(x, m.layers[0]["ln_1"], c.norm_eps)
+        for i, L in enumerate(m.layers):
             qkv = F.linear(h, L["c_attn"])
             q = ops.rot_embed_append(qkv, m.freqs_cis, L["cache_k"], L["cache_v"], self.pos, c.n_head)
             y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
                                                   L["cache_v"][:B].transpose(1, 2), self.kv_len)
-            x = x + F.linear(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"])
-            h = ops.rms_norm(x, L["ln_2"], c.norm_eps)
-            x = x + F.linear(F.silu(F.linear(h, L["c_fc2"])) * F.linear(h, L["c_fc"]), L["mlp_proj"])
-        x = ops.rms_norm(x, m.ln_f, c.norm_eps)
-        logits = F.linear(x[:, -1], m.wte).float()
+            # residual add fused with the norm that follows it (same bits as add, then rms_norm)
+            x, h = ops.add_rms_norm(x, F.linear(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"]),
+                                    L["ln_2"], c.norm_eps)
+            mlp = F.linear(F.silu(F.linear(h, L["c_fc2"])) * F.linear(h, L["c_fc"]), L["mlp_proj"])
+            next_norm = m.layers[i + 1]["ln_1"] if i + 1 < len(m.layers) else m.ln_f
+            x, h = ops.add_rms_norm(x, mlp, next_norm, c.norm_eps)
+        logits = F.linear(h[:, -1], m.wte).float()
         nxt = torch.argmax(logits, dim=-1)
         # generate() bookkeeping (model.py:373-378) at position pos + 1, all on the device
         cur = (self.pos + 1).long().clamp_(max=self.total_len - 1)

@@ -37,7 +37,9 @@ def test_ragged_lengths(gpu, HD, S):
 
 
 @pytest.mark.parametrize("HD,QH,KVH", [(64, 4, 4), (64, 8, 4), (64, 12, 4), (64, 32, 8), (64, 16, 2),
-                                        (128, 4, 4), (128, 4, 2), (128, 24, 8), (128, 32, 8), (128, 64, 8)])
+                                        (128, 4, 4), (128, 4, 2), (128, 24, 8), (128, 32, 8), (128, 64, 8),
+                                        (64, 6, 3), (128, 6, 6), (64, 5, 5), (128, 16, 16), (64, 32, 16),
+                                        (128, 8, 1), (64, 7, 7)])
 @pytest.mark.parametrize("splits", [0, 1, 4])
 def test_head_ratios(gpu, HD, QH, KVH, splits):
     _run(gpu, 2, QH, KVH, 333, HD, seed=QH + KVH, splits=splits)
@@ -100,6 +102,29 @@ def test_equal_value_rows_return_that_row(gpu):
     want = row.repeat_interleave(4, dim=1)
     # a convex combination of identical rows: only bf16 rounding of the normalised sum remains
     assert (out.float() - want.float()).abs().max().item() <= 2.0 ** -7 * want.float().abs().max().item()
+
+
+def test_very_long_sequence_by_property(gpu):
+    """KV length 131072 at head size 128 (0.5 GB of K+V): too large for the float64 oracle to be
+    worth it, so the result is pinned by a size-independent property -- with identical V rows per
+    head the output must be that row whatever the scores are -- plus agreement between the
+    automatic plan and a forced, different split count."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, QH, KVH, S, HD = 1, 32, 8, 131072, 128
+    g = torch.Generator(device="cpu").manual_seed(5)
+    q = torch.randn((B, 1, QH, HD), generator=g).to(torch.bfloat16).to(gpu).transpose(1, 2)
+    k = torch.randn((B, S, KVH, HD), generator=g).to(torch.bfloat16).to(gpu).transpose(1, 2)
+    row = torch.randn((B, 1, KVH, HD), generator=g).to(torch.bfloat16).to(gpu)
+    v = row.expand(B, S, KVH, HD).contiguous().transpose(1, 2)
+    out = cke.flash_attention_decode(q, k, v)
+    want = row.transpose(1, 2).repeat_interleave(QH // KVH, dim=1)
+    assert (out.float() - want.float()).abs().max().item() <= 2.0 ** -7 * want.float().abs().max().item()
+    v2 = torch.randn((B, S, KVH, HD), generator=g).to(torch.bfloat16).to(gpu).transpose(1, 2)
+    a = cke.flash_attention_decode(q, k, v2)
+    b2 = cke.flash_attention_decode(q, k, v2, 37)
+    torch.cuda.synchronize()
+    assert (a.float() - b2.float()).abs().max().item() <= 2.0 ** -7
 
 
 def test_inputs_are_not_modified_and_errors_are_raised(gpu):

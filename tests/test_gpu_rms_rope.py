@@ -186,3 +186,24 @@ def test_rot_embed_append_fuses_rope_and_cache_write(gpu, HD, NH, KVH):
     cke.rot_embed_append(qkv.to(gpu), tab_g, ck, cv, pos, NH)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(t2bits(ck), t2bits(ck0))
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 2048), (64, 1, 2048), (2, 700, 4096), (1, 3, 136), (1, 5, 100), (1, 2, 8200)])
+def test_add_rms_norm_equals_add_then_norm(gpu, shape):
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, T, C = shape
+    print(f"add_rms_norm {shape}", flush=True)
+    x = randn_bf16(shape, 71)
+    r = randn_bf16(shape, 72, scale=0.5)
+    w = randn_bf16((C,), 73, scale=0.02, mean=1.0)
+    s, y = cke.add_rms_norm(x.to(gpu), r.to(gpu), w.to(gpu), 1e-5)
+    torch.cuda.synchronize()
+    # the sum is torch's bf16 addition, bit for bit
+    s_ref = (x.to(gpu) + r.to(gpu))
+    np.testing.assert_array_equal(t2bits(s), t2bits(s_ref))
+    # the norm is the unfused kernel on that sum, bit for bit, and within 1 ulp of the oracle
+    np.testing.assert_array_equal(t2bits(y), t2bits(cke.rms_norm(s_ref, w.to(gpu), 1e-5)))
+    assert_within_ulps(y, rms_norm_ref(t2f32(s_ref), t2f32(w), 1e-5), 1, what=f"add_rms_norm {shape}")
+    with pytest.raises(RuntimeError):
+        cke.add_rms_norm(x.to(gpu), r.to(gpu)[:, :, : C // 2], w.to(gpu), 1e-5)
