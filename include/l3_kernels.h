@@ -171,6 +171,23 @@ int l3_add_rms_norm(const void* x, const void* residual, const void* w, void* su
                     int C, float eps, void* stream);
 
 /*
+ * y[i] = bf16( bf16(silu(a[i])) * b[i] ) over n contiguous bf16 values: the SwiGLU elementwise
+ * product of model.py:134, F.silu(c_fc2(x)) * c_fc(x), in one launch with the same two roundings
+ * as the two torch kernels.  No counterpart among the reference's kernels.
+ */
+int l3_silu_mul(const void* a, const void* b, void* y, int64_t n, void* stream);
+
+/*
+ * out[r] = index of the first maximum of the bf16 row logits[r*row_stride : r*row_stride + V]
+ * (int64, like torch.argmax; a row of NaNs gives 0): the greedy pick of model.py:371.  Two small
+ * launches (per-chunk maxima into the caller's workspace of l3_argmax_workspace_bytes(rows, V)
+ * bytes, then one merge per row).  rows <= 65535.  No counterpart among the reference's kernels.
+ */
+size_t l3_argmax_workspace_bytes(int rows, int V);
+int l3_argmax(const void* logits, int64_t row_stride, int rows, int V, void* workspace, size_t workspace_bytes,
+              int64_t* out, void* stream);
+
+/*
  * Rotary embedding on adjacent pairs:
  *   y[b,t,h,2i]   = bf16( x[b,t,h,2i] * freq[t,2i] - x[b,t,h,2i+1] * freq[t,2i+1] )
  *   y[b,t,h,2i+1] = bf16( x[b,t,h,2i] * freq[t,2i+1] + x[b,t,h,2i+1] * freq[t,2i] )

@@ -1,0 +1,127 @@
+// Two small decode-step kernels next to the three operators: the SwiGLU elementwise product
+// silu(a) * b (model.py:134 evaluates it with two torch kernels) and the greedy argmax over the
+// logits row (model.py:371).  In a graph-replayed decode step both are dispatch-bound; one
+// launch each instead of two resp. a 40 us single-workgroup library reduction.
+#include "l3_device.hpp"
+#include "l3_host.hpp"
+
+namespace l3 {
+
+namespace {
+
+constexpr int kMiscThreads = 256;
+
+// y = bf16( bf16(silu(a)) * b ): the intermediate rounding reproduces torch's F.silu(a) * b,
+// where silu's bf16 result is materialised before the multiplication.
+__device__ __forceinline__ float silu_rounded(float a) {
+    const float s = a / (1.0f + expf(-a));
+    return __uint_as_float(f32_to_bf16_bits(s) << 16);
+}
+
+__global__ void __launch_bounds__(kMiscThreads)
+silu_mul_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ y,
+                int64_t nvec) {
+    const int64_t i = int64_t(blockIdx.x) * kMiscThreads + threadIdx.x;
+    if (i >= nvec) return;
+    float fa[8], fb[8];
+    unpack8(load16(a + i * 8), fa);
+    unpack8(load16(b + i * 8), fb);
+    uint4 o;
+    o.x = pack_bf16x2(silu_rounded(fa[0]) * fb[0], silu_rounded(fa[1]) * fb[1]);
+    o.y = pack_bf16x2(silu_rounded(fa[2]) * fb[2], silu_rounded(fa[3]) * fb[3]);
+    o.z = pack_bf16x2(silu_rounded(fa[4]) * fb[4], silu_rounded(fa[5]) * fb[5]);
+    o.w = pack_bf16x2(silu_rounded(fa[6]) * fb[6], silu_rounded(fa[7]) * fb[7]);
+    store16(y + i * 8, o);
+}
+
+__global__ void __launch_bounds__(kMiscThreads)
+silu_mul_scalar_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ y,
+                       int64_t n) {
+    const int64_t i = int64_t(blockIdx.x) * kMiscThreads + threadIdx.x;
+    if (i >= n) return;
+    y[i] = uint16_t(f32_to_bf16_bits(silu_rounded(bf16_to_f32(a[i])) * bf16_to_f32(b[i])));
+}
+
+// (value, index) pairs ordered by value, then by smaller index: the first maximum wins, as
+// torch.argmax documents.  NaN never wins against a number (comparisons with NaN are false).
+__device__ __forceinline__ void argmax_merge(float& v, int& idx, float ov, int oidx) {
+    if (ov > v || (ov == v && oidx < idx)) {
+        v = ov;
+        idx = oidx;
+    }
+}
+
+// Stage 1: each workgroup scans a contiguous chunk of one row (bf16 logits) and writes its
+// best (value, index).  Stage 2 (one workgroup per row) merges the chunks.
+__global__ void __launch_bounds__(kMiscThreads)
+argmax_partial_kernel(const uint16_t* __restrict__ logits, int64_t row_stride, int V, int chunk,
+                      float* __restrict__ part_val, int* __restrict__ part_idx) {
+    const int row = blockIdx.y;
+    const int c0 = blockIdx.x * chunk;
+    const int c1 = min(V, c0 + chunk);
+    const uint16_t* r = logits + row * row_stride;
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = c0 + threadIdx.x; i < c1; i += kMiscThreads) argmax_merge(v, idx, bf16_to_f32(r[i]), i);
+#pragma unroll
+    for (int off = 1; off < kWaveSize; off <<= 1) {
+        argmax_merge(v, idx, __shfl_xor(v, off, kWaveSize), __shfl_xor(idx, off, kWaveSize));
+    }
+    __shared__ float s_v[kMiscThreads / kWaveSize];
+    __shared__ int s_i[kMiscThreads / kWaveSize];
+    if ((threadIdx.x & (kWaveSize - 1)) == 0) {
+        s_v[threadIdx.x / kWaveSize] = v;
+        s_i[threadIdx.x / kWaveSize] = idx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < kMiscThreads / kWaveSize; ++w) argmax_merge(v, idx, s_v[w], s_i[w]);
+        part_val[row * gridDim.x + blockIdx.x] = v;
+        part_idx[row * gridDim.x + blockIdx.x] = idx;
+    }
+}
+
+__global__ void __launch_bounds__(kWaveSize)
+argmax_final_kernel(const float* __restrict__ part_val, const int* __restrict__ part_idx, int nparts,
+                    int64_t* __restrict__ out) {
+    const int row = blockIdx.x;
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < nparts; i += kWaveSize) {
+        argmax_merge(v, idx, part_val[row * nparts + i], part_idx[row * nparts + i]);
+    }
+#pragma unroll
+    for (int off = 1; off < kWaveSize; off <<= 1) {
+        argmax_merge(v, idx, __shfl_xor(v, off, kWaveSize), __shfl_xor(idx, off, kWaveSize));
+    }
+    if (threadIdx.x == 0) out[row] = (idx == 0x7fffffff) ? 0 : idx;  // all-NaN row: index 0
+}
+
+}  // namespace
+
+int launch_silu_mul(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n, bool vec_ok, hipStream_t stream) {
+    if (vec_ok) {
+        const int64_t nvec = n / 8;
+        hipLaunchKernelGGL(silu_mul_kernel, dim3(unsigned((nvec + kMiscThreads - 1) / kMiscThreads)),
+                           dim3(kMiscThreads), 0, stream, a, b, y, nvec);
+    } else {
+        hipLaunchKernelGGL(silu_mul_scalar_kernel, dim3(unsigned((n + kMiscThreads - 1) / kMiscThreads)),
+                           dim3(kMiscThreads), 0, stream, a, b, y, n);
+    }
+    return int(hipGetLastError());
+}
+
+int argmax_parts(int V) { return (V + kArgmaxChunk - 1) / kArgmaxChunk; }
+
+int launch_argmax(const uint16_t* logits, int64_t row_stride, int rows, int V, float* part_val, int* part_idx,
+                  int64_t* out, hipStream_t stream) {
+    const int parts = argmax_parts(V);
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(unsigned(parts), unsigned(rows)), dim3(kMiscThreads), 0, stream,
+                       logits, row_stride, V, kArgmaxChunk, part_val, part_idx);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(unsigned(rows)), dim3(kWaveSize), 0, stream, part_val, part_idx,
+                       parts, out);
+    return int(hipGetLastError());
+}
+
+}  // namespace l3

@@ -330,6 +330,35 @@ int l3_add_rms_norm(const void* x, const void* residual, const void* w, void* su
                                static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 
+int l3_silu_mul(const void* a, const void* b, void* y, int64_t n, void* stream) {
+    if (!a || !b || !y) return L3_ERR_NULL_POINTER;
+    if (n <= 0 || n >= (int64_t(1) << 38)) return L3_ERR_SHAPE;
+    if (!aligned(a, 2) || !aligned(b, 2) || !aligned(y, 2)) return L3_ERR_ALIGNMENT;
+    const bool vec_ok = (n % 8 == 0) && aligned(a, 16) && aligned(b, 16) && aligned(y, 16);
+    return launch_silu_mul(static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b),
+                           static_cast<uint16_t*>(y), n, vec_ok, static_cast<hipStream_t>(stream)) == 0
+               ? L3_OK : L3_ERR_HIP;
+}
+
+size_t l3_argmax_workspace_bytes(int rows, int V) {
+    if (rows <= 0 || V <= 0) return 0;
+    return size_t(rows) * size_t(argmax_parts(V)) * (sizeof(float) + sizeof(int));
+}
+
+int l3_argmax(const void* logits, int64_t row_stride, int rows, int V, void* workspace, size_t workspace_bytes,
+              int64_t* out, void* stream) {
+    if (!logits || !out || !workspace) return L3_ERR_NULL_POINTER;
+    if (rows <= 0 || V <= 0 || rows > 65535) return L3_ERR_SHAPE;
+    if (row_stride < V) return L3_ERR_STRIDE;
+    if (!aligned(logits, 2) || !aligned(out, 8) || !aligned(workspace, 8)) return L3_ERR_ALIGNMENT;
+    if (workspace_bytes < l3_argmax_workspace_bytes(rows, V)) return L3_ERR_WORKSPACE;
+    const size_t parts = size_t(rows) * size_t(argmax_parts(V));
+    float* pv = static_cast<float*>(workspace);
+    int* pi = reinterpret_cast<int*>(pv + parts);
+    return launch_argmax(static_cast<const uint16_t*>(logits), row_stride, rows, V, pv, pi, out,
+                         static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
 int l3_rot_embed(const void* x, const float* freq, void* y, int B, int T, int NH, int HD,
                  const int64_t x_strides[3], void* stream) {
     if (!x || !freq || !y || !x_strides) return L3_ERR_NULL_POINTER;

@@ -66,6 +66,11 @@ int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t r
                     bool vec_ok, hipStream_t stream);
 int launch_add_rms_norm(const uint16_t* x, const uint16_t* res, const uint16_t* w, uint16_t* sum_out, uint16_t* y,
                         int64_t rows, int C, float eps, bool vec_ok, hipStream_t stream);
+int launch_silu_mul(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n, bool vec_ok, hipStream_t stream);
+constexpr int kArgmaxChunk = 2048;  // logits one workgroup of the first argmax stage scans
+int argmax_parts(int V);
+int launch_argmax(const uint16_t* logits, int64_t row_stride, int rows, int V, float* part_val, int* part_idx,
+                  int64_t* out, hipStream_t stream);
 int launch_rot_embed(const uint16_t* x, const float* freq, uint16_t* y, int B, int T, int NH, int HD,
                      int64_t sb, int64_t st, int64_t sh, bool vec_ok, hipStream_t stream);
 int launch_rot_embed_append(const uint16_t* qkv, const float* table, uint16_t* q_out, uint16_t* cache_k,

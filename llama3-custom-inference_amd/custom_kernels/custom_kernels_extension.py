@@ -20,7 +20,7 @@ from . import _l3lib
 
 __all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits",
            "flash_attention_split", "flash_attention_combine", "flash_attention_decode_devlen",
-           "rot_embed_append", "add_rms_norm"]
+           "rot_embed_append", "add_rms_norm", "silu_mul", "argmax"]
 
 _cu_count = {}
 _workspaces = {}  # (device index, stream handle) -> uint8 tensor
@@ -55,9 +55,13 @@ def _cus(device) -> int:
 
 
 def _workspace(device, stream_ptr: int, nbytes: int):
-    """Attention workspace (float32 partials), kept per (device, stream) and grown on demand so
-    that a decode step does not allocate.  Calls on one stream are ordered and can share it;
-    another stream gets its own."""
+    """Scratch for the kernels that need it (attention partials, argmax partials), kept per
+    (device, stream) and grown on demand so that a decode step does not allocate.  Calls on one
+    stream are ordered and can share it; another stream gets its own.  While a stream is being
+    captured into a HIP graph the buffer comes from the graph's own memory pool instead (a plain
+    allocation that lives and dies with the graph) and is not cached."""
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
@@ -299,6 +303,49 @@ def add_rms_norm(input, residual, weight, eps):
     if rc != 0:
         _fail(rc, f"rows={rows} C={C}")
     return s, y
+
+
+def silu_mul(a, b):
+    """F.silu(a) * b for two bf16 tensors of the same shape in one launch (model.py:134), with the
+    two roundings of the two torch kernels, so the bits are the same.  An extension."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("a", a)
+    _require_gpu_bf16("b", b)
+    if tuple(a.shape) != tuple(b.shape):
+        raise RuntimeError(f"silu_mul: shapes differ: {tuple(a.shape)} vs {tuple(b.shape)}")
+    ac = a if a.is_contiguous() else a.contiguous()
+    bc = b if b.is_contiguous() else b.contiguous()
+    y = torch.empty(ac.shape, dtype=ac.dtype, device=ac.device)
+    if y.numel() == 0:
+        return y
+    with torch.cuda.device(ac.device):
+        rc = lib.l3_silu_mul(ac.data_ptr(), bc.data_ptr(), y.data_ptr(), y.numel(), _stream_ptr(ac.device))
+    if rc != 0:
+        _fail(rc, f"n={y.numel()}")
+    return y
+
+
+def argmax(logits):
+    """Index of the first maximum along the last dimension of a 2-D bf16 tensor (rows, V), as
+    int64 -- torch.argmax(logits.float(), dim=-1) for the greedy pick of model.py:371 (the float
+    conversion of model.py:225 is monotone, so it is skipped).  An extension."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("logits", logits)
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise RuntimeError("argmax expects a 2-D (rows, V) tensor with a contiguous last dimension")
+    rows, V = logits.shape
+    out = torch.empty(rows, dtype=torch.int64, device=logits.device)
+    if rows == 0:
+        return out
+    with torch.cuda.device(logits.device):
+        ws_bytes = lib.l3_argmax_workspace_bytes(rows, V)
+        stream_ptr = _stream_ptr(logits.device)
+        ws = _workspace(logits.device, stream_ptr, ws_bytes)
+        rc = lib.l3_argmax(logits.data_ptr(), logits.stride(0), rows, V, ws.data_ptr(), ws_bytes, out.data_ptr(),
+                           stream_ptr)
+    if rc != 0:
+        _fail(rc, f"rows={rows} V={V}")
+    return out
 
 
 def rot_embed(input, freq):

@@ -172,7 +172,7 @@ class LlamaDecoder:
         loop.pos.fill_(min_prompt_len)
         loop.kv_len.fill_(min_prompt_len + 1)
         if loop.graph is None:
-            loop.capture()
+            loop.capture(self)
         for cur_pos in range(min_prompt_len + 1, total_len):
             loop.graph.replay()
             if not ignore_eos and (cur_pos - min_prompt_len) % 16 == 0 and bool(loop.eos.all()):
@@ -243,7 +243,10 @@ class GraphedDecodeLoop:
     def __init__(self, model: "LlamaDecoder", batch: int, total_len: int):
         import torch as _t
 
-        self.m, self.B, self.total_len = model, batch, total_len
+        # The loop does not keep the model: the model owns its loops (LlamaDecoder._graphs), and a
+        # reference cycle would leave the recorded graph to the cyclic garbage collector, which may
+        # then destroy it in the middle of another stream capture (that aborts the process).
+        self.B, self.total_len = batch, total_len
         dev = model.device
         self.tokens = _t.zeros((batch, total_len), dtype=_t.long, device=dev)
         self.text_mask = _t.zeros((batch, total_len), dtype=_t.bool, device=dev)
@@ -254,8 +257,8 @@ class GraphedDecodeLoop:
         self.stop = _t.tensor(list(model.tokenizer.stop_tokens), device=dev)
         self.graph = None
 
-    def step(self):
-        m, c, B = self.m, self.m.config, self.B
+    def step(self, m: "LlamaDecoder"):
+        c, B = m.config, self.B
         ops = m.ops
         x = F.embedding(self.tok, m.wte)
         h = ops.rms_norm(x, m.layers[0]["ln_1"], c.norm_eps)
@@ -267,11 +270,10 @@ class GraphedDecodeLoop:
             # residual add fused with the norm that follows it (same bits as add, then rms_norm)
             x, h = ops.add_rms_norm(x, F.linear(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"]),
                                     L["ln_2"], c.norm_eps)
-            mlp = F.linear(F.silu(F.linear(h, L["c_fc2"])) * F.linear(h, L["c_fc"]), L["mlp_proj"])
+            mlp = F.linear(ops.silu_mul(F.linear(h, L["c_fc2"]), F.linear(h, L["c_fc"])), L["mlp_proj"])
             next_norm = m.layers[i + 1]["ln_1"] if i + 1 < len(m.layers) else m.ln_f
             x, h = ops.add_rms_norm(x, mlp, next_norm, c.norm_eps)
-        logits = F.linear(h[:, -1], m.wte).float()
-        nxt = torch.argmax(logits, dim=-1)
+        nxt = ops.argmax(F.linear(h[:, -1], m.wte))   # first maximum of the bf16 logits = argmax of their float copy
         # generate() bookkeeping (model.py:373-378) at position pos + 1, all on the device
         cur = (self.pos + 1).long().clamp_(max=self.total_len - 1)
         keep = self.text_mask.index_select(1, cur).squeeze(1)
@@ -282,22 +284,34 @@ class GraphedDecodeLoop:
         self.pos += 1
         self.kv_len += 1
 
-    def capture(self):
-        side = torch.cuda.Stream(device=self.m.device)
-        saved = [t.clone() for t in (self.tokens, self.tok, self.pos, self.kv_len, self.eos)]
-        side.wait_stream(torch.cuda.current_stream(self.m.device))
+    def capture(self, m: "LlamaDecoder"):
+        import gc
+
+        state = (self.tokens, self.tok, self.pos, self.kv_len, self.eos)
+        saved = [t.clone() for t in state]
+        side = torch.cuda.Stream(device=m.device)
+        side.wait_stream(torch.cuda.current_stream(m.device))
         with torch.cuda.stream(side):
-            self.step()   # warm-up outside capture: workspaces, hipBLASLt handles, allocator
-        torch.cuda.current_stream(self.m.device).wait_stream(side)
-        torch.cuda.synchronize(self.m.device)
-        for t, s in zip((self.tokens, self.tok, self.pos, self.kv_len, self.eos), saved):
+            self.step(m)   # warm-up outside capture: workspaces, hipBLASLt handles, allocator
+        torch.cuda.current_stream(m.device).wait_stream(side)
+        torch.cuda.synchronize(m.device)
+        for t, s in zip(state, saved):
             t.copy_(s)
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.step()
-        for t, s in zip((self.tokens, self.tok, self.pos, self.kv_len, self.eos), saved):
+        # No garbage collection while the stream is capturing: a collected CUDAGraph or cached
+        # block would be freed with calls that are illegal during capture.
+        gc.collect()
+        gc_was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.step(m)
+        finally:
+            if gc_was_enabled:
+                gc.enable()
+        for t, s in zip(state, saved):
             t.copy_(s)   # capture does not execute, but keep the state explicit
-        torch.cuda.synchronize(self.m.device)
+        torch.cuda.synchronize(m.device)
 
 
 def random_prompts(batch, length, vocab_size, seed, exclude=(128004, 128001)):

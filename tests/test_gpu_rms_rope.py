@@ -5,10 +5,14 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import assert_within_ulps, randn_bf16, t2bits, t2f32, to_device_like
+from helpers import assert_within_ulps, bf16_ulp_distance, randn_bf16, round_to_bf16, t2bits, t2f32, to_device_like
 from oracle import precompute_freqs_cis_ref, rms_norm_ref, rot_embed_ref
 
 pytestmark = pytest.mark.gpu
+
+
+def bf16_ulp(a, b):
+    return bf16_ulp_distance(t2bits(a), t2bits(b))
 
 
 # ------------------------------------------------------------------------------ RMSNorm
@@ -207,3 +211,45 @@ def test_add_rms_norm_equals_add_then_norm(gpu, shape):
     assert_within_ulps(y, rms_norm_ref(t2f32(s_ref), t2f32(w), 1e-5), 1, what=f"add_rms_norm {shape}")
     with pytest.raises(RuntimeError):
         cke.add_rms_norm(x.to(gpu), r.to(gpu)[:, :, : C // 2], w.to(gpu), 1e-5)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 8192), (64, 1, 8192), (2, 300, 1000), (3, 7, 13)])
+def test_silu_mul_matches_torch(gpu, shape):
+    from custom_kernels import custom_kernels_extension as cke
+    import torch.nn.functional as F
+
+    a = randn_bf16(shape, 81, scale=3.0).to(gpu)
+    b = randn_bf16(shape, 82).to(gpu)
+    y = cke.silu_mul(a, b)
+    torch.cuda.synchronize()
+    ref = F.silu(a) * b
+    d = bf16_ulp(y, ref)
+    assert d.max() <= 1 and (d > 0).mean() < 1e-3, f"silu_mul differs from torch: max {d.max()} ulp, {(d > 0).mean():.2e} of elements"
+    # and against exact arithmetic with the same two roundings
+    af, bf = t2f32(a).astype(np.float64), t2f32(b).astype(np.float64)
+    s = round_to_bf16(af / (1.0 + np.exp(-af))).astype(np.float64)
+    assert_within_ulps(y, s * bf, 1, what=f"silu_mul {shape}")
+
+
+@pytest.mark.parametrize("rows,V", [(1, 128256), (64, 128256), (3, 1000), (2, 2048), (5, 2049), (1, 7)])
+def test_argmax_first_maximum(gpu, rows, V):
+    from custom_kernels import custom_kernels_extension as cke
+
+    x = randn_bf16((rows, V), 91)
+    # plant ties of the row maximum: the first one must win
+    for r in range(rows):
+        top = x[r].float().max().item() + 1.0
+        pos = sorted({(r * 37 + 5) % V, (V - 1 - r) % V, V // 2})
+        for p in pos:
+            x[r, p] = top
+    out = cke.argmax(x.to(gpu))
+    torch.cuda.synchronize()
+    want = torch.argmax(x.float(), dim=-1)
+    first = torch.tensor([int(np.flatnonzero(t2f32(x[r]) == t2f32(x[r]).max())[0]) for r in range(rows)])
+    assert out.dtype == torch.int64
+    np.testing.assert_array_equal(out.cpu().numpy(), first.numpy())
+    np.testing.assert_array_equal(out.cpu().numpy(), want.numpy())
+    # strided rows (a slice of a wider matrix)
+    wide = randn_bf16((rows, V + 9), 92).to(gpu)
+    np.testing.assert_array_equal(cke.argmax(wide[:, :V]).cpu().numpy(),
+                                  torch.argmax(wide[:, :V].float(), dim=-1).cpu().numpy())
