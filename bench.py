@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the custom-kernel hot path on one MI355X.
 
-Default workload (BASELINE.json configs[1]): decode attention at head_dim 128, batch 1,
+Default workload (the headline configuration): decode attention at head_dim 128, batch 1,
 32 query / 8 KV heads, bf16, KV length swept over every power of two from 512 to 32768.
 One step = one pass over the seven lengths (split-KV kernel + combine each).  Inputs are
 resident in HBM before the timed region; each length owns several copies of its K/V and a
@@ -14,7 +14,7 @@ Prints ONE JSON line: value = algorithmic GB/s (K+V+Q read, O written) over the 
 steps; "roofline" prices the same bytes against the 8 TB/s HBM peak from HIP-event timing;
 "cpu_baseline" is stock PyTorch on the host cores for a bounded sample of the same sweep.
 
-Other workloads (--workload c1|c3a|c3b|rms|rope|e2e) report the remaining BASELINE configs
+Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|e2e|copy) report the remaining configurations
 in the same format.
 """
 
@@ -266,7 +266,7 @@ def run_attention(args, torch, lib, l3, dev, name):
 
 
 def run_rows(args, torch, lib, l3, dev, name):
-    """RMSNorm / rotary embedding at the largest BASELINE config-4 shape, plus the small ones."""
+    """RMSNorm / rotary embedding at the largest configured shape (4096 rows / tokens), plus the small ones."""
     from custom_kernels import custom_kernels_extension as cke
     from custom_kernels import precompute_freqs_cis
     from oracle.cpu_baseline import rms_norm_cpu, rot_embed_cpu
@@ -381,7 +381,7 @@ def main():
     FORCE_SPLITS = args.splits
     if args.gpus != 1:
         print(f"bench.py: this path runs on one GPU with no sharding; --gpus {args.gpus} is not supported "
-              "(every (batch, kv head) pair is independent, see DESIGN.md for how it would shard)", file=sys.stderr)
+              "(every (batch, kv head) pair is independent and could be sharded by batch or kv head)", file=sys.stderr)
         sys.exit(2)
 
     import torch

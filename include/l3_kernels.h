@@ -121,6 +121,21 @@ int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out
                           float scale, int num_splits, const int32_t* kv_len_dev, void* stream);
 
 /*
+ * Causal GQA attention for T > 1 query tokens per sequence (prompt prefill):
+ *   out[b, h, i, :] = softmax_j<=p(i)( scale * q[b, h, i, :] . k[b, h/(QH/KVH), j, :] ) @ v[...],
+ *   p(i) = S - T + i
+ * i.e. query i sits at absolute position S - T + i of a cache that holds S >= T tokens.  For
+ * S == T this is scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True), which
+ * the reference calls for this case (model.py:114-116) instead of a kernel of its own.
+ *   q, out : (B, QH, T, HD) bf16 with {batch, head, token} strides
+ *   k, v   : (B, KVH, S, HD) bf16 with {batch, head, token} strides
+ * Same head sizes, ratios and alignment rules as l3_attn_decode; no workspace.
+ */
+int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int B, int QH, int KVH, int T, int S,
+                    int HD, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                    const int64_t out_strides[3], float scale, void* stream);
+
+/*
  * The two stages of l3_attn_decode on their own, for callers that hold one sequence's KV
  * cache in several pieces (e.g. token ranges on different GPUs): every piece runs the split
  * stage on its range, the partials are concatenated along the split axis, and one combine

@@ -1,0 +1,194 @@
+// The tile loop shared by the MFMA attention kernels (decode: attn_mfma.hip, prefill:
+// attn_prefill.hip): one wavefront streams K/V tiles of a single kv head through its private LDS
+// slab and keeps an online softmax for the 16 columns of its MFMA tiles.  A column is a query
+// row: a query head of the GQA group (decode) or a (query position, query head) pair (prefill).
+//
+//   S[16 tokens x 16 columns]  = K[16 x 32 dims]          . Q^T[32 dims x 16 columns]  (per 32-dim chunk)
+//   O^T[16 dims x 16 columns] += V^T[16 dims x 32 tokens] . P[32 tokens x 16 columns]  (per 16-dim block)
+//
+// with v_mfma_f32_16x16x32_bf16.  A tile (32 tokens at HD 128, 64 at HD 64: 16 KiB of K+V) is
+// loaded with 16-byte global loads that each cover whole head rows, written to the slab and read
+// back in operand layout: ds_read_b128 for K (lane = token row, 8 consecutive dims),
+// ds_read_b64_tr_b16 for V, whose transpose turns token-major rows into "8 tokens of one dim" per
+// lane.  Slab rows are padded (16 bytes for K, 32 for V) to keep both read patterns off the same
+// banks.  The S accumulator layout (lane = column, 4 token rows) is exactly the B-operand layout
+// of the second product, so P never moves between lanes.  LDS executes one wavefront's accesses in
+// order, which is all the synchronisation the slab needs.
+#pragma once
+
+#include "attn_common.hpp"
+
+namespace l3 {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+
+#define L3_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// Keeps the compiler from moving LDS accesses across a phase boundary of the slab (the
+// hardware already executes one wavefront's LDS accesses in order).
+__device__ __forceinline__ void lds_phase_fence() { asm volatile("" ::: "memory"); }
+
+template <int HD>
+struct MfmaTile {
+    static constexpr int LPR = HD / 8;            // lanes per token row in a global load
+    static constexpr int G = kWaveSize / LPR;     // token rows per wavefront-wide load
+    static constexpr int U = 8;                   // loads of K (and of V) per tile and lane
+    static constexpr int WT = U * G;              // tokens per wavefront tile: 32 (HD 128) or 64 (HD 64)
+    static constexpr int NG = WT / 16;            // 16-token groups per tile (rows of one S tile)
+    static constexpr int KC = HD / 32;            // 32-dim chunks of the head dimension
+    static constexpr int NB = HD / 16;            // 16-dim blocks of the output
+    static constexpr int KS = WT / 32;            // 32-token steps of the second product
+    static constexpr int KPITCH = HD * 2 + 16;    // slab row pitch while it holds K
+    static constexpr int VPITCH = HD * 2 + 32;    // slab row pitch while it holds V
+    static constexpr int SLAB = WT * VPITCH;      // bytes of LDS per wavefront
+};
+
+// Streams the tiles t_first, t_first + step, ... < t_end of one kv head (kbase / vbase point at
+// this lane's 16-byte chunk of token 0; token strides in elements) and updates the wavefront's
+// softmax state.  `qfrag` is the B operand of the first product: lane (column fn, k group fg)
+// holds dims (m*4 + fg)*8 .. +8 of its column's query row.  A score of token t against this
+// lane's column counts only if t < col_limit (col_limit_min = the smallest limit in the wavefront,
+// wave-uniform; tiles below it skip the masking).  On return O[nb][r] is dim 16*nb + 4*fg + r of
+// column fn (unnormalised), m_run the column's running maximum of the raw scores (shared by its
+// four k groups) and l_part this lane's share of the column's softmax denominator.
+template <int HD>
+__device__ __forceinline__ void mfma_tile_loop(const uint16_t* kbase, const uint16_t* vbase, int64_t k_st,
+                                               int64_t v_st, unsigned char* slab,
+                                               const bf16x8_t (&qfrag)[MfmaTile<HD>::KC], int t_first, int t_end,
+                                               int step, int col_limit, int col_limit_min, float c,
+                                               f32x4_t (&O)[MfmaTile<HD>::NB], float& m_run, float& l_part) {
+    using T = MfmaTile<HD>;
+    constexpr int LPR = T::LPR, G = T::G, U = T::U, WT = T::WT, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
+    constexpr int KPITCH = T::KPITCH, VPITCH = T::VPITCH;
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int ld_row = lane / LPR;   // role in a global load: token row within the load ...
+    const int ld_c = lane % LPR;     // ... and 16-byte chunk of that row
+    const int fn = lane & 15;        // role in an MFMA operand: row/column index ...
+    const int fg = lane >> 4;        // ... and k group
+    (void)fn;
+
+    unsigned char* wr_k = slab + ld_row * KPITCH + ld_c * 16;
+    unsigned char* wr_v = slab + ld_row * VPITCH + ld_c * 16;
+    const unsigned char* rd_k = slab + (lane & 15) * KPITCH + fg * 16;
+    // transpose read: the 16 lanes of k group fg present a 4-token x 16-dim patch, row-major
+    const unsigned char* rd_v = slab + (4 * fg + ((lane & 15) >> 2)) * VPITCH + (lane & 3) * 8;
+
+    uint4 kr[U], vr[U];
+    auto issue_k = [&](int tbase) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int tok = min(tbase + u * G + ld_row, t_end - 1);  // clamped rows are masked below
+            kr[u] = load16(kbase + int64_t(tok) * k_st);
+        }
+    };
+    auto issue_v = [&](int tbase) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int tok = min(tbase + u * G + ld_row, t_end - 1);
+            vr[u] = load16(vbase + int64_t(tok) * v_st);
+        }
+    };
+
+    int t0 = t_first;
+    issue_k(t0);
+    issue_v(t0);
+    for (; t0 < t_end; t0 += step) {
+        const int tn = t0 + step;
+        // ---- K tile -> slab; its registers are free again, so the next K tile starts loading
+#pragma unroll
+        for (int u = 0; u < U; ++u) *reinterpret_cast<uint4*>(wr_k + u * G * KPITCH) = kr[u];
+        lds_phase_fence();
+        if (tn < t_end) issue_k(tn);
+
+        // ---- S = K Q^T
+        f32x4_t S[NG];
+#pragma unroll
+        for (int tg = 0; tg < NG; ++tg) {
+            S[tg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int m = 0; m < KC; ++m) {
+                const uint4 a = *reinterpret_cast<const uint4*>(rd_k + tg * 16 * KPITCH + m * 64);
+                S[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[m], S[tg],
+                                                                0, 0, 0);
+            }
+        }
+        lds_phase_fence();
+
+        // S[tg][j] is token t0 + tg*16 + 4*fg + j against column fn.  Mask what the column may not
+        // see (the ragged tail of the range; for prefill, tokens after the query's position).
+        if (t0 + WT > col_limit_min) {
+#pragma unroll
+            for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (t0 + tg * 16 + 4 * fg + j >= col_limit) S[tg][j] = kMaskedScore;
+                }
+            }
+        }
+
+        // ---- online softmax; the maximum is shared by the four k groups of a head column
+        float mloc = S[0][0];
+#pragma unroll
+        for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) mloc = fmaxf(mloc, S[tg][j]);
+        }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWaveSize));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWaveSize));
+        if (__builtin_amdgcn_ballot_w64(mloc > m_run) != 0) {  // wave-uniform: rescale only when some maximum moved
+            const float m_new = fmaxf(m_run, mloc);
+            const float alpha = fast_exp2((m_run - m_new) * c);
+            l_part *= alpha;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) O[nb] *= alpha;
+            m_run = m_new;
+        }
+        const float mc = m_run * c;
+        float psum = 0.f;
+#pragma unroll
+        for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float pj = fast_exp2(fmaf(S[tg][j], c, -mc));  // masked scores give exactly 0
+                S[tg][j] = pj;
+                psum += pj;
+            }
+        }
+        l_part += psum;
+
+        // ---- V tile -> the same slab (all K reads were issued before these writes)
+#pragma unroll
+        for (int u = 0; u < U; ++u) *reinterpret_cast<uint4*>(wr_v + u * G * VPITCH) = vr[u];
+        lds_phase_fence();
+        if (tn < t_end) issue_v(tn);
+
+        // ---- O^T += V^T P.  k slot (fg, i) of a 32-token step is token 4*fg + i of its first
+        //      16-token group for i < 4 and of its second group for i >= 4, on both operands.
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            uint4 pw;
+            pw.x = pack_bf16x2(S[2 * ks][0], S[2 * ks][1]);
+            pw.y = pack_bf16x2(S[2 * ks][2], S[2 * ks][3]);
+            pw.z = pack_bf16x2(S[2 * ks + 1][0], S[2 * ks + 1][1]);
+            pw.w = pack_bf16x2(S[2 * ks + 1][2], S[2 * ks + 1][3]);
+            const bf16x8_t pfrag = __builtin_bit_cast(bf16x8_t, pw);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, rd_v + (2 * ks) * 16 * VPITCH + nb * 32));
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, rd_v + (2 * ks + 1) * 16 * VPITCH + nb * 32));
+                const s16x8_t vv = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                O[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pfrag, O[nb],
+                                                                0, 0, 0);
+            }
+        }
+        lds_phase_fence();
+    }
+
+}
+
+}  // namespace l3

@@ -265,6 +265,37 @@ int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out
                             v_strides, out_strides, scale, num_splits, kv_len_dev, stream);
 }
 
+int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int B, int QH, int KVH, int T, int S,
+                    int HD, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                    const int64_t out_strides[3], float scale, void* stream) {
+    if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !out_strides)
+        return L3_ERR_NULL_POINTER;
+    if (int rc = check_attn_shape(B, QH, KVH, S, HD); rc != L3_OK) return rc;
+    if (T <= 0 || T > S) return L3_ERR_SHAPE;
+    if (int64_t(B) * KVH * ((int64_t(T) + 1) / 2 + kMfmaWaves) >= (int64_t(1) << 31)) return L3_ERR_SHAPE;  // grid
+    const int q_dims[3] = {B, QH, T};
+    const int kv_dims[3] = {B, KVH, S};
+    for (int i = 0; i < 3; ++i) {
+        if (q_dims[i] != 1 && (q_strides[i] < 0 || out_strides[i] < 0 || q_strides[i] % 8 || out_strides[i] % 8))
+            return L3_ERR_STRIDE;
+        if (kv_dims[i] != 1 && (k_strides[i] < 0 || v_strides[i] < 0 || k_strides[i] % 8 || v_strides[i] % 8))
+            return L3_ERR_STRIDE;
+    }
+    if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 16)) return L3_ERR_ALIGNMENT;
+    PrefillParams p;
+    p.q = static_cast<const uint16_t*>(q);
+    p.k = static_cast<const uint16_t*>(k);
+    p.v = static_cast<const uint16_t*>(v);
+    p.out = static_cast<uint16_t*>(out);
+    p.B = B; p.QH = QH; p.KVH = KVH; p.T = T; p.S = S;
+    p.q_sb = q_strides[0]; p.q_sh = q_strides[1]; p.q_st = q_strides[2];
+    p.k_sb = k_strides[0]; p.k_sh = k_strides[1]; p.k_st = k_strides[2];
+    p.v_sb = v_strides[0]; p.v_sh = v_strides[1]; p.v_st = v_strides[2];
+    p.o_sb = out_strides[0]; p.o_sh = out_strides[1]; p.o_st = out_strides[2];
+    p.scale_log2e = scale * 1.4426950408889634f;
+    return launch_attn_prefill(p, HD, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
 int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, float* part_ml,
                   int B, int QH, int KVH, int S, int HD,
                   const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],

@@ -58,7 +58,21 @@ struct AttnParams {
     float scale_log2e;
 };
 
+struct PrefillParams {
+    const uint16_t* q;   // (B, QH, T, HD) with {batch, head, token} strides
+    const uint16_t* k;   // (B, KVH, S, HD)
+    const uint16_t* v;
+    uint16_t* out;       // (B, QH, T, HD) with {batch, head, token} strides
+    int B, QH, KVH, T, S;
+    int64_t q_sb, q_sh, q_st;
+    int64_t k_sb, k_sh, k_st;
+    int64_t v_sb, v_sh, v_st;
+    int64_t o_sb, o_sh, o_st;
+    float scale_log2e;
+};
+
 // Launchers: return a hipError_t cast to int (0 = success).
+int launch_attn_prefill(const PrefillParams& p, int HD, hipStream_t stream);
 int launch_attn_splitkv_fma(const AttnParams& p, int HD, int R, hipStream_t stream);
 int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipStream_t stream);
 int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream);

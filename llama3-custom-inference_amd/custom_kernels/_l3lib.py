@@ -52,6 +52,12 @@ SIGNATURES = {
          ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64, _c_i64p, ctypes.c_int, ctypes.c_int,
          ctypes.c_void_p],
     ),
+    "l3_attn_prefill": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,  # B QH KVH T S HD
+         _c_i64p, _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_void_p],
+    ),
     "l3_attn_split": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v part_o part_ml

@@ -20,7 +20,7 @@ from . import _l3lib
 
 __all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits",
            "flash_attention_split", "flash_attention_combine", "flash_attention_decode_devlen",
-           "rot_embed_append", "add_rms_norm", "silu_mul", "argmax"]
+           "rot_embed_append", "add_rms_norm", "silu_mul", "argmax", "flash_attention_prefill"]
 
 _cu_count = {}
 _workspaces = {}  # (device index, stream handle) -> uint8 tensor
@@ -132,6 +132,44 @@ def _check_qkv(query, keys, values):
     if query.stride(3) != 1 or keys.stride(3) != 1 or values.stride(3) != 1:
         raise RuntimeError("the head dimension of query, keys and values must be contiguous")
     return B, QH, KVH, S, HD
+
+
+def flash_attention_prefill(query, keys, values):
+    """Causal GQA attention for T > 1 query tokens: query (B, QH, T, HD), keys / values
+    (B, KVH, S, HD) cache views with S >= T; query i attends to tokens 0 .. S - T + i.  Returns a
+    (B, QH, T, HD) view of a contiguous (B, T, QH, HD) tensor, so the model's
+    ``y.transpose(1, 2).contiguous()`` (model.py:120) is free.  For S == T it computes what the
+    reference asks of torch for this case (model.py:114-116).  An extension of the operator set."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("query", query)
+    _require_gpu_bf16("keys", keys)
+    _require_gpu_bf16("values", values)
+    if query.dim() != 4 or keys.dim() != 4 or tuple(values.shape) != tuple(keys.shape):
+        raise RuntimeError("flash_attention_prefill expects 4-D query, keys and values (keys and values alike)")
+    B, QH, T, HD = query.shape
+    Bk, KVH, S, HDk = keys.shape
+    if Bk != B or HDk != HD or T > S:
+        raise RuntimeError(f"shape mismatch: query {tuple(query.shape)}, keys {tuple(keys.shape)}")
+    if query.stride(3) != 1 or keys.stride(3) != 1 or values.stride(3) != 1:
+        raise RuntimeError("the head dimension of query, keys and values must be contiguous")
+    if HD not in (64, 128):
+        _fail(_l3lib.L3_ERR_HEAD_SIZE, str(HD))
+    if KVH == 0 or QH % KVH != 0 or (QH // KVH) not in (1, 2, 3, 4, 8):
+        _fail(_l3lib.L3_ERR_HEAD_RATIO, f"{QH}/{KVH}")
+    out = torch.empty((B, T, QH, HD), dtype=query.dtype, device=query.device).transpose(1, 2)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(query.device):
+        rc = lib.l3_attn_prefill(
+            query.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr(), B, QH, KVH, T, S, HD,
+            _l3lib.i64_array((query.stride(0), query.stride(1), query.stride(2))),
+            _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
+            _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
+            _l3lib.i64_array((out.stride(0), out.stride(1), out.stride(2))),
+            1.0 / math.sqrt(HD), _stream_ptr(query.device))
+    if rc != 0:
+        _fail(rc, f"B={B} QH={QH} KVH={KVH} T={T} S={S} HD={HD}")
+    return out
 
 
 def flash_attention_split(query, keys, values, num_splits: int = 0):

@@ -9,7 +9,7 @@ the same tensor layouts and views -- without its checkpoint loading:
                                                        projection, freqs), static KV cache
                                                        (maxB, L, KVH, HD) sliced and transposed,
                                                        ops.flash_attention_decode(q, k, v) when T == 1,
-                                                       torch SDPA (causal, GQA) for the prefill
+                                                       ops.flash_attention_prefill (or torch SDPA) for the prefill
   LLaMA3.forward                 model.py:203-232   -> embedding, blocks, final norm, tied lm_head
                                                        on the last position, float32 logits
   LLaMA3.generate                model.py:313-396   -> prompt mask keep, argmax when temperature is 0,
@@ -116,11 +116,15 @@ class LlamaDecoder:
         return F.linear(y, L["c_proj"])
 
     def _prefill_attention(self, q, k, v):
-        """Causal GQA attention for T > 1: stock PyTorch, as in the reference (model.py:114-116),
-        which pins the FLASH backend; here whichever fused backend this build offers is used."""
-        y = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
-        self.prefill_backend = "torch.sdpa(default backend selection)"
-        return y
+        """Causal GQA attention for T > 1.  The reference hands this case to torch
+        (model.py:114-116); here it goes through the library's prefill kernel when the operator
+        module provides one (the CPU stand-in does not and uses torch, like the reference)."""
+        op = getattr(self.ops, "flash_attention_prefill", None)
+        if op is not None:
+            self.prefill_backend = "l3 prefill kernel"
+            return op(q, k, v)
+        self.prefill_backend = "torch.sdpa"
+        return F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
 
     def forward(self, idx, start_pos=0):
         """idx (B, T) token ids -> float32 logits (B, 1, vocab) of the last position."""
@@ -341,7 +345,7 @@ def timed_generate(model, batch, input_len, gen_len, seed=42, sync=None, graphed
 
 
 def bench_e2e(args, torch_mod, dev):
-    """bench.py --workload e2e: BASELINE config 5 (16 layers, hidden 2048, 32/8 heads, head_dim 64,
+    """bench.py --workload e2e: the end-to-end configuration (16 layers, hidden 2048, 32/8 heads, head_dim 64,
     FFN 8192, vocab 128256 tied, N(0, 0.02) weights, 128 random prompt ids + 128 greedy tokens) at
     batch 1 and 64, every RMSNorm / rotary / decode-attention call going through the HIP operators."""
     import os

@@ -8,6 +8,7 @@ missing instead of falling back to anything in here.
 
 What is restated, and from where (paths relative to the reference checkout):
 
+* prefill attention     model.py:114-116 (what the reference asks of torch for T > 1).
 * decode attention      custom_kernels/custom_kernels.cu:233-253 (shape, stride
                         and scale conventions), :55 and :163 (GQA head mapping,
                         output layout).  The arithmetic is textbook softmax
@@ -34,6 +35,7 @@ from .bf16 import (  # noqa: F401
 )
 from .ops_ref import (  # noqa: F401
     attention_decode_ref,
+    attention_prefill_ref,
     attention_split_partials_ref,
     lse_combine_ref,
     precompute_freqs_cis_ref,

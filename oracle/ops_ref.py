@@ -40,6 +40,33 @@ def attention_decode_ref(q, k, v, scale=None) -> np.ndarray:
     return o.reshape(B, QH, 1, HD)
 
 
+def attention_prefill_ref(q, k, v, scale=None) -> np.ndarray:
+    """Causal GQA attention for T query tokens against S >= T cached tokens.
+
+    q (B, QH, T, HD); k, v (B, KVH, S, HD); returns (B, QH, T, HD) float64.  Query i sits at
+    absolute position S - T + i and attends to tokens 0 .. S - T + i; for S == T this is the
+    is_causal mask of the scaled_dot_product_attention call the reference makes for T > 1
+    (model.py:114-116).  Head mapping and scale as in attention_decode_ref.
+    """
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    B, QH, T, HD = q.shape
+    _, KVH, S, _ = k.shape
+    assert S >= T and QH % KVH == 0
+    R = QH // KVH
+    if scale is None:
+        scale = 1.0 / math.sqrt(HD)
+    qg = q.reshape(B, KVH, R, T, HD)
+    s = np.einsum("bgrtd,bgsd->bgrts", qg, k) * scale
+    allowed = np.arange(S)[None, :] <= (S - T + np.arange(T))[:, None]
+    s = np.where(allowed, s, -np.inf)
+    s -= s.max(axis=-1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(axis=-1, keepdims=True)
+    return np.einsum("bgrts,bgsd->bgrtd", p, v).reshape(B, QH, T, HD)
+
+
 def attention_split_partials_ref(q, k, v, bounds, scale=None):
     """Per-split unnormalised partials over token ranges ``bounds`` = [0, ..., S].
 

@@ -13,7 +13,7 @@ from helpers import make_qkv, randn_bf16, t2bits
 
 ATTN_CASES = {
     # name: (B, QH, KVH, S, HD, cache_len, seed)
-    "c1_llama32_1b_s256": (1, 32, 8, 256, 64, None, 42),          # BASELINE config 1
+    "c1_llama32_1b_s256": (1, 32, 8, 256, 64, None, 42),          # Llama-3.2-1B decode shape, KV length 256
     "hd128_s130_cacheview": (1, 32, 8, 130, 128, 192, 43),        # ragged S, batch stride of a longer cache
     "b2_r4_s200": (2, 8, 2, 200, 64, None, 44),
     "r1_s65": (2, 4, 4, 65, 64, None, 45),

@@ -148,3 +148,22 @@ def test_stage_entry_points_argument_checks():
     assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 0, 32, 64, 4, qs, None) == _l3lib.L3_ERR_SHAPE
     assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 2, 32, 64, 4, _l3lib.i64_array((2049, 64)), None) \
         == _l3lib.L3_ERR_STRIDE
+
+
+def test_prefill_argument_checks():
+    lib = _l3lib.load()
+    qs, ks = _l3lib.i64_array((131072, 64, 2048)), _l3lib.i64_array((131072, 64, 512))
+
+    def call(q=FAKE, out=FAKE, B=1, QH=32, KVH=8, T=16, S=64, HD=64, q_strides=qs, k_strides=ks):
+        return lib.l3_attn_prefill(q, FAKE, FAKE, out, B, QH, KVH, T, S, HD, q_strides, k_strides, k_strides,
+                                   q_strides, 0.125, None)
+
+    assert call(out=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert call(HD=96) == _l3lib.L3_ERR_HEAD_SIZE
+    assert call(QH=40) == _l3lib.L3_ERR_HEAD_RATIO      # ratio 5
+    assert call(QH=30) == _l3lib.L3_ERR_SHAPE           # not a multiple of KVH
+    assert call(T=0) == _l3lib.L3_ERR_SHAPE
+    assert call(T=65) == _l3lib.L3_ERR_SHAPE              # more queries than cached tokens
+    assert call(q=FAKE + 8) == _l3lib.L3_ERR_ALIGNMENT
+    assert call(q_strides=_l3lib.i64_array((131072, 64, 2052))) == _l3lib.L3_ERR_STRIDE
+    assert call(k_strides=_l3lib.i64_array((131072, -64, 512))) == _l3lib.L3_ERR_STRIDE

@@ -158,7 +158,7 @@ def test_runs_on_the_current_stream(gpu):
     np.testing.assert_array_equal(t2bits(out), t2bits(ref))
 
 
-# ---- BASELINE.json shapes at full size (oracle in float64, chunked over the batch)
+# ---- the benchmark configurations at full size (oracle in float64, chunked over the batch)
 FULL = {
     "c1": (1, 32, 8, 256, 64),
     "c2_s512": (1, 32, 8, 512, 128),
@@ -251,3 +251,64 @@ def test_device_side_kv_length(gpu, HD, B, L):
         # a forced split count (streaming form of the kernel) agrees to bf16 rounding
         forced = cke.flash_attention_decode_devlen(qg, kg, vg, kv_len, 3)
         assert (out.float() - forced.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, np.abs(ref).max())
+
+
+def test_concurrent_streams_do_not_share_scratch(gpu):
+    """Two streams run split + combine calls at the same time; each stream has its own workspace
+    in the shim, so the results must equal the serial ones bit for bit."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    a = make_qkv(1, 32, 8, 6000, 128, seed=51, device=gpu)
+    b = make_qkv(1, 32, 8, 5000, 128, seed=52, device=gpu)
+    ra, rb = cke.flash_attention_decode(*a), cke.flash_attention_decode(*b)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(device=gpu), torch.cuda.Stream(device=gpu)
+    outs_a, outs_b = [], []
+    for _ in range(20):
+        with torch.cuda.stream(s1):
+            outs_a.append(cke.flash_attention_decode(*a))
+        with torch.cuda.stream(s2):
+            outs_b.append(cke.flash_attention_decode(*b))
+    torch.cuda.synchronize()
+    for o in outs_a:
+        np.testing.assert_array_equal(t2bits(o), t2bits(ra))
+    for o in outs_b:
+        np.testing.assert_array_equal(t2bits(o), t2bits(rb))
+
+
+# ---- causal prefill (T > 1) through the same tile loop
+@pytest.mark.parametrize("HD", [64, 128])
+@pytest.mark.parametrize("B,QH,KVH,T,S", [(1, 32, 8, 128, 128), (2, 8, 2, 37, 37), (1, 4, 4, 16, 16), (3, 24, 8, 5, 5),
+                                           (1, 16, 2, 130, 130), (2, 32, 8, 64, 200), (1, 8, 8, 2, 2),
+                                           (1, 32, 8, 1000, 1000), (1, 6, 3, 33, 40)])
+def test_prefill_against_oracle(gpu, HD, B, QH, KVH, T, S):
+    from custom_kernels import custom_kernels_extension as cke
+    from oracle import attention_prefill_ref
+
+    print(f"prefill B={B} QH={QH} KVH={KVH} T={T} S={S} HD={HD}", flush=True)
+    L = S + 7   # the cache is longer than what is attended
+    q = randn_bf16((B, T, QH, HD), 61)
+    kc = randn_bf16((B, L, KVH, HD), 62)
+    vc = randn_bf16((B, L, KVH, HD), 63)
+    out = cke.flash_attention_prefill(q.to(gpu).transpose(1, 2), kc.to(gpu)[:, :S].transpose(1, 2),
+                                      vc.to(gpu)[:, :S].transpose(1, 2))
+    torch.cuda.synchronize()
+    assert out.shape == (B, QH, T, HD) and out.transpose(1, 2).is_contiguous()
+    ref = attention_prefill_ref(t2f32(q.transpose(1, 2)), t2f32(kc[:, :S].transpose(1, 2)),
+                                t2f32(vc[:, :S].transpose(1, 2)))
+    assert_attn_close(out, ref, what=f"prefill T={T} S={S} HD={HD}")
+
+
+def test_prefill_last_row_equals_decode(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, QH, KVH, T, HD = 2, 32, 8, 96, 64
+    q = randn_bf16((B, T, QH, HD), 71).to(gpu).transpose(1, 2)
+    k = randn_bf16((B, T, KVH, HD), 72).to(gpu).transpose(1, 2)
+    v = randn_bf16((B, T, KVH, HD), 73).to(gpu).transpose(1, 2)
+    pre = cke.flash_attention_prefill(q, k, v)
+    dec = cke.flash_attention_decode(q[:, :, T - 1:T], k, v)
+    torch.cuda.synchronize()
+    assert (pre[:, :, T - 1:T].float() - dec.float()).abs().max().item() <= 2.0 ** -7
+    with pytest.raises(RuntimeError):
+        cke.flash_attention_prefill(q, k[:, :, :10], v[:, :, :10])     # fewer cached tokens than queries

@@ -94,3 +94,44 @@ def test_split_then_combine_reproduces_unsplit(bounds):
     if len(bounds) > 2:
         mean_of_splits = (o / l[..., None]).mean(axis=0)[:, :, None, :]
         assert np.abs(mean_of_splits - full).max() > 1e-2
+
+
+# ------------------------------------------------------------------ causal prefill oracle
+from oracle import attention_prefill_ref  # noqa: E402
+
+
+def _prefill_inputs(B, QH, KVH, T, S, HD, seed):
+    from helpers import randn_bf16
+    q = randn_bf16((B, T, QH, HD), seed).transpose(1, 2)
+    k = randn_bf16((B, S, KVH, HD), seed + 1).transpose(1, 2)
+    v = randn_bf16((B, S, KVH, HD), seed + 2).transpose(1, 2)
+    return q, k, v
+
+
+@pytest.mark.parametrize("B,QH,KVH,T,HD", [(1, 8, 2, 17, 64), (2, 4, 4, 5, 128), (1, 12, 4, 33, 64)])
+def test_prefill_matches_torch_causal_sdpa(B, QH, KVH, T, HD):
+    q, k, v = _prefill_inputs(B, QH, KVH, T, T, HD, seed=T)
+    ref = attention_prefill_ref(t2f32(q), t2f32(k), t2f32(v))
+    lib = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True, enable_gqa=True)
+    np.testing.assert_allclose(ref, lib.numpy(), rtol=2e-5, atol=2e-6)
+
+
+def test_prefill_rows_are_decode_calls_on_prefixes():
+    """Row i of a prefill over S cached tokens is single-token attention over the first S-T+i+1
+    tokens; the first row of a prompt from position 0 sees only token 0."""
+    B, QH, KVH, T, S, HD = 2, 8, 2, 6, 10, 64
+    q, k, v = (t2f32(t) for t in _prefill_inputs(B, QH, KVH, T, S, HD, seed=3))
+    ref = attention_prefill_ref(q, k, v)
+    for i in range(T):
+        n = S - T + i + 1
+        row = attention_decode_ref(q[:, :, i:i + 1], k[:, :, :n], v[:, :, :n])
+        np.testing.assert_allclose(ref[:, :, i:i + 1], row, atol=1e-13)
+    q2, k2, v2 = (t2f32(t) for t in _prefill_inputs(1, 4, 2, 5, 5, 64, seed=4))
+    first = attention_prefill_ref(q2, k2, v2)[:, :, 0]
+    np.testing.assert_allclose(first, np.repeat(v2[:, :, 0], 2, axis=1), atol=1e-13)
+    # an explicit mask with the same alignment gives the same thing through torch
+    mask = torch.ones(T, S, dtype=torch.bool).tril(diagonal=S - T)
+    lib = F.scaled_dot_product_attention(torch.from_numpy(q).double(), torch.from_numpy(k).double(),
+                                         torch.from_numpy(v).double(),
+                                         attn_mask=mask, enable_gqa=True)
+    np.testing.assert_allclose(ref, lib.numpy(), rtol=1e-9, atol=1e-12)
