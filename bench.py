@@ -14,7 +14,7 @@ Prints ONE JSON line: value = algorithmic GB/s (K+V+Q read, O written) over the 
 steps; "roofline" prices the same bytes against the 8 TB/s HBM peak from HIP-event timing;
 "cpu_baseline" is stock PyTorch on the host cores for a bounded sample of the same sweep.
 
-Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|e2e|copy) report the remaining configurations
+Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|prefill|e2e|copy) report the remaining configurations
 in the same format.
 """
 
@@ -339,6 +339,62 @@ def run_rows(args, torch, lib, l3, dev, name):
     }
 
 
+def run_prefill(args, torch, lib, l3, dev):
+    """Causal prefill attention (T query tokens against T cached tokens).  Compute-bound: priced
+    against the dense bf16 MFMA peak with the causal flop count 4*HD per (query, attended token)
+    pair.  torch's own scaled_dot_product_attention on the same tensors is timed beside it."""
+    import torch.nn.functional as F
+    from custom_kernels import custom_kernels_extension as cke
+
+    MFMA_PEAK_TFLOPS = 2500.0
+    shapes = [(1, 32, 8, 128, 64), (2, 32, 8, 2048, 64), (1, 32, 8, 2048, 128), (1, 32, 8, 4096, 128),
+              (1, 32, 8, 8192, 128)]
+    detail, head = [], None
+    for (B, QH, KVH, T, HD) in shapes:
+        g = torch.Generator().manual_seed(SEED)
+        q = torch.randn((B, T, QH, HD), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+        k = torch.randn((B, T, KVH, HD), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+        v = torch.randn((B, T, KVH, HD), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+        flops = 4.0 * B * QH * HD * (T * (T + 1) / 2)
+        reps = 8
+        cke.flash_attention_prefill(q, k, v)
+        gph = capture_graph(torch, lambda: [cke.flash_attention_prefill(q, k, v) for _ in range(reps)])
+        gph.replay()
+        ms = event_time_ms(torch, gph.replay, 5) / reps
+        try:
+            F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+            sd_ms = event_time_ms(torch, lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True,
+                                                                                enable_gqa=True), 10)
+        except Exception as exc:  # informational only
+            sd_ms = None
+            print(f"bench.py: torch SDPA failed for {B, QH, KVH, T, HD}: {exc}", file=sys.stderr)
+        rec = {"B": B, "QH": QH, "KVH": KVH, "T": T, "HD": HD, "us": round(ms * 1e3, 2),
+               "TFLOPs": round(flops / ms / 1e9, 1), "frac": round(flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4),
+               "flops": flops, "torch_sdpa_us": None if sd_ms is None else round(sd_ms * 1e3, 2)}
+        detail.append(rec)
+        if (B, T, HD) == (2, 2048, 64):
+            head = (rec, ms, q, k, v)
+    rec, ms, q, k, v = head
+    cpu = None
+    if not args.no_cpu_baseline:
+        qc, kc, vc = q.cpu(), k.cpu(), v.cpu()
+        sec, n = time_cpu(lambda: F.scaled_dot_product_attention(qc, kc, vc, is_causal=True, enable_gqa=True),
+                          min(args.cpu_seconds, 10.0))
+        cpu = {"value": round(rec["flops"] / sec / 1e12, 3), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+               "kind": "port", "host_cpus": os.cpu_count(),
+               "sample": f"{n} runs of the same shape with torch CPU scaled_dot_product_attention (bf16, causal)"}
+    return {
+        "metric": "prefill_attn_TFLOPs", "value": rec["TFLOPs"], "unit": "TFLOP/s", "steps": args.steps,
+        "ms_per_step": round(ms, 5), "dtype": "bf16",
+        "config": {"workload": "causal prefill attention: B2 QH32 KVH8 HD64 bf16, 2048 tokens (the 2x2048-token "
+                               "prefill of the 1B shape)", "accumulate": "f32", "launch": "hip graph", "seed": SEED},
+        "roofline": {"bound": "mfma", "achieved": rec["TFLOPs"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": rec["frac"], "traffic": None, "kernel": "attn_prefill_mfma_kernel",
+                     "algorithmic_flops_per_launch": rec["flops"]},
+        "cpu_baseline": cpu, "per_shape": detail,
+    }
+
+
 def run_copy(args, torch, dev):
     """A plain device copy of known size (torch's copy kernel): the yardstick that the FETCH_SIZE /
     WRITE_SIZE counters are scaled by, and the practical rate of a read+write stream."""
@@ -367,7 +423,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "e2e", "copy"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "prefill", "e2e", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall time spent on the CPU baseline sample")
     ap.add_argument("--e2e-batch", type=int, default=1)
@@ -403,6 +459,8 @@ def main():
         res = run_attention(args, torch, lib, l3, dev, args.workload)
     elif args.workload in ("rms", "rope"):
         res = run_rows(args, torch, lib, l3, dev, args.workload)
+    elif args.workload == "prefill":
+        res = run_prefill(args, torch, lib, l3, dev)
     elif args.workload == "copy":
         res = run_copy(args, torch, dev)
     else:
