@@ -357,10 +357,17 @@ def run_prefill(args, torch, lib, l3, dev):
         v = torch.randn((B, T, KVH, HD), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
         flops = 4.0 * B * QH * HD * (T * (T + 1) / 2)
         reps = 8
-        cke.flash_attention_prefill(q, k, v)
-        gph = capture_graph(torch, lambda: [cke.flash_attention_prefill(q, k, v) for _ in range(reps)])
-        gph.replay()
-        ms = event_time_ms(torch, gph.replay, 5) / reps
+        forms = {}
+        for fname, form in (("auto", l3.L3_ATTN_PREFILL_AUTO), ("wave", l3.L3_ATTN_PREFILL_WAVE),
+                            ("tiled", l3.L3_ATTN_PREFILL_TILED)):
+            prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, form)
+            cke.flash_attention_prefill(q, k, v)
+            gph = capture_graph(torch, lambda: [cke.flash_attention_prefill(q, k, v) for _ in range(reps)])
+            gph.replay()
+            forms[fname] = event_time_ms(torch, gph.replay, 5) / reps
+            del gph
+            lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, prev)
+        ms = forms["auto"]
         try:
             F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
             sd_ms = event_time_ms(torch, lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True,
@@ -370,7 +377,9 @@ def run_prefill(args, torch, lib, l3, dev):
             print(f"bench.py: torch SDPA failed for {B, QH, KVH, T, HD}: {exc}", file=sys.stderr)
         rec = {"B": B, "QH": QH, "KVH": KVH, "T": T, "HD": HD, "us": round(ms * 1e3, 2),
                "TFLOPs": round(flops / ms / 1e9, 1), "frac": round(flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4),
-               "flops": flops, "torch_sdpa_us": None if sd_ms is None else round(sd_ms * 1e3, 2)}
+               "flops": flops, "wave_form_us": round(forms["wave"] * 1e3, 2),
+               "tiled_form_us": round(forms["tiled"] * 1e3, 2),
+               "torch_sdpa_us": None if sd_ms is None else round(sd_ms * 1e3, 2)}
         detail.append(rec)
         if (B, T, HD) == (2, 2048, 64):
             head = (rec, ms, q, k, v)

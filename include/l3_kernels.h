@@ -56,10 +56,17 @@ const char* l3_strerror(int code);
  * L3_ATTN_OPT_KERNEL; returns the previous value; a `value` other than the two kernels only
  * queries.  The initial value is MFMA unless the environment variable L3_ATTN_IMPL is "fma".
  * Split planning depends on the kernel, so choose before sizing workspaces.
+ *
+ * L3_ATTN_OPT_PREFILL chooses the form of l3_attn_prefill in the same way: AUTO (by prompt
+ * length), WAVE (every wavefront streams K/V on its own) or TILED (a workgroup shares K/V tiles).
  */
 #define L3_ATTN_OPT_KERNEL 0
 #define L3_ATTN_KERNEL_FMA 0
 #define L3_ATTN_KERNEL_MFMA 1
+#define L3_ATTN_OPT_PREFILL 1
+#define L3_ATTN_PREFILL_AUTO 0
+#define L3_ATTN_PREFILL_WAVE 1
+#define L3_ATTN_PREFILL_TILED 2
 int l3_attn_set_option(int option, int value);
 
 /*

@@ -61,6 +61,7 @@ int current_device_cus() {
 
 namespace {
 std::atomic<int> g_attn_kernel{-1};  // -1: not chosen yet
+std::atomic<int> g_prefill_form{L3_ATTN_PREFILL_AUTO};
 }  // namespace
 
 int attn_kernel_option() {
@@ -136,6 +137,12 @@ const char* l3_strerror(int code) {
 }
 
 int l3_attn_set_option(int option, int value) {
+    if (option == L3_ATTN_OPT_PREFILL) {
+        const int prev_form = g_prefill_form.load(std::memory_order_relaxed);
+        if (value == L3_ATTN_PREFILL_AUTO || value == L3_ATTN_PREFILL_WAVE || value == L3_ATTN_PREFILL_TILED)
+            g_prefill_form.store(value, std::memory_order_relaxed);
+        return prev_form;
+    }
     if (option != L3_ATTN_OPT_KERNEL) return L3_ERR_SHAPE;
     const int prev = attn_kernel_option();
     if (value == L3_ATTN_KERNEL_FMA || value == L3_ATTN_KERNEL_MFMA) g_attn_kernel.store(value, std::memory_order_relaxed);
@@ -293,7 +300,18 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     p.v_sb = v_strides[0]; p.v_sh = v_strides[1]; p.v_st = v_strides[2];
     p.o_sb = out_strides[0]; p.o_sh = out_strides[1]; p.o_st = out_strides[2];
     p.scale_log2e = scale * 1.4426950408889634f;
-    return launch_attn_prefill(p, HD, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+    // Long prompts share K/V tiles across a workgroup; short ones (few columns per kv head) are
+    // better spread over many independent wavefronts.
+    int form = g_prefill_form.load(std::memory_order_relaxed);
+    if (form == L3_ATTN_PREFILL_AUTO) {
+        const int wg_pos = prefill_tiled_positions_per_wg(QH / KVH);
+        const int64_t tiled_wgs = int64_t(B) * KVH * ((T + wg_pos - 1) / wg_pos);
+        form = (T >= 4 * wg_pos && tiled_wgs >= current_device_cus() / 2) ? L3_ATTN_PREFILL_TILED
+                                                                          : L3_ATTN_PREFILL_WAVE;
+    }
+    const int rc = (form == L3_ATTN_PREFILL_TILED) ? launch_attn_prefill_tiled(p, HD, static_cast<hipStream_t>(stream))
+                                                   : launch_attn_prefill(p, HD, static_cast<hipStream_t>(stream));
+    return rc == 0 ? L3_OK : L3_ERR_HIP;
 }
 
 int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, float* part_ml,

@@ -23,6 +23,10 @@ L3_ATTN_MAX_SPLITS = 512
 L3_ATTN_OPT_KERNEL = 0
 L3_ATTN_KERNEL_FMA = 0
 L3_ATTN_KERNEL_MFMA = 1
+L3_ATTN_OPT_PREFILL = 1
+L3_ATTN_PREFILL_AUTO = 0
+L3_ATTN_PREFILL_WAVE = 1
+L3_ATTN_PREFILL_TILED = 2
 
 # name -> (restype, argtypes); mirrors include/l3_kernels.h line by line
 _c_i64p = ctypes.POINTER(ctypes.c_int64)

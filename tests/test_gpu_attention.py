@@ -280,12 +280,13 @@ def test_concurrent_streams_do_not_share_scratch(gpu):
 @pytest.mark.parametrize("HD", [64, 128])
 @pytest.mark.parametrize("B,QH,KVH,T,S", [(1, 32, 8, 128, 128), (2, 8, 2, 37, 37), (1, 4, 4, 16, 16), (3, 24, 8, 5, 5),
                                            (1, 16, 2, 130, 130), (2, 32, 8, 64, 200), (1, 8, 8, 2, 2),
-                                           (1, 32, 8, 1000, 1000), (1, 6, 3, 33, 40)])
-def test_prefill_against_oracle(gpu, HD, B, QH, KVH, T, S):
+                                           (1, 32, 8, 1000, 1000), (1, 6, 3, 33, 40), (1, 16, 16, 300, 300),
+                                           (1, 16, 2, 257, 321)])
+def test_prefill_against_oracle(gpu, prefill_form, HD, B, QH, KVH, T, S):
     from custom_kernels import custom_kernels_extension as cke
     from oracle import attention_prefill_ref
 
-    print(f"prefill B={B} QH={QH} KVH={KVH} T={T} S={S} HD={HD}", flush=True)
+    print(f"prefill form={prefill_form} B={B} QH={QH} KVH={KVH} T={T} S={S} HD={HD}", flush=True)
     L = S + 7   # the cache is longer than what is attended
     q = randn_bf16((B, T, QH, HD), 61)
     kc = randn_bf16((B, L, KVH, HD), 62)
@@ -297,6 +298,36 @@ def test_prefill_against_oracle(gpu, HD, B, QH, KVH, T, S):
     ref = attention_prefill_ref(t2f32(q.transpose(1, 2)), t2f32(kc[:, :S].transpose(1, 2)),
                                 t2f32(vc[:, :S].transpose(1, 2)))
     assert_attn_close(out, ref, what=f"prefill T={T} S={S} HD={HD}")
+
+
+def test_prefill_forms_agree_on_a_long_prompt(gpu):
+    """2048 tokens (the auto choice is the tiled form): tiled and wavefront-private forms against
+    each other, and sampled rows against the float64 oracle."""
+    from custom_kernels import _l3lib as l3
+    from custom_kernels import custom_kernels_extension as cke
+    from oracle import attention_decode_ref
+
+    lib = l3.load()
+    B, QH, KVH, T, HD = 2, 32, 8, 2048, 128
+    q = randn_bf16((B, T, QH, HD), 81)
+    k = randn_bf16((B, T, KVH, HD), 82)
+    v = randn_bf16((B, T, KVH, HD), 83)
+    qd, kd, vd = (t.to(gpu).transpose(1, 2) for t in (q, k, v))
+    outs = {}
+    for name, form in (("auto", l3.L3_ATTN_PREFILL_AUTO), ("wave", l3.L3_ATTN_PREFILL_WAVE),
+                       ("tiled", l3.L3_ATTN_PREFILL_TILED)):
+        print(f"long prefill form={name}", flush=True)
+        prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, form)
+        try:
+            outs[name] = cke.flash_attention_prefill(qd, kd, vd).float().cpu()
+        finally:
+            lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, prev)
+    assert torch.equal(outs["auto"], outs["tiled"])
+    assert (outs["wave"] - outs["tiled"]).abs().max().item() <= 2.0 ** -6
+    for i in (0, 1, 63, 64, 65, 1000, 2047):
+        ref = attention_decode_ref(t2f32(q[:, i:i + 1].transpose(1, 2)), t2f32(k[:, :i + 1].transpose(1, 2)),
+                                   t2f32(v[:, :i + 1].transpose(1, 2)))
+        assert_attn_close(outs["tiled"][:, :, i:i + 1], ref, what=f"long prefill row {i}")
 
 
 def test_prefill_last_row_equals_decode(gpu):
