@@ -14,7 +14,7 @@ Prints ONE JSON line: value = algorithmic GB/s (K+V+Q read, O written) over the 
 steps; "roofline" prices the same bytes against the 8 TB/s HBM peak from HIP-event timing;
 "cpu_baseline" is stock PyTorch on the host cores for a bounded sample of the same sweep.
 
-Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|prefill|e2e|copy) report the remaining configurations
+Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|prefill|linear|e2e|copy) report the remaining configurations
 in the same format.
 """
 
@@ -404,6 +404,72 @@ def run_prefill(args, torch, lib, l3, dev):
     }
 
 
+def run_linear(args, torch, lib, l3, dev):
+    """The nn.Linear calls of one decode step of the 1B architecture (model.py:95,121,134,225) at
+    batch 1 and 64 through l3_linear_decode / l3_linear_swiglu_decode: a stream over the weight
+    matrix, priced against HBM.  Each shape owns enough weight copies that the Infinity Cache
+    cannot hold them; stock F.linear (hipBLASLt) on the same tensors is timed beside it."""
+    import torch.nn.functional as F
+    from custom_kernels import custom_kernels_extension as cke
+
+    shapes = [("c_attn", 3072, 2048, False), ("c_proj", 2048, 2048, False), ("mlp gate+up (SwiGLU)", 8192, 2048, True),
+              ("mlp c_proj", 2048, 8192, False), ("lm_head", 128256, 2048, False)]
+    detail, head = [], None
+    for M in (1, 64):
+        total_us, total_bytes, torch_us = 0.0, 0, 0.0
+        for (name, N, K, swiglu) in shapes:
+            wbytes = N * K * 2 * (2 if swiglu else 1)
+            copies = max(2, min(48, (1 << 30) // wbytes + 1))
+            g = torch.Generator().manual_seed(SEED)
+            x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(dev)
+            w0 = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(dev)
+            ws = [w0] + [w0.clone() for _ in range(copies - 1)]
+            ws2 = [w.clone() for w in ws] if swiglu else None
+            if swiglu:
+                run_l3 = lambda: [cke.linear_swiglu_decode(x, a, b) for a, b in zip(ws, ws2)]  # noqa: E731
+                run_t = lambda: [F.silu(F.linear(x, a)) * F.linear(x, b) for a, b in zip(ws, ws2)]  # noqa: E731
+            else:
+                run_l3 = lambda: [cke.linear_decode(x, a) for a in ws]  # noqa: E731
+                run_t = lambda: [F.linear(x, a) for a in ws]  # noqa: E731
+            run_l3()
+            gph = capture_graph(torch, run_l3)
+            gph.replay()
+            ms = event_time_ms(torch, gph.replay, 5) / copies
+            del gph
+            run_t()
+            gph = capture_graph(torch, run_t)
+            gph.replay()
+            tms = event_time_ms(torch, gph.replay, 5) / copies
+            del gph
+            nbytes = wbytes + M * K * 2 + M * N * 2
+            detail.append({"M": M, "layer": name, "N": N, "K": K, "us": round(ms * 1e3, 2),
+                           "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                           "bytes": nbytes, "torch_us": round(tms * 1e3, 2)})
+            per_token = 1 if name == "lm_head" else 16
+            total_us += ms * 1e3 * per_token
+            torch_us += tms * 1e3 * per_token
+            total_bytes += nbytes * per_token
+            del ws, ws2
+            torch.cuda.empty_cache()
+        detail.append({"M": M, "layer": "all linears of one decode step (16 layers + lm_head)",
+                       "us": round(total_us, 1), "GBps": round(total_bytes / total_us / 1e3, 1),
+                       "frac": round(total_bytes / total_us / 1e3 / HBM_PEAK_GBPS, 4), "bytes": total_bytes,
+                       "torch_us": round(torch_us, 1)})
+        if M == 1:
+            head = detail[-1]
+    return {
+        "metric": "decode_linear_hbm_GBps", "value": head["GBps"], "unit": "GB/s", "frac_of_hbm_peak": head["frac"],
+        "steps": args.steps, "ms_per_step": round(head["us"] / 1e3, 5), "dtype": "bf16",
+        "config": {"workload": "all nn.Linear calls of one batch-1 decode step of the Llama-3.2-1B architecture "
+                               "(16 x [c_attn, c_proj, gate+up with SwiGLU, mlp c_proj] + lm_head), weights "
+                               "N(0, 0.02)", "accumulate": "f32", "launch": "hip graph", "seed": SEED},
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": head["frac"], "traffic": None, "kernel": "linear_skinny_kernel",
+                     "algorithmic_bytes_per_launch": head["bytes"] // 65},
+        "cpu_baseline": None, "per_shape": detail,
+    }
+
+
 def run_copy(args, torch, dev):
     """A plain device copy of known size (torch's copy kernel): the yardstick that the FETCH_SIZE /
     WRITE_SIZE counters are scaled by, and the practical rate of a read+write stream."""
@@ -432,7 +498,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "prefill", "e2e", "copy"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "prefill", "linear", "e2e", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall time spent on the CPU baseline sample")
     ap.add_argument("--e2e-batch", type=int, default=1)
@@ -470,6 +536,8 @@ def main():
         res = run_rows(args, torch, lib, l3, dev, args.workload)
     elif args.workload == "prefill":
         res = run_prefill(args, torch, lib, l3, dev)
+    elif args.workload == "linear":
+        res = run_linear(args, torch, lib, l3, dev)
     elif args.workload == "copy":
         res = run_copy(args, torch, dev)
     else:

@@ -200,6 +200,28 @@ int l3_add_rms_norm(const void* x, const void* residual, const void* w, void* su
 int l3_silu_mul(const void* a, const void* b, void* y, int64_t n, void* stream);
 
 /*
+ * y[M, N] = x[M, K] . w[N, K]^T for the few activation rows of a decode step: bf16 in and out,
+ * float32 accumulation, one rounding.  Stands where the reference calls nn.Linear with T == 1
+ * (model.py:95 c_attn, :121 c_proj, :134 mlp c_proj, :225 lm_head); hipBLASLt treats these as
+ * GEMMs, this entry point as a single pass over the weight matrix at HBM speed.
+ * 1 <= M <= L3_LINEAR_MAX_ROWS; N % 4 == 0; K % 32 == 0; strides are row strides in elements
+ * (x_stride, w_stride >= K and multiples of 8; y_stride >= N and a multiple of 4); x and w
+ * 16-byte aligned, y 8-byte aligned.  Needs no workspace.
+ */
+#define L3_LINEAR_MAX_ROWS 64
+int l3_linear_decode(const void* x, const void* w, void* y, int M, int N, int K, int64_t x_stride,
+                     int64_t w_stride, int64_t y_stride, void* stream);
+
+/*
+ * y[M, N] = silu(x . w_gate^T) * (x . w_up^T) in one pass over both weight matrices: the
+ * SwiGLU front half of model.py:134 (F.silu(c_fc2(x)) * c_fc(x)).  Both products and the silu
+ * are rounded to bf16 before the multiplication, as the three separate torch operators do.
+ * Same constraints as l3_linear_decode; w_gate and w_up share w_stride.
+ */
+int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up, void* y, int M, int N, int K,
+                            int64_t x_stride, int64_t w_stride, int64_t y_stride, void* stream);
+
+/*
  * out[r] = index of the first maximum of the bf16 row logits[r*row_stride : r*row_stride + V]
  * (int64, like torch.argmax; a row of NaNs gives 0): the greedy pick of model.py:371.  Two small
  * launches (per-chunk maxima into the caller's workspace of l3_argmax_workspace_bytes(rows, V)

@@ -11,12 +11,7 @@ namespace {
 
 constexpr int kMiscThreads = 256;
 
-// y = bf16( bf16(silu(a)) * b ): the intermediate rounding reproduces torch's F.silu(a) * b,
-// where silu's bf16 result is materialised before the multiplication.
-__device__ __forceinline__ float silu_rounded(float a) {
-    const float s = a / (1.0f + expf(-a));
-    return __uint_as_float(f32_to_bf16_bits(s) << 16);
-}
+// y = bf16( bf16(silu(a)) * b ) with silu_rounded of l3_device.hpp.
 
 __global__ void __launch_bounds__(kMiscThreads)
 silu_mul_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ y,

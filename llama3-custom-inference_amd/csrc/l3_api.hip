@@ -389,6 +389,41 @@ int l3_silu_mul(const void* a, const void* b, void* y, int64_t n, void* stream) 
                ? L3_OK : L3_ERR_HIP;
 }
 
+namespace {
+
+int linear_decode_impl(const void* x, const void* w0, const void* w1, void* y, int M, int N, int K, int64_t x_stride,
+                       int64_t w_stride, int64_t y_stride, bool swiglu, void* stream) {
+    if (!x || !w0 || !y || (swiglu && !w1)) return L3_ERR_NULL_POINTER;
+    if (M <= 0 || M > L3_LINEAR_MAX_ROWS || N <= 0 || K <= 0 || N % 4 != 0 || K % 32 != 0) return L3_ERR_SHAPE;
+    if (N > (1 << 24) || K > (1 << 24)) return L3_ERR_SHAPE;
+    if (x_stride < K || w_stride < K || y_stride < N || x_stride % 8 || w_stride % 8 || y_stride % 4)
+        return L3_ERR_STRIDE;
+    if (!aligned(x, 16) || !aligned(w0, 16) || (swiglu && !aligned(w1, 16)) || !aligned(y, 8))
+        return L3_ERR_ALIGNMENT;
+    LinearParams p;
+    p.x = static_cast<const uint16_t*>(x);
+    p.w0 = static_cast<const uint16_t*>(w0);
+    p.w1 = static_cast<const uint16_t*>(w1);
+    p.y = static_cast<uint16_t*>(y);
+    p.M = M; p.N = N; p.K = K;
+    p.x_stride = x_stride; p.w_stride = w_stride; p.y_stride = y_stride;
+    p.sk = 1;
+    return launch_linear_skinny(p, swiglu, current_device_cus(), static_cast<hipStream_t>(stream)) == 0 ? L3_OK
+                                                                                                        : L3_ERR_HIP;
+}
+
+}  // namespace
+
+int l3_linear_decode(const void* x, const void* w, void* y, int M, int N, int K, int64_t x_stride, int64_t w_stride,
+                     int64_t y_stride, void* stream) {
+    return linear_decode_impl(x, w, nullptr, y, M, N, K, x_stride, w_stride, y_stride, false, stream);
+}
+
+int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up, void* y, int M, int N, int K,
+                            int64_t x_stride, int64_t w_stride, int64_t y_stride, void* stream) {
+    return linear_decode_impl(x, w_gate, w_up, y, M, N, K, x_stride, w_stride, y_stride, true, stream);
+}
+
 size_t l3_argmax_workspace_bytes(int rows, int V) {
     if (rows <= 0 || V <= 0) return 0;
     return size_t(rows) * size_t(argmax_parts(V)) * (sizeof(float) + sizeof(int));

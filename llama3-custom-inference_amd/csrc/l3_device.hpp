@@ -101,6 +101,13 @@ __device__ __forceinline__ float wave_max(float x) {
 // 2^x through the hardware v_exp_f32 (inputs here are <= 0 or small; no denormal fix-up).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// bf16(silu(a)) as a float: torch's F.silu(a) * b materialises silu's bf16 result before the
+// multiplication (model.py:134), and so does every kernel here that fuses the product.
+__device__ __forceinline__ float silu_rounded(float a) {
+    const float s = a / (1.0f + expf(-a));
+    return __uint_as_float(f32_to_bf16_bits(s) << 16);
+}
+
 // 16-byte global load / store on element pointers.
 __device__ __forceinline__ uint4 load16(const uint16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ void store16(uint16_t* p, const uint4& v) { *reinterpret_cast<uint4*>(p) = v; }

@@ -71,7 +71,19 @@ struct PrefillParams {
     float scale_log2e;
 };
 
+struct LinearParams {
+    const uint16_t* x;    // (M, K) activations, row stride x_stride
+    const uint16_t* w0;   // (N, K) weights, row stride w_stride
+    const uint16_t* w1;   // second weight matrix of the SwiGLU form (else null)
+    uint16_t* y;          // (M, N), row stride y_stride
+    int M, N, K;
+    int64_t x_stride, w_stride, y_stride;
+    int sk;               // wavefronts that split K for one block of 16 weight rows (set by the launcher)
+};
+
 // Launchers: return a hipError_t cast to int (0 = success).
+int linear_skinny_plan(int N, int K, int waves_per_wg, int num_cus);
+int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream);
 int launch_attn_prefill(const PrefillParams& p, int HD, hipStream_t stream);        // a wavefront per column group
 constexpr int kPrefillTiledWaves = 8;      // wavefronts per workgroup of the tiled prefill kernel
 constexpr int kPrefillTiledColBlocks = 2;  // 16-column blocks per wavefront

@@ -20,6 +20,7 @@ L3_ERR_WORKSPACE = -7
 L3_ERR_SPLITS = -8
 L3_ERR_HIP = -9
 L3_ATTN_MAX_SPLITS = 512
+L3_LINEAR_MAX_ROWS = 64
 L3_ATTN_OPT_KERNEL = 0
 L3_ATTN_KERNEL_FMA = 0
 L3_ATTN_KERNEL_MFMA = 1
@@ -84,6 +85,16 @@ SIGNATURES = {
          ctypes.c_int, ctypes.c_float, ctypes.c_void_p],
     ),
     "l3_silu_mul": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
+    "l3_linear_decode": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p],
+    ),
+    "l3_linear_swiglu_decode": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p],
+    ),
     "l3_argmax_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "l3_argmax": (
         ctypes.c_int,

@@ -363,6 +363,53 @@ def silu_mul(a, b):
     return y
 
 
+def _linear_args(x, weights):
+    _require_gpu_bf16("x", x)
+    K = x.shape[-1]
+    rows = x.numel() // max(K, 1)
+    if x.dim() < 1 or rows < 1 or rows > _l3lib.L3_LINEAR_MAX_ROWS:
+        raise RuntimeError(f"linear_decode: 1..{_l3lib.L3_LINEAR_MAX_ROWS} activation rows expected, got "
+                           f"{tuple(x.shape)}")
+    for w in weights:
+        _require_gpu_bf16("weight", w)
+        if w.dim() != 2 or w.shape[1] != K or w.stride(1) != 1 or tuple(w.shape) != tuple(weights[0].shape) \
+                or w.stride(0) != weights[0].stride(0):
+            raise RuntimeError(f"linear_decode: weight {tuple(w.shape)} does not fit x {tuple(x.shape)}")
+    x2 = x.reshape(rows, K)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    return x2, rows, weights[0].shape[0], K
+
+
+def linear_decode(x, weight):
+    """F.linear(x, weight) for at most 64 activation rows (model.py:95,121,134,225 when T == 1):
+    one pass over the weight matrix at HBM speed instead of a GEMM.  x (..., K), weight (N, K)
+    -> (..., N).  An extension."""
+    lib = _l3lib.load()
+    x2, rows, N, K = _linear_args(x, (weight,))
+    y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.l3_linear_decode(x2.data_ptr(), weight.data_ptr(), y.data_ptr(), rows, N, K, x2.stride(0),
+                                  weight.stride(0), N, _stream_ptr(x.device))
+    if rc != 0:
+        _fail(rc, f"M={rows} N={N} K={K}")
+    return y.view(*x.shape[:-1], N)
+
+
+def linear_swiglu_decode(x, w_gate, w_up):
+    """F.silu(F.linear(x, w_gate)) * F.linear(x, w_up) for at most 64 activation rows in one
+    launch (model.py:134 with w_gate = c_fc2, w_up = c_fc), same rounding points.  An extension."""
+    lib = _l3lib.load()
+    x2, rows, N, K = _linear_args(x, (w_gate, w_up))
+    y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.l3_linear_swiglu_decode(x2.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(), y.data_ptr(), rows, N, K,
+                                         x2.stride(0), w_gate.stride(0), N, _stream_ptr(x.device))
+    if rc != 0:
+        _fail(rc, f"M={rows} N={N} K={K}")
+    return y.view(*x.shape[:-1], N)
+
+
 def argmax(logits):
     """Index of the first maximum along the last dimension of a 2-D bf16 tensor (rows, V), as
     int64 -- torch.argmax(logits.float(), dim=-1) for the greedy pick of model.py:371 (the float

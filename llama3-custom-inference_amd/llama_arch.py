@@ -16,7 +16,9 @@ the same tensor layouts and views -- without its checkpoint loading:
                                                        stop-token bookkeeping with one device-side .all()
                                                        (the reference iterates the tensor in Python, :380)
 
-GEMMs, SwiGLU, embedding and sampling stay stock PyTorch, as in the reference.  `ops` is the
+Embedding, sampling and every nn.Linear with more than a few activation rows stay stock PyTorch,
+as in the reference; the linears of the decode step (T == 1) use ops.linear_decode /
+ops.linear_swiglu_decode when the operator module has them.  `ops` is the
 module that provides the three operators: custom_kernels.custom_kernels_extension on the GPU,
 or any object with the same three functions (the CPU baseline passes torch restatements).
 """
@@ -92,13 +94,32 @@ class LlamaDecoder:
                                               scale_factor=c.rope_scale_factor, device=self.device)
         self.prefill_backend = "unset"
         self._graphs = {}
+        # nn.Linear calls with at most this many activation rows (the decode step) go through the
+        # library's weight-streaming kernels when the operator module has them; 0 = always F.linear
+        self.decode_linear_rows = 16 if hasattr(ops, "linear_decode") else 0
+
+    def set_decode_linear_rows(self, rows: int):
+        self.decode_linear_rows = rows if hasattr(self.ops, "linear_decode") else 0
+        self._graphs.clear()   # recorded decode steps contain the previous choice
+
+    def _linear(self, x, w):
+        """x @ w.T (nn.Linear without bias: model.py:95,121,134,225)."""
+        if 0 < x.numel() // x.shape[-1] <= self.decode_linear_rows:
+            return self.ops.linear_decode(x, w)
+        return F.linear(x, w)
+
+    def _mlp(self, L, h):
+        """c_proj(silu(c_fc2(h)) * c_fc(h)) (model.py:134)."""
+        if 0 < h.numel() // h.shape[-1] <= self.decode_linear_rows:
+            return self.ops.linear_decode(self.ops.linear_swiglu_decode(h, L["c_fc2"], L["c_fc"]), L["mlp_proj"])
+        return F.linear(F.silu(F.linear(h, L["c_fc2"])) * F.linear(h, L["c_fc"]), L["mlp_proj"])
 
     # ------------------------------------------------------------------ attention block
     def _attention(self, L, x, freqs_cis, start_pos):
         c = self.config
         B, T, C = x.shape
         hd = self.hd
-        qkv = F.linear(x, L["c_attn"])
+        qkv = self._linear(x, L["c_attn"])
         q, k, v = qkv.split([c.n_head * hd, c.n_kv_head * hd, c.n_kv_head * hd], dim=-1)
         q, k, v = (t.view(B, T, -1, hd) for t in (q, k, v))        # strided views into qkv
         q = self.ops.rot_embed(q, freqs_cis)
@@ -113,7 +134,7 @@ class LlamaDecoder:
         else:
             y = self.ops.flash_attention_decode(q, k, v)
         y = y.transpose(1, 2).contiguous().view(B, T, C)
-        return F.linear(y, L["c_proj"])
+        return self._linear(y, L["c_proj"])
 
     def _prefill_attention(self, q, k, v):
         """Causal GQA attention for T > 1.  The reference hands this case to torch
@@ -136,9 +157,9 @@ class LlamaDecoder:
         for L in self.layers:
             x = x + self._attention(L, self.ops.rms_norm(x, L["ln_1"], c.norm_eps), freqs_cis, start_pos)
             h = self.ops.rms_norm(x, L["ln_2"], c.norm_eps)
-            x = x + F.linear(F.silu(F.linear(h, L["c_fc2"])) * F.linear(h, L["c_fc"]), L["mlp_proj"])
+            x = x + self._mlp(L, h)
         x = self.ops.rms_norm(x, self.ln_f, c.norm_eps)
-        return F.linear(x[:, [-1], :], self.wte).float()
+        return self._linear(x[:, [-1], :], self.wte).float()
 
     # ------------------------------------------------------------------------- generate
     @torch.inference_mode()
@@ -267,17 +288,20 @@ class GraphedDecodeLoop:
         x = F.embedding(self.tok, m.wte)
         h = ops.rms_norm(x, m.layers[0]["ln_1"], c.norm_eps)
         for i, L in enumerate(m.layers):
-            qkv = F.linear(h, L["c_attn"])
+            qkv = m._linear(h, L["c_attn"])
             q = ops.rot_embed_append(qkv, m.freqs_cis, L["cache_k"], L["cache_v"], self.pos, c.n_head)
             y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
                                                   L["cache_v"][:B].transpose(1, 2), self.kv_len)
             # residual add fused with the norm that follows it (same bits as add, then rms_norm)
-            x, h = ops.add_rms_norm(x, F.linear(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"]),
+            x, h = ops.add_rms_norm(x, m._linear(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"]),
                                     L["ln_2"], c.norm_eps)
-            mlp = F.linear(ops.silu_mul(F.linear(h, L["c_fc2"]), F.linear(h, L["c_fc"])), L["mlp_proj"])
+            if 0 < B <= m.decode_linear_rows:
+                mlp = m._mlp(L, h)
+            else:
+                mlp = F.linear(ops.silu_mul(F.linear(h, L["c_fc2"]), F.linear(h, L["c_fc"])), L["mlp_proj"])
             next_norm = m.layers[i + 1]["ln_1"] if i + 1 < len(m.layers) else m.ln_f
             x, h = ops.add_rms_norm(x, mlp, next_norm, c.norm_eps)
-        nxt = ops.argmax(F.linear(h[:, -1], m.wte))   # first maximum of the bf16 logits = argmax of their float copy
+        nxt = ops.argmax(m._linear(h[:, -1], m.wte))   # first maximum of the bf16 logits = argmax of their float copy
         # generate() bookkeeping (model.py:373-378) at position pos + 1, all on the device
         cur = (self.pos + 1).long().clamp_(max=self.total_len - 1)
         keep = self.text_mask.index_select(1, cur).squeeze(1)
@@ -358,6 +382,15 @@ def bench_e2e(args, torch_mod, dev):
         cfg = LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=batch)
         model = LlamaDecoder(cfg, cke, dev)
         rec = {}
+        # stock F.linear (hipBLASLt) in the decode step first, for the comparison ...
+        model.set_decode_linear_rows(0)
+        timed_generate(model, batch, input_len, gen_len, seed=1, graphed=True)
+        best = max(timed_generate(model, batch, input_len, gen_len, sync=torch_mod.cuda.synchronize, graphed=True)[0]
+                   for _ in range(3))
+        rec["graphed_torch_linear"] = {"tok_per_s": round(best, 1)}
+        # ... then the library's weight-streaming linear kernels where they apply (up to 16 rows)
+        model.set_decode_linear_rows(16)
+        rec["decode_linear"] = "l3_linear_decode" if 0 < batch <= model.decode_linear_rows else "torch F.linear"
         for mode in ("eager", "graphed"):
             graphed = mode == "graphed"
             # warm-up generate, as llama3_inference.py:31-36 does (for the graphed loop it also records the graph)

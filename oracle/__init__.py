@@ -18,6 +18,7 @@ What is restated, and from where (paths relative to the reference checkout):
 * RMSNorm               custom_kernels/custom_kernels.cu:341-366 (formula), with
                         a single final rounding instead of the bf16 multiplies.
 * rotary embedding      custom_kernels/custom_kernels.cu:400-414.
+* decode-step linear    model.py:95,121,134,225 (nn.Linear without bias; SwiGLU front half).
 * frequency table       model.py:27-60.
 
 Pinning status (every function below is pinned; none is "parity unpinned"):
@@ -37,6 +38,8 @@ from .ops_ref import (  # noqa: F401
     attention_decode_ref,
     attention_prefill_ref,
     attention_split_partials_ref,
+    linear_ref,
+    swiglu_linear_ref,
     lse_combine_ref,
     precompute_freqs_cis_ref,
     llama3_scaled_inv_freq_ref,

@@ -122,6 +122,24 @@ def rms_norm_ref(x, w, eps) -> np.ndarray:
     return x / np.sqrt(ms + float(eps)) * w
 
 
+# ------------------------------------------------------------------------------ linear
+def linear_ref(x, w) -> np.ndarray:
+    """y = x . w^T in float64: x (..., K), w (N, K) -> (..., N).  What nn.Linear without bias
+    computes (model.py:95,121,134,225)."""
+    return np.asarray(x, dtype=np.float64) @ np.asarray(w, dtype=np.float64).T
+
+
+def swiglu_linear_ref(x, w_gate, w_up) -> np.ndarray:
+    """bf16(silu(g)) * u with g = bf16(x . w_gate^T), u = bf16(x . w_up^T): the front half of the
+    MLP (model.py:134, F.silu(c_fc2(x)) * c_fc(x)) with the roundings of its three bf16 torch
+    operators; the final product is left unrounded for the caller."""
+    from .bf16 import round_to_bf16
+    g = round_to_bf16(linear_ref(x, w_gate)).astype(np.float64)
+    u = round_to_bf16(linear_ref(x, w_up)).astype(np.float64)
+    s = round_to_bf16(g / (1.0 + np.exp(-g))).astype(np.float64)
+    return s * u
+
+
 # -------------------------------------------------------------------------------- RoPE
 def rot_embed_ref(x, freq) -> np.ndarray:
     """Rotate adjacent pairs: x (B, T, NH, HD), freq (T, HD) = [cos0, sin0, cos1, sin1, ...].

@@ -167,3 +167,25 @@ def test_prefill_argument_checks():
     assert call(q=FAKE + 8) == _l3lib.L3_ERR_ALIGNMENT
     assert call(q_strides=_l3lib.i64_array((131072, 64, 2052))) == _l3lib.L3_ERR_STRIDE
     assert call(k_strides=_l3lib.i64_array((131072, -64, 512))) == _l3lib.L3_ERR_STRIDE
+
+
+def test_linear_decode_argument_checks():
+    lib = _l3lib.load()
+
+    def call(x=FAKE, w=FAKE, y=FAKE, M=1, N=2048, K=2048, xs=2048, ws=2048, ys=2048):
+        return lib.l3_linear_decode(x, w, y, M, N, K, xs, ws, ys, None)
+
+    assert call(w=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert call(M=0) == _l3lib.L3_ERR_SHAPE
+    assert call(M=_l3lib.L3_LINEAR_MAX_ROWS + 1) == _l3lib.L3_ERR_SHAPE
+    assert call(K=2040, xs=2040, ws=2040) == _l3lib.L3_ERR_SHAPE       # K not a multiple of 32
+    assert call(N=2046, ys=2048) == _l3lib.L3_ERR_SHAPE                # N not a multiple of 4
+    assert call(xs=1024) == _l3lib.L3_ERR_STRIDE                       # rows would overlap
+    assert call(ws=2052) == _l3lib.L3_ERR_STRIDE                       # weight rows not 16-byte aligned
+    assert call(ys=2046) == _l3lib.L3_ERR_STRIDE
+    assert call(x=FAKE + 8) == _l3lib.L3_ERR_ALIGNMENT
+    assert call(y=FAKE + 4) == _l3lib.L3_ERR_ALIGNMENT
+    assert lib.l3_linear_swiglu_decode(FAKE, FAKE, None, FAKE, 1, 8192, 2048, 2048, 2048, 8192, None) \
+        == _l3lib.L3_ERR_NULL_POINTER
+    assert lib.l3_linear_swiglu_decode(FAKE, FAKE, FAKE + 2, FAKE, 1, 8192, 2048, 2048, 2048, 8192, None) \
+        == _l3lib.L3_ERR_ALIGNMENT

@@ -1,0 +1,96 @@
+"""GPU parity: the decode-step linear kernels (through the C ABI) against the float64 oracle."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import bf16_ulp_distance, randn_bf16, t2bits, t2f32
+from oracle import linear_ref, swiglu_linear_ref
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_linear_close(y, ref, what):
+    """Within 1 bf16 ulp of the float64 result, except where the sum cancels to (nearly) nothing:
+    there the float32 accumulation error, about 2^-24 per term relative to the LARGEST partial
+    sum, can exceed the tiny result's own ulp, so an absolute 2^-18 of the row's largest |y| also
+    passes."""
+    ref = np.asarray(ref, dtype=np.float64)
+    got = t2f32(y).astype(np.float64)
+    d = bf16_ulp_distance(t2bits(y), t2bits(torch.from_numpy(ref.astype(np.float32)).to(torch.bfloat16)))
+    slack = 2.0 ** -18 * np.abs(ref).max(axis=-1, keepdims=True)
+    bad = (d > 1) & (np.abs(got - ref) > slack)
+    assert not bad.any(), f"{what}: {bad.sum()} elements off by more than 1 ulp and the cancellation slack; " \
+                          f"max distance {d.max()} ulp"
+
+# (M, N, K): the 1B-architecture decode shapes (qkv, out projection, MLP down projection, lm head),
+# batch sizes up to 64, and shapes off every multiple the kernel tiles by
+SHAPES = [(1, 3072, 2048), (1, 2048, 2048), (1, 2048, 8192), (1, 128256, 2048), (3, 1024, 512), (16, 3072, 2048),
+          (17, 512, 256), (64, 3072, 2048), (64, 2048, 8192), (5, 20, 32), (2, 36, 64), (33, 100, 96),
+          (64, 16, 4096), (1, 16, 32), (8, 6144, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_linear_decode_against_oracle(gpu, M, N, K):
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"linear_decode M={M} N={N} K={K}", flush=True)
+    x = randn_bf16((M, K), 11)
+    w = randn_bf16((N, K), 12, scale=0.05)
+    y = cke.linear_decode(x.to(gpu), w.to(gpu))
+    torch.cuda.synchronize()
+    assert y.shape == (M, N) and y.dtype == torch.bfloat16
+    assert_linear_close(y, linear_ref(t2f32(x), t2f32(w)), f"linear {M}x{N}x{K}")
+
+
+def test_linear_decode_layouts_and_errors(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    M, N, K = 4, 256, 512
+    w = randn_bf16((N, K), 21, scale=0.05).to(gpu)
+    buf = randn_bf16((M, 1, K + 64), 22).to(gpu)
+    x = buf[..., :K]                                   # (M, 1, K) rows with a padded stride
+    y = cke.linear_decode(x, w)
+    assert y.shape == (M, 1, N)
+    dense = cke.linear_decode(x.contiguous(), w)
+    assert torch.equal(y, dense)
+    wide = randn_bf16((N, K + 32), 23, scale=0.05).to(gpu)
+    ys = cke.linear_decode(x, wide[:, :K])             # weight rows with a padded stride
+    assert_linear_close(ys, linear_ref(t2f32(x), t2f32(wide[:, :K])), "strided weight")
+    # the rows of a batch do not influence each other: row 2 alone gives the same bits
+    assert torch.equal(cke.linear_decode(x[2:3], w), y[2:3])
+    with pytest.raises(RuntimeError):
+        cke.linear_decode(randn_bf16((65, K), 1).to(gpu), w)          # too many rows for this entry point
+    with pytest.raises(RuntimeError):
+        cke.linear_decode(randn_bf16((2, 48), 1).to(gpu), randn_bf16((8, 48), 2).to(gpu))   # K % 32 != 0
+    with pytest.raises(RuntimeError):
+        cke.linear_decode(randn_bf16((2, K + 32), 1).to(gpu), w)      # K mismatch
+    with pytest.raises(RuntimeError):
+        cke.linear_decode(randn_bf16((2, K), 1), w)                   # CPU tensor
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 8192, 2048), (64, 8192, 2048), (7, 1024, 256), (16, 14336, 4096), (40, 52, 64)])
+def test_linear_swiglu_decode(gpu, M, N, K):
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"linear_swiglu_decode M={M} N={N} K={K}", flush=True)
+    x = randn_bf16((M, K), 31)
+    wg = randn_bf16((N, K), 32, scale=0.05)
+    wu = randn_bf16((N, K), 33, scale=0.05)
+    xd, wgd, wud = x.to(gpu), wg.to(gpu), wu.to(gpu)
+    y = cke.linear_swiglu_decode(xd, wgd, wud)
+    torch.cuda.synchronize()
+    assert y.shape == (M, N)
+    # the fused kernel accumulates in the same order as the plain one: the three-operator sequence
+    # gives the same bits
+    seq = cke.silu_mul(cke.linear_decode(xd, wgd), cke.linear_decode(xd, wud))
+    assert torch.equal(y, seq)
+    # against exact arithmetic with the same rounding points: a gate or up value that rounds the other
+    # way moves the product by about one ulp of that factor
+    ref = swiglu_linear_ref(t2f32(x), t2f32(wg), t2f32(wu))
+    d = bf16_ulp_distance(t2bits(y), t2bits(torch.from_numpy(ref.astype(np.float32)).to(torch.bfloat16)))
+    assert (d > 2).mean() < 2e-3 and np.abs(t2f32(y) - ref).max() <= 0.02 * max(1.0, np.abs(ref).max())
+    # and torch's own three operators on the same device
+    lib = F.silu(F.linear(xd, wgd)) * F.linear(xd, wud)
+    assert (y.float() - lib.float()).abs().max().item() <= 0.02 * max(1.0, lib.float().abs().max().item())
