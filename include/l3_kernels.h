@@ -222,6 +222,21 @@ int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up,
                             int64_t x_stride, int64_t w_stride, int64_t y_stride, void* stream);
 
 /*
+ * l3_linear_decode with what a transformer block does around its linears folded in; each of
+ * norm_weight, w_up and residual may be NULL:
+ *   h = norm_weight ? bf16(x * rsqrt(mean(x^2) + norm_eps) * norm_weight) : x     (model.py:70-72 in front of
+ *                                                                                 c_attn / the MLP / lm_head)
+ *   t = w_up ? bf16(silu(bf16(h.w^T))) * bf16(h.w_up^T) : h.w^T                   (model.py:134)
+ *   y = residual ? bf16(residual + bf16(t)) : bf16(t)                             (model.py:147-148)
+ * with the rounding points of the separate operators.  residual has y's shape and row stride and
+ * may be y itself.  The input norm stages x in LDS and needs M <= 16, K % 512 == 0 and M * (K + 8) <= 24576
+ * (L3_ERR_SHAPE otherwise); everything else as for l3_linear_decode.
+ */
+int l3_linear_decode_fused(const void* x, const void* norm_weight, float norm_eps, const void* w, const void* w_up,
+                           const void* residual, void* y, int M, int N, int K, int64_t x_stride, int64_t w_stride,
+                           int64_t y_stride, void* stream);
+
+/*
  * out[r] = index of the first maximum of the bf16 row logits[r*row_stride : r*row_stride + V]
  * (int64, like torch.argmax; a row of NaNs gives 0): the greedy pick of model.py:371.  Two small
  * launches (per-chunk maxima into the caller's workspace of l3_argmax_workspace_bytes(rows, V)

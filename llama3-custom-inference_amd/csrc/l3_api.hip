@@ -391,19 +391,25 @@ int l3_silu_mul(const void* a, const void* b, void* y, int64_t n, void* stream) 
 
 namespace {
 
-int linear_decode_impl(const void* x, const void* w0, const void* w1, void* y, int M, int N, int K, int64_t x_stride,
-                       int64_t w_stride, int64_t y_stride, bool swiglu, void* stream) {
+int linear_decode_impl(const void* x, const void* norm_w, float norm_eps, const void* w0, const void* w1,
+                       const void* res, void* y, int M, int N, int K, int64_t x_stride, int64_t w_stride,
+                       int64_t y_stride, bool swiglu, void* stream) {
     if (!x || !w0 || !y || (swiglu && !w1)) return L3_ERR_NULL_POINTER;
     if (M <= 0 || M > L3_LINEAR_MAX_ROWS || N <= 0 || K <= 0 || N % 4 != 0 || K % 32 != 0) return L3_ERR_SHAPE;
     if (N > (1 << 24) || K > (1 << 24)) return L3_ERR_SHAPE;
+    if (norm_w && !linear_skinny_can_stage(M, K)) return L3_ERR_SHAPE;
     if (x_stride < K || w_stride < K || y_stride < N || x_stride % 8 || w_stride % 8 || y_stride % 4)
         return L3_ERR_STRIDE;
-    if (!aligned(x, 16) || !aligned(w0, 16) || (swiglu && !aligned(w1, 16)) || !aligned(y, 8))
+    if (!aligned(x, 16) || !aligned(w0, 16) || (swiglu && !aligned(w1, 16)) || !aligned(y, 8) ||
+        (norm_w && !aligned(norm_w, 16)) || (res && !aligned(res, 8)))
         return L3_ERR_ALIGNMENT;
     LinearParams p;
     p.x = static_cast<const uint16_t*>(x);
     p.w0 = static_cast<const uint16_t*>(w0);
     p.w1 = static_cast<const uint16_t*>(w1);
+    p.norm_w = static_cast<const uint16_t*>(norm_w);
+    p.res = static_cast<const uint16_t*>(res);
+    p.norm_eps = norm_eps;
     p.y = static_cast<uint16_t*>(y);
     p.M = M; p.N = N; p.K = K;
     p.x_stride = x_stride; p.w_stride = w_stride; p.y_stride = y_stride;
@@ -416,12 +422,21 @@ int linear_decode_impl(const void* x, const void* w0, const void* w1, void* y, i
 
 int l3_linear_decode(const void* x, const void* w, void* y, int M, int N, int K, int64_t x_stride, int64_t w_stride,
                      int64_t y_stride, void* stream) {
-    return linear_decode_impl(x, w, nullptr, y, M, N, K, x_stride, w_stride, y_stride, false, stream);
+    return linear_decode_impl(x, nullptr, 0.f, w, nullptr, nullptr, y, M, N, K, x_stride, w_stride, y_stride, false,
+                              stream);
 }
 
 int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up, void* y, int M, int N, int K,
                             int64_t x_stride, int64_t w_stride, int64_t y_stride, void* stream) {
-    return linear_decode_impl(x, w_gate, w_up, y, M, N, K, x_stride, w_stride, y_stride, true, stream);
+    return linear_decode_impl(x, nullptr, 0.f, w_gate, w_up, nullptr, y, M, N, K, x_stride, w_stride, y_stride, true,
+                              stream);
+}
+
+int l3_linear_decode_fused(const void* x, const void* norm_weight, float norm_eps, const void* w, const void* w_up,
+                           const void* residual, void* y, int M, int N, int K, int64_t x_stride, int64_t w_stride,
+                           int64_t y_stride, void* stream) {
+    return linear_decode_impl(x, norm_weight, norm_eps, w, w_up, residual, y, M, N, K, x_stride, w_stride, y_stride,
+                              w_up != nullptr, stream);
 }
 
 size_t l3_argmax_workspace_bytes(int rows, int V) {

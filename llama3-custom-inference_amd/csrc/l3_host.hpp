@@ -75,6 +75,9 @@ struct LinearParams {
     const uint16_t* x;    // (M, K) activations, row stride x_stride
     const uint16_t* w0;   // (N, K) weights, row stride w_stride
     const uint16_t* w1;   // second weight matrix of the SwiGLU form (else null)
+    const uint16_t* norm_w;  // (K) RMSNorm weight applied to x first (else null)
+    const uint16_t* res;     // (M, N) residual added to the product, y's row stride (else null)
+    float norm_eps;
     uint16_t* y;          // (M, N), row stride y_stride
     int M, N, K;
     int64_t x_stride, w_stride, y_stride;
@@ -83,6 +86,7 @@ struct LinearParams {
 
 // Launchers: return a hipError_t cast to int (0 = success).
 int linear_skinny_plan(int N, int K, int waves_per_wg, int num_cus);
+bool linear_skinny_can_stage(int M, int K);
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream);
 int launch_attn_prefill(const PrefillParams& p, int HD, hipStream_t stream);        // a wavefront per column group
 constexpr int kPrefillTiledWaves = 8;      // wavefronts per workgroup of the tiled prefill kernel

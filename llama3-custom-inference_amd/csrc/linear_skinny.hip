@@ -7,20 +7,33 @@
 //
 // A lane of the A operand holds 8 consecutive k of one weight row, which is exactly a 16-byte
 // global load: weights go from HBM into operand registers with no staging.  A wavefront owns 16
-// weight rows over a slice of K; the `sk` wavefronts that share a row block meet in LDS.  With
-// SWIGLU the wavefront streams the same rows of two matrices and writes
-// bf16(silu(x.Wg^T)) * bf16(x.Wu^T) with torch's rounding points (model.py:134).
+// weight rows over a slice of K; the `sk` wavefronts that share a row block meet in LDS.
+//
+// What a transformer block does around its linears rides along (each optional):
+//   * RMSNorm of the input (model.py:147-148, ln_1 / ln_2 in front of c_attn / the MLP): with at
+//     most 16 activation rows the workgroup first writes the normalised x into LDS, with the
+//     rounding of the stand-alone operator (bf16(x * inv_rms * w)), and the B operands come
+//     from there;
+//   * SwiGLU: the wavefront streams the same rows of two matrices and writes
+//     bf16(silu(x.Wg^T)) * bf16(x.Wu^T) with torch's rounding points (model.py:134);
+//   * the residual addition that follows c_proj and the MLP (model.py:147-148):
+//     y = bf16(residual + bf16(x.W^T)), the two roundings of the separate operators.
 #include "attn_mfma_core.hpp"
 
 namespace l3 {
 
 namespace {
 
-template <int NW, int CBLK, int U, bool SWIGLU>
+// Elements of LDS the staged activations may take (rows are padded by 8 elements).
+constexpr int kXldsMaxElems = 24576;
+
+template <int NW, int CBLK, int U, bool SWIGLU, bool XLDS>
 __global__ void __launch_bounds__(NW * kWaveSize)
 linear_skinny_kernel(const LinearParams p) {
+    static_assert(!XLDS || CBLK == 1, "activations are staged in LDS only for up to 16 rows");
     constexpr int ACC = SWIGLU ? 2 : 1;
     __shared__ float s_red[NW][ACC][CBLK][256];
+    extern __shared__ __align__(16) uint16_t s_x[];        // XLDS: M rows of K + 8 elements
 
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int wave = threadIdx.x / kWaveSize;
@@ -56,26 +69,95 @@ linear_skinny_kernel(const LinearParams p) {
 
     // A ring of U k steps in registers: a slot is refilled for step ks + U as soon as the matrix
     // instructions of step ks have read it, so about U loads per operand stay in flight.
-    uint4 rw0[U], rw1[SWIGLU ? U : 1], rx[CBLK][U];
+    uint4 rw0[U], rw1[SWIGLU ? U : 1], rx[XLDS ? 1 : CBLK][XLDS ? 1 : U];
     auto fill = [&](int u, int ks) {
         rw0[u] = load16(wp0 + ks * 32);
         if constexpr (SWIGLU) rw1[u] = load16(wp1 + ks * 32);
+        if constexpr (!XLDS) {
 #pragma unroll
-        for (int cb = 0; cb < CBLK; ++cb) {
-            rx[cb][u] = xvalid[cb] ? load16(xp[cb] + ks * 32) : make_uint4(0u, 0u, 0u, 0u);
+            for (int cb = 0; cb < CBLK; ++cb) {
+                rx[cb][u] = xvalid[cb] ? load16(xp[cb] + ks * 32) : make_uint4(0u, 0u, 0u, 0u);
+            }
         }
     };
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         if (ks0 + u < ks1) fill(u, ks0 + u);
     }
+
+    const int KP = p.K + 8;                                // LDS row pitch in elements
+    if constexpr (XLDS) {
+        // RMSNorm of the activations into LDS while the first weight loads are in flight.  The
+        // workgroup shares the 16-byte chunks of all rows; K % 512 == 0, so the 64 chunks of a
+        // wavefront lie in one row and the row's sum of squares is a fixed-order sum of
+        // per-wavefront parts.
+        constexpr int NT = NW * kWaveSize;
+        constexpr int MAXC = (kXldsMaxElems / 8 + NT - 1) / NT;
+        __shared__ float s_part[kXldsMaxElems / 8 / kWaveSize];
+        const int cpr = p.K / 8;                           // chunks per row
+        const int nchunks = p.M * cpr;
+        const int parts_per_row = cpr / kWaveSize;
+        uint4 xv[MAXC], gv[MAXC];
+#pragma unroll
+        for (int j = 0; j < MAXC; ++j) {
+            const int c = int(threadIdx.x) + j * NT;
+            if (c < nchunks) {                             // wave-uniform
+                const int r = c / cpr, col = c % cpr;
+                xv[j] = load16(p.x + int64_t(r) * p.x_stride + col * 8);
+                gv[j] = load16(p.norm_w + col * 8);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < MAXC; ++j) {
+            const int c = int(threadIdx.x) + j * NT;
+            if (c < nchunks) {
+                float f[8];
+                unpack8(xv[j], f);
+                float ss = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+                ss = wave_sum(ss);
+                if (lane == 0) s_part[c / kWaveSize] = ss;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < MAXC; ++j) {
+            const int c = int(threadIdx.x) + j * NT;
+            if (c < nchunks) {
+                const int r = c / cpr, col = c % cpr;
+                float ss = 0.f;
+                for (int q = 0; q < parts_per_row; ++q) ss += s_part[r * parts_per_row + q];
+                const float inv = rsqrtf(ss / float(p.K) + p.norm_eps);
+                float f[8], g[8];
+                unpack8(xv[j], f);
+                unpack8(gv[j], g);
+                uint4 o;
+                o.x = pack_bf16x2(f[0] * inv * g[0], f[1] * inv * g[1]);
+                o.y = pack_bf16x2(f[2] * inv * g[2], f[3] * inv * g[3]);
+                o.z = pack_bf16x2(f[4] * inv * g[4], f[5] * inv * g[5]);
+                o.w = pack_bf16x2(f[6] * inv * g[6], f[7] * inv * g[7]);
+                *reinterpret_cast<uint4*>(s_x + r * KP + col * 8) = o;
+            }
+        }
+        __syncthreads();
+    }
+    const uint16_t* lx = s_x + (xvalid[0] ? fn : 0) * KP + fg * 8;
+
     for (int ks = ks0; ks < ks1; ks += U) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (ks + u < ks1) {                            // wave-uniform
 #pragma unroll
                 for (int cb = 0; cb < CBLK; ++cb) {
-                    const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, rx[cb][u]);
+                    uint4 xv;
+                    if constexpr (XLDS) {
+                        xv = *reinterpret_cast<const uint4*>(lx + (ks + u) * 32);
+                        if (!xvalid[0]) xv = make_uint4(0u, 0u, 0u, 0u);
+                    } else {
+                        xv = rx[cb][u];
+                    }
+                    const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, xv);
                     acc[0][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, rw0[u]), xf,
                                                                          acc[0][cb], 0, 0, 0);
                     if constexpr (SWIGLU) {
@@ -132,6 +214,13 @@ linear_skinny_kernel(const LinearParams p) {
                 o[r] = acc[0][cb][r];
             }
         }
+        if (p.res) {   // bf16(residual + bf16(product)), as the separate addition would give
+            const uint2 rv = *reinterpret_cast<const uint2*>(p.res + int64_t(m) * p.y_stride + n);
+            o[0] = bf16lo_to_f32(rv.x) + __uint_as_float(f32_to_bf16_bits(o[0]) << 16);
+            o[1] = bf16hi_to_f32(rv.x) + __uint_as_float(f32_to_bf16_bits(o[1]) << 16);
+            o[2] = bf16lo_to_f32(rv.y) + __uint_as_float(f32_to_bf16_bits(o[2]) << 16);
+            o[3] = bf16hi_to_f32(rv.y) + __uint_as_float(f32_to_bf16_bits(o[3]) << 16);
+        }
         uint2 w;
         w.x = pack_bf16x2(o[0], o[1]);
         w.y = pack_bf16x2(o[2], o[3]);
@@ -139,12 +228,13 @@ linear_skinny_kernel(const LinearParams p) {
     }
 }
 
-template <int NW, int CBLK, int U, bool SWIGLU>
+template <int NW, int CBLK, int U, bool SWIGLU, bool XLDS>
 int launch_variant(const LinearParams& p, hipStream_t stream) {
     const int row_blocks = (p.N + 15) / 16;
     const int rb_per_wg = NW / p.sk;
     const dim3 grid(unsigned((row_blocks + rb_per_wg - 1) / rb_per_wg));
-    hipLaunchKernelGGL((linear_skinny_kernel<NW, CBLK, U, SWIGLU>), grid, dim3(NW * kWaveSize), 0, stream, p);
+    const size_t lds = XLDS ? size_t(p.M) * size_t(p.K + 8) * sizeof(uint16_t) : 0;
+    hipLaunchKernelGGL((linear_skinny_kernel<NW, CBLK, U, SWIGLU, XLDS>), grid, dim3(NW * kWaveSize), lds, stream, p);
     return int(hipGetLastError());
 }
 
@@ -163,17 +253,29 @@ int linear_skinny_plan(int N, int K, int waves_per_wg, int num_cus) {
     return sk;
 }
 
+// The input RMSNorm needs the activations staged in LDS: at most 16 rows that fit there, of a
+// width that lets every wavefront of the staging pass stay within one row.
+bool linear_skinny_can_stage(int M, int K) {
+    return M <= 16 && K % 512 == 0 && int64_t(M) * (K + 8) <= kXldsMaxElems;
+}
+
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream) {
     const bool wide = p.M > 16;
+    const bool stage = p.norm_w != nullptr;   // the caller has checked linear_skinny_can_stage
     // few row blocks and a long K (the MLP's down projection): sixteen wavefronts share a row block
     const int row_blocks = (p.N + 15) / 16;
     const bool big_wg = !wide && !swiglu && row_blocks < num_cus && p.K / 32 >= 128;
     p.sk = linear_skinny_plan(p.N, p.K, big_wg ? 16 : 8, num_cus);
     if (swiglu) {
-        return wide ? launch_variant<8, 4, 4, true>(p, stream) : launch_variant<8, 1, 8, true>(p, stream);
+        if (wide) return launch_variant<8, 4, 4, true, false>(p, stream);
+        return stage ? launch_variant<8, 1, 8, true, true>(p, stream) : launch_variant<8, 1, 8, true, false>(p, stream);
     }
-    if (wide) return launch_variant<8, 4, 8, false>(p, stream);
-    return big_wg ? launch_variant<16, 1, 8, false>(p, stream) : launch_variant<8, 1, 16, false>(p, stream);
+    if (wide) return launch_variant<8, 4, 8, false, false>(p, stream);
+    if (big_wg) {
+        return stage ? launch_variant<16, 1, 8, false, true>(p, stream)
+                     : launch_variant<16, 1, 8, false, false>(p, stream);
+    }
+    return stage ? launch_variant<8, 1, 16, false, true>(p, stream) : launch_variant<8, 1, 16, false, false>(p, stream);
 }
 
 }  // namespace l3

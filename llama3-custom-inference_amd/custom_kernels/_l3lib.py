@@ -21,6 +21,7 @@ L3_ERR_SPLITS = -8
 L3_ERR_HIP = -9
 L3_ATTN_MAX_SPLITS = 512
 L3_LINEAR_MAX_ROWS = 64
+L3_LINEAR_STAGE_ELEMS = 24576   # activations (rows padded by 8) the fused input norm can stage in LDS
 L3_ATTN_OPT_KERNEL = 0
 L3_ATTN_KERNEL_FMA = 0
 L3_ATTN_KERNEL_MFMA = 1
@@ -94,6 +95,12 @@ SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
          ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p],
+    ),
+    "l3_linear_decode_fused": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+         ctypes.c_void_p],
     ),
     "l3_argmax_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "l3_argmax": (

@@ -410,6 +410,44 @@ def linear_swiglu_decode(x, w_gate, w_up):
     return y.view(*x.shape[:-1], N)
 
 
+def linear_decode_fused_max_rows(K: int) -> int:
+    """Most activation rows of width K for which linear_decode_fused accepts a norm_weight."""
+    return min(16, _l3lib.L3_LINEAR_STAGE_ELEMS // (K + 8)) if K % 512 == 0 else 0
+
+
+def linear_decode_fused(x, weight, norm_weight=None, eps: float = 1e-5, w_up=None, residual=None):
+    """linear_decode with the operators around it folded into the one launch, each optional:
+    rms_norm(x, norm_weight, eps) in front (model.py:70-72), the SwiGLU product with a second
+    matrix w_up (weight is then the gate, model.py:134), and `residual + result` behind
+    (model.py:147-148) -- all with the rounding points of the separate operators.  An extension."""
+    lib = _l3lib.load()
+    x2, rows, N, K = _linear_args(x, (weight,) if w_up is None else (weight, w_up))
+    if norm_weight is not None:
+        _require_gpu_bf16("norm_weight", norm_weight)
+        if tuple(norm_weight.shape) != (K,) or not norm_weight.is_contiguous():
+            raise RuntimeError(f"linear_decode_fused: norm_weight {tuple(norm_weight.shape)} does not fit K={K}")
+        if rows > linear_decode_fused_max_rows(K):
+            raise RuntimeError(f"linear_decode_fused: the input norm takes at most "
+                               f"{linear_decode_fused_max_rows(K)} rows of width {K}, got {rows}")
+    r2 = None
+    if residual is not None:
+        _require_gpu_bf16("residual", residual)
+        if residual.numel() != rows * N or residual.shape[-1] != N:
+            raise RuntimeError(f"linear_decode_fused: residual {tuple(residual.shape)} does not fit ({rows}, {N})")
+        r2 = residual.reshape(rows, N)
+        if not r2.is_contiguous():
+            r2 = r2.contiguous()
+    y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.l3_linear_decode_fused(x2.data_ptr(), None if norm_weight is None else norm_weight.data_ptr(),
+                                        float(eps), weight.data_ptr(), None if w_up is None else w_up.data_ptr(),
+                                        None if r2 is None else r2.data_ptr(), y.data_ptr(), rows, N, K,
+                                        x2.stride(0), weight.stride(0), N, _stream_ptr(x.device))
+    if rc != 0:
+        _fail(rc, f"M={rows} N={N} K={K}")
+    return y.view(*x.shape[:-1], N)
+
+
 def argmax(logits):
     """Index of the first maximum along the last dimension of a 2-D bf16 tensor (rows, V), as
     int64 -- torch.argmax(logits.float(), dim=-1) for the greedy pick of model.py:371 (the float

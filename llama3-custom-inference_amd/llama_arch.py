@@ -116,10 +116,14 @@ class LlamaDecoder:
 
     # ------------------------------------------------------------------ attention block
     def _attention(self, L, x, freqs_cis, start_pos):
+        y = self._attention_core(L, self._linear(x, L["c_attn"]), freqs_cis, start_pos)
+        return self._linear(y, L["c_proj"])
+
+    def _attention_core(self, L, qkv, freqs_cis, start_pos):
+        """From the fused qkv projection to the attention output (B, T, C), before c_proj."""
         c = self.config
-        B, T, C = x.shape
+        B, T = qkv.shape[:2]
         hd = self.hd
-        qkv = self._linear(x, L["c_attn"])
         q, k, v = qkv.split([c.n_head * hd, c.n_kv_head * hd, c.n_kv_head * hd], dim=-1)
         q, k, v = (t.view(B, T, -1, hd) for t in (q, k, v))        # strided views into qkv
         q = self.ops.rot_embed(q, freqs_cis)
@@ -133,8 +137,13 @@ class LlamaDecoder:
             y = self._prefill_attention(q, k, v)
         else:
             y = self.ops.flash_attention_decode(q, k, v)
-        y = y.transpose(1, 2).contiguous().view(B, T, C)
-        return self._linear(y, L["c_proj"])
+        return y.transpose(1, 2).contiguous().view(B, T, c.n_embd)
+
+    def _fused_rows(self) -> int:
+        """Rows up to which the decode step uses linear_decode_fused (norms and residual additions
+        folded into the linears); 0 when the operator module has no such operator."""
+        f = getattr(self.ops, "linear_decode_fused_max_rows", None)
+        return min(self.decode_linear_rows, f(self.config.n_embd)) if f else 0
 
     def _prefill_attention(self, q, k, v):
         """Causal GQA attention for T > 1.  The reference hands this case to torch
@@ -154,6 +163,15 @@ class LlamaDecoder:
         assert T <= c.block_size
         x = F.embedding(idx, self.wte)
         freqs_cis = self.freqs_cis[start_pos:start_pos + T]
+        if T == 1 and 0 < B <= self._fused_rows():
+            # decode step with the norms and residual additions folded into the linears
+            lin = self.ops.linear_decode_fused
+            for L in self.layers:
+                qkv = lin(x, L["c_attn"], norm_weight=L["ln_1"], eps=c.norm_eps)
+                x = lin(self._attention_core(L, qkv, freqs_cis, start_pos), L["c_proj"], residual=x)
+                t = lin(x, L["c_fc2"], norm_weight=L["ln_2"], eps=c.norm_eps, w_up=L["c_fc"])
+                x = lin(t, L["mlp_proj"], residual=x)
+            return lin(x, self.wte, norm_weight=self.ln_f, eps=c.norm_eps).float()
         for L in self.layers:
             x = x + self._attention(L, self.ops.rms_norm(x, L["ln_1"], c.norm_eps), freqs_cis, start_pos)
             h = self.ops.rms_norm(x, L["ln_2"], c.norm_eps)
@@ -286,22 +304,36 @@ class GraphedDecodeLoop:
         c, B = m.config, self.B
         ops = m.ops
         x = F.embedding(self.tok, m.wte)
-        h = ops.rms_norm(x, m.layers[0]["ln_1"], c.norm_eps)
-        for i, L in enumerate(m.layers):
-            qkv = m._linear(h, L["c_attn"])
-            q = ops.rot_embed_append(qkv, m.freqs_cis, L["cache_k"], L["cache_v"], self.pos, c.n_head)
-            y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
-                                                  L["cache_v"][:B].transpose(1, 2), self.kv_len)
-            # residual add fused with the norm that follows it (same bits as add, then rms_norm)
-            x, h = ops.add_rms_norm(x, m._linear(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"]),
-                                    L["ln_2"], c.norm_eps)
-            if 0 < B <= m.decode_linear_rows:
-                mlp = m._mlp(L, h)
-            else:
-                mlp = F.linear(ops.silu_mul(F.linear(h, L["c_fc2"]), F.linear(h, L["c_fc"])), L["mlp_proj"])
-            next_norm = m.layers[i + 1]["ln_1"] if i + 1 < len(m.layers) else m.ln_f
-            x, h = ops.add_rms_norm(x, mlp, next_norm, c.norm_eps)
-        nxt = ops.argmax(m._linear(h[:, -1], m.wte))   # first maximum of the bf16 logits = argmax of their float copy
+        if 0 < B <= m._fused_rows():
+            # five launches per layer: norms and residual additions ride with the linears
+            lin = ops.linear_decode_fused
+            for L in m.layers:
+                qkv = lin(x, L["c_attn"], norm_weight=L["ln_1"], eps=c.norm_eps)
+                q = ops.rot_embed_append(qkv, m.freqs_cis, L["cache_k"], L["cache_v"], self.pos, c.n_head)
+                y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
+                                                      L["cache_v"][:B].transpose(1, 2), self.kv_len)
+                x = lin(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"], residual=x)
+                t = lin(x, L["c_fc2"], norm_weight=L["ln_2"], eps=c.norm_eps, w_up=L["c_fc"])
+                x = lin(t, L["mlp_proj"], residual=x)
+            logits = lin(x[:, -1], m.wte, norm_weight=m.ln_f, eps=c.norm_eps)
+        else:
+            h = ops.rms_norm(x, m.layers[0]["ln_1"], c.norm_eps)
+            for i, L in enumerate(m.layers):
+                qkv = m._linear(h, L["c_attn"])
+                q = ops.rot_embed_append(qkv, m.freqs_cis, L["cache_k"], L["cache_v"], self.pos, c.n_head)
+                y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
+                                                      L["cache_v"][:B].transpose(1, 2), self.kv_len)
+                # residual add fused with the norm that follows it (same bits as add, then rms_norm)
+                x, h = ops.add_rms_norm(x, m._linear(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"]),
+                                        L["ln_2"], c.norm_eps)
+                if 0 < B <= m.decode_linear_rows:
+                    mlp = m._mlp(L, h)
+                else:
+                    mlp = F.linear(ops.silu_mul(F.linear(h, L["c_fc2"]), F.linear(h, L["c_fc"])), L["mlp_proj"])
+                next_norm = m.layers[i + 1]["ln_1"] if i + 1 < len(m.layers) else m.ln_f
+                x, h = ops.add_rms_norm(x, mlp, next_norm, c.norm_eps)
+            logits = m._linear(h[:, -1], m.wte)
+        nxt = ops.argmax(logits)   # first maximum of the bf16 logits = argmax of their float copy
         # generate() bookkeeping (model.py:373-378) at position pos + 1, all on the device
         cur = (self.pos + 1).long().clamp_(max=self.total_len - 1)
         keep = self.text_mask.index_select(1, cur).squeeze(1)

@@ -189,3 +189,15 @@ def test_linear_decode_argument_checks():
         == _l3lib.L3_ERR_NULL_POINTER
     assert lib.l3_linear_swiglu_decode(FAKE, FAKE, FAKE + 2, FAKE, 1, 8192, 2048, 2048, 2048, 8192, None) \
         == _l3lib.L3_ERR_ALIGNMENT
+
+
+def test_linear_decode_fused_argument_checks():
+    lib = _l3lib.load()
+
+    def call(norm=FAKE, res=FAKE, M=1, K=2048):
+        return lib.l3_linear_decode_fused(FAKE, norm, 1e-5, FAKE, None, res, FAKE, M, 2048, K, K, K, 2048, None)
+
+    assert call(M=12) == _l3lib.L3_ERR_SHAPE              # 12 rows of 2048 do not fit the LDS stage
+    assert call(M=3, K=8192) == _l3lib.L3_ERR_SHAPE
+    assert call(norm=FAKE + 2) == _l3lib.L3_ERR_ALIGNMENT
+    assert call(res=FAKE + 4) == _l3lib.L3_ERR_ALIGNMENT

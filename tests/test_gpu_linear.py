@@ -94,3 +94,71 @@ def test_linear_swiglu_decode(gpu, M, N, K):
     # and torch's own three operators on the same device
     lib = F.silu(F.linear(xd, wgd)) * F.linear(xd, wud)
     assert (y.float() - lib.float()).abs().max().item() <= 0.02 * max(1.0, lib.float().abs().max().item())
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 3072, 2048), (8, 3072, 2048), (11, 512, 2048), (1, 2048, 8192), (2, 128, 8192),
+                                   (16, 100, 512), (3, 128256, 2048), (5, 64, 1536), (5, 4096, 4096)])
+def test_linear_fused_input_norm(gpu, M, N, K):
+    from custom_kernels import custom_kernels_extension as cke
+    from oracle import rms_norm_ref, round_to_bf16
+
+    print(f"linear_decode_fused norm M={M} N={N} K={K}", flush=True)
+    x = randn_bf16((M, 1, K), 41, scale=2.0)
+    nw = randn_bf16((K,), 42, scale=0.1, mean=1.0)
+    w = randn_bf16((N, K), 43, scale=0.05)
+    xd, nwd, wd = x.to(gpu), nw.to(gpu), w.to(gpu)
+    y = cke.linear_decode_fused(xd, wd, norm_weight=nwd, eps=1e-5)
+    torch.cuda.synchronize()
+    assert y.shape == (M, 1, N)
+    # the two separate operators: the same bits except where the row's inverse rms differs in its
+    # last float32 bit (the two kernels add the squares in different orders)
+    seq = cke.linear_decode(cke.rms_norm(xd, nwd, 1e-5), wd)
+    d = bf16_ulp_distance(t2bits(y), t2bits(seq))
+    assert d.max() <= 1 and (d > 0).mean() < 0.02, f"fused norm vs sequence: max {d.max()} ulp, {(d > 0).mean():.3f} differ"
+    # exact arithmetic with the rounding point of the stand-alone norm
+    h = round_to_bf16(rms_norm_ref(t2f32(x), t2f32(nw), 1e-5))
+    ref = linear_ref(h, t2f32(w))
+    err = np.abs(t2f32(y).astype(np.float64) - ref)
+    assert err.max() <= 2.0 ** -6 * max(1.0, np.abs(ref).max()), f"fused norm vs oracle: max err {err.max()}"
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (1, 2048, 8192), (9, 2048, 8192), (16, 256, 512), (64, 2048, 8192)])
+def test_linear_fused_residual(gpu, M, N, K):
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"linear_decode_fused residual M={M} N={N} K={K}", flush=True)
+    x = randn_bf16((M, 1, K), 51).to(gpu)
+    w = randn_bf16((N, K), 52, scale=0.05).to(gpu)
+    r = randn_bf16((M, 1, N), 53, scale=3.0).to(gpu)
+    y = cke.linear_decode_fused(x, w, residual=r)
+    torch.cuda.synchronize()
+    assert torch.equal(y, r + cke.linear_decode(x, w))    # torch's bf16 add: float sum, one rounding
+
+
+def test_linear_fused_whole_mlp_and_limits(gpu):
+    """ln_2 -> SwiGLU -> down projection + residual as the decode step chains them, against the
+    separate operators; and the row limit of the input norm."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    M, C, H = 4, 2048, 8192
+    x = randn_bf16((M, 1, C), 61).to(gpu)
+    nw = randn_bf16((C,), 62, scale=0.1, mean=1.0).to(gpu)
+    wg = randn_bf16((H, C), 63, scale=0.03).to(gpu)
+    wu = randn_bf16((H, C), 64, scale=0.03).to(gpu)
+    wd = randn_bf16((C, H), 65, scale=0.03).to(gpu)
+    t = cke.linear_decode_fused(x, wg, norm_weight=nw, eps=1e-5, w_up=wu)
+    y = cke.linear_decode_fused(t, wd, residual=x)
+    h = cke.rms_norm(x, nw, 1e-5)
+    t_seq = cke.silu_mul(cke.linear_decode(h, wg), cke.linear_decode(h, wu))
+    y_seq = x + cke.linear_decode(t_seq, wd)
+    torch.cuda.synchronize()
+    assert (t.float() - t_seq.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, t_seq.float().abs().max().item())
+    assert (y.float() - y_seq.float()).abs().max().item() <= 2.0 ** -6 * max(1.0, y_seq.float().abs().max().item())
+    assert cke.linear_decode_fused_max_rows(2048) == 11 and cke.linear_decode_fused_max_rows(8192) == 2
+    with pytest.raises(RuntimeError):
+        cke.linear_decode_fused(randn_bf16((12, C), 1).to(gpu), wg, norm_weight=nw)   # too many rows to stage
+    with pytest.raises(RuntimeError):
+        cke.linear_decode_fused(x, wg, norm_weight=nw[:100])
+    with pytest.raises(RuntimeError):                                                  # width not a multiple of 512
+        cke.linear_decode_fused(randn_bf16((2, 1056), 1).to(gpu), randn_bf16((64, 1056), 2).to(gpu),
+                                norm_weight=randn_bf16((1056,), 3).to(gpu))
