@@ -85,7 +85,7 @@ struct LinearParams {
 };
 
 // Launchers: return a hipError_t cast to int (0 = success).
-int linear_skinny_plan(int N, int K, int waves_per_wg, int num_cus);
+int linear_skinny_plan(int N, int K, int waves_per_wg, int num_cus, int rows_per_wave, int kstep);
 bool linear_skinny_can_stage(int M, int K);
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream);
 int launch_attn_prefill(const PrefillParams& p, int HD, hipStream_t stream);        // a wavefront per column group

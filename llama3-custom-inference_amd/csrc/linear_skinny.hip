@@ -27,10 +27,19 @@ namespace {
 // Elements of LDS the staged activations may take (rows are padded by 8 elements).
 constexpr int kXldsMaxElems = 24576;
 
-template <int NW, int CBLK, int U, bool SWIGLU, bool XLDS>
+// RW = weight rows per wavefront.  16: the plain mapping above.  4 (at most 4 activation rows, one
+// matrix): the 16 rows and the 16 columns of a matrix instruction are both split into four k
+// ranges -- tile row i is weight row i % 4 over k range i / 4, tile column j is activation row
+// j % 4 over k range j / 4 -- so one instruction covers 4 weight rows x 128 k, the blocks on the
+// diagonal (i / 4 == j / 4) hold the products and the rest is ignored.  Four times as many
+// wavefronts share a matrix with few rows, and a weight row is read 256 contiguous bytes at a time.
+template <int NW, int CBLK, int U, bool SWIGLU, bool XLDS, int RW>
 __global__ void __launch_bounds__(NW * kWaveSize)
 linear_skinny_kernel(const LinearParams p) {
     static_assert(!XLDS || CBLK == 1, "activations are staged in LDS only for up to 16 rows");
+    static_assert(RW == 16 || (RW == 4 && CBLK == 1 && !SWIGLU), "the four-row mapping is for one matrix");
+    constexpr int KQ = 16 / RW;                            // k ranges per matrix instruction
+    constexpr int KSTEP = 32 * KQ;                         // k covered by one step
     constexpr int ACC = SWIGLU ? 2 : 1;
     __shared__ float s_red[NW][ACC][CBLK][256];
     extern __shared__ __align__(16) uint16_t s_x[];        // XLDS: M rows of K + 8 elements
@@ -43,21 +52,22 @@ linear_skinny_kernel(const LinearParams p) {
     const int sk = p.sk;                                   // wavefronts per row block (divides NW)
     const int rb = int(blockIdx.x) * (NW / sk) + wave / sk;
     const int kslice = wave % sk;
-    const int n0 = rb * 16;
-    const int ksteps = p.K / 32;
+    const int n0 = rb * RW;
+    const int ksteps = p.K / KSTEP;
     const int kpw = (ksteps + sk - 1) / sk;
     const int ks0 = kslice * kpw;
     const int ks1 = min(ksteps, ks0 + kpw);
 
-    const int row = min(n0 + fn, p.N - 1);                 // rows past N are loaded clamped and never stored
-    const uint16_t* wp0 = p.w0 + int64_t(row) * p.w_stride + fg * 8;
-    const uint16_t* wp1 = SWIGLU ? p.w1 + int64_t(row) * p.w_stride + fg * 8 : nullptr;
+    const int row = min(n0 + fn % RW, p.N - 1);            // rows past N are loaded clamped and never stored
+    const int koff = (fn / RW) * 32 + fg * 8;              // this lane's k offset within a step
+    const uint16_t* wp0 = p.w0 + int64_t(row) * p.w_stride + koff;
+    const uint16_t* wp1 = SWIGLU ? p.w1 + int64_t(row) * p.w_stride + koff : nullptr;
     const uint16_t* xp[CBLK];
     bool xvalid[CBLK];
 #pragma unroll
     for (int cb = 0; cb < CBLK; ++cb) {
-        xvalid[cb] = cb * 16 + fn < p.M;
-        xp[cb] = p.x + int64_t(xvalid[cb] ? cb * 16 + fn : 0) * p.x_stride + fg * 8;
+        xvalid[cb] = cb * 16 + fn % RW < p.M;
+        xp[cb] = p.x + int64_t(xvalid[cb] ? cb * 16 + fn % RW : 0) * p.x_stride + koff;
     }
 
     f32x4_t acc[ACC][CBLK];
@@ -71,12 +81,12 @@ linear_skinny_kernel(const LinearParams p) {
     // instructions of step ks have read it, so about U loads per operand stay in flight.
     uint4 rw0[U], rw1[SWIGLU ? U : 1], rx[XLDS ? 1 : CBLK][XLDS ? 1 : U];
     auto fill = [&](int u, int ks) {
-        rw0[u] = load16(wp0 + ks * 32);
-        if constexpr (SWIGLU) rw1[u] = load16(wp1 + ks * 32);
+        rw0[u] = load16(wp0 + ks * KSTEP);
+        if constexpr (SWIGLU) rw1[u] = load16(wp1 + ks * KSTEP);
         if constexpr (!XLDS) {
 #pragma unroll
             for (int cb = 0; cb < CBLK; ++cb) {
-                rx[cb][u] = xvalid[cb] ? load16(xp[cb] + ks * 32) : make_uint4(0u, 0u, 0u, 0u);
+                rx[cb][u] = xvalid[cb] ? load16(xp[cb] + ks * KSTEP) : make_uint4(0u, 0u, 0u, 0u);
             }
         }
     };
@@ -142,7 +152,7 @@ linear_skinny_kernel(const LinearParams p) {
         }
         __syncthreads();
     }
-    const uint16_t* lx = s_x + (xvalid[0] ? fn : 0) * KP + fg * 8;
+    const uint16_t* lx = s_x + (xvalid[0] ? fn % RW : 0) * KP + koff;
 
     for (int ks = ks0; ks < ks1; ks += U) {
 #pragma unroll
@@ -152,7 +162,7 @@ linear_skinny_kernel(const LinearParams p) {
                 for (int cb = 0; cb < CBLK; ++cb) {
                     uint4 xv;
                     if constexpr (XLDS) {
-                        xv = *reinterpret_cast<const uint4*>(lx + (ks + u) * 32);
+                        xv = *reinterpret_cast<const uint4*>(lx + (ks + u) * KSTEP);
                         if (!xvalid[0]) xv = make_uint4(0u, 0u, 0u, 0u);
                     } else {
                         xv = rx[cb][u];
@@ -168,6 +178,31 @@ linear_skinny_kernel(const LinearParams p) {
                 if (ks + U + u < ks1) fill(u, ks + U + u);
             }
         }
+    }
+
+    if constexpr (RW == 4) {
+        // acc[0][0][t] of lane l is tile row 4*(l/16) + t, column l % 16: weight row n0 + t over k
+        // range l / 16 against activation row (l % 16) % 4 over k range (l % 16) / 4.  The lanes
+        // whose two k ranges agree hold products; they meet, with the other wavefronts of the row
+        // group, in LDS, and the group's first wavefront finishes its 4 x 4 results.
+        float* part = &s_red[wave][0][0][0];
+        if ((fn >> 2) == fg) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) part[(fg * 4 + (fn & 3)) * 4 + t] = acc[0][0][t];
+        }
+        __syncthreads();
+        if (kslice != 0 || lane >= 16) return;
+        const int m = lane >> 2, t = lane & 3;             // activation row, weight row within the group
+        const int n = n0 + t;
+        if (m >= p.M || n >= p.N) return;
+        float o = 0.f;
+        for (int w = 0; w < sk; ++w) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) o += s_red[wave + w][0][0][(q * 4 + m) * 4 + t];
+        }
+        if (p.res) o = bf16_to_f32(p.res[int64_t(m) * p.y_stride + n]) + __uint_as_float(f32_to_bf16_bits(o) << 16);
+        p.y[int64_t(m) * p.y_stride + n] = uint16_t(f32_to_bf16_bits(o));
+        return;
     }
 
     // ---- the sk wavefronts of a row block add up in LDS; the first of them finishes the rows
@@ -228,23 +263,24 @@ linear_skinny_kernel(const LinearParams p) {
     }
 }
 
-template <int NW, int CBLK, int U, bool SWIGLU, bool XLDS>
+template <int NW, int CBLK, int U, bool SWIGLU, bool XLDS, int RW = 16>
 int launch_variant(const LinearParams& p, hipStream_t stream) {
-    const int row_blocks = (p.N + 15) / 16;
+    const int row_blocks = (p.N + RW - 1) / RW;
     const int rb_per_wg = NW / p.sk;
     const dim3 grid(unsigned((row_blocks + rb_per_wg - 1) / rb_per_wg));
     const size_t lds = XLDS ? size_t(p.M) * size_t(p.K + 8) * sizeof(uint16_t) : 0;
-    hipLaunchKernelGGL((linear_skinny_kernel<NW, CBLK, U, SWIGLU, XLDS>), grid, dim3(NW * kWaveSize), lds, stream, p);
+    hipLaunchKernelGGL((linear_skinny_kernel<NW, CBLK, U, SWIGLU, XLDS, RW>), grid, dim3(NW * kWaveSize), lds, stream,
+                       p);
     return int(hipGetLastError());
 }
 
 }  // namespace
 
-// Wavefronts per row block: split K until the launch has about two workgroups per CU, as long
-// as every wavefront keeps at least four k steps.
-int linear_skinny_plan(int N, int K, int waves_per_wg, int num_cus) {
-    const int row_blocks = (N + 15) / 16;
-    const int ksteps = K / 32;
+// Wavefronts per row block (of `rows_per_wave` weight rows, `kstep` k per step): split K until
+// the launch has about two workgroups per CU, as long as every wavefront keeps at least four steps.
+int linear_skinny_plan(int N, int K, int waves_per_wg, int num_cus, int rows_per_wave, int kstep) {
+    const int row_blocks = (N + rows_per_wave - 1) / rows_per_wave;
+    const int ksteps = K / kstep;
     int sk = 1;
     while (sk < waves_per_wg && int64_t(row_blocks) * sk / waves_per_wg < 2 * int64_t(num_cus) &&
            ksteps / (2 * sk) >= 4) {
@@ -262,10 +298,17 @@ bool linear_skinny_can_stage(int M, int K) {
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream) {
     const bool wide = p.M > 16;
     const bool stage = p.norm_w != nullptr;   // the caller has checked linear_skinny_can_stage
-    // few row blocks and a long K (the MLP's down projection): sixteen wavefronts share a row block
     const int row_blocks = (p.N + 15) / 16;
+    // a matrix with too few 16-row blocks to fill the device, and at most four activation rows:
+    // four weight rows per wavefront
+    if (!swiglu && p.M <= 4 && p.K % 128 == 0 && row_blocks < 2 * num_cus) {
+        p.sk = linear_skinny_plan(p.N, p.K, 8, num_cus, 4, 128);
+        return stage ? launch_variant<8, 1, 8, false, true, 4>(p, stream)
+                     : launch_variant<8, 1, 8, false, false, 4>(p, stream);
+    }
+    // few row blocks and a long K (the MLP's down projection): sixteen wavefronts share a row block
     const bool big_wg = !wide && !swiglu && row_blocks < num_cus && p.K / 32 >= 128;
-    p.sk = linear_skinny_plan(p.N, p.K, big_wg ? 16 : 8, num_cus);
+    p.sk = linear_skinny_plan(p.N, p.K, big_wg ? 16 : 8, num_cus, 16, 32);
     if (swiglu) {
         if (wide) return launch_variant<8, 4, 4, true, false>(p, stream);
         return stage ? launch_variant<8, 1, 8, true, true>(p, stream) : launch_variant<8, 1, 8, true, false>(p, stream);

@@ -28,7 +28,7 @@ def assert_linear_close(y, ref, what):
 # batch sizes up to 64, and shapes off every multiple the kernel tiles by
 SHAPES = [(1, 3072, 2048), (1, 2048, 2048), (1, 2048, 8192), (1, 128256, 2048), (3, 1024, 512), (16, 3072, 2048),
           (17, 512, 256), (64, 3072, 2048), (64, 2048, 8192), (5, 20, 32), (2, 36, 64), (33, 100, 96),
-          (64, 16, 4096), (1, 16, 32), (8, 6144, 4096)]
+          (64, 16, 4096), (1, 16, 32), (8, 6144, 4096), (4, 2048, 8192), (4, 20, 128), (2, 3072, 2048), (3, 4, 384)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
