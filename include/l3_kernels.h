@@ -247,6 +247,21 @@ int l3_argmax(const void* logits, int64_t row_stride, int rows, int V, void* wor
               int64_t* out, void* stream);
 
 /*
+ * One greedy decoding step's tail on the device: the argmax of every logits row, then the
+ * bookkeeping of the reference's generate() loop (model.py:371-378) with next = *pos + 1
+ * (clamped to total_len - 1):
+ *   nxt = text_mask[b][next] ? tokens[b][next] : argmax(logits[b])
+ *   tokens[b][next] = nxt;  tok[b] = nxt;  eos[b] |= !text_mask[b][next] && nxt in stop_tokens
+ * and finally *pos += 1, *kv_len += 1.  tokens (rows, total_len) int64 and text_mask (rows,
+ * total_len) one byte per element, both contiguous; tok (rows) int64; eos (rows) one byte per
+ * element; pos, kv_len device int32.  Workspace as for l3_argmax.  With every operand in device
+ * memory the step can be replayed from a HIP graph.
+ */
+int l3_greedy_step(const void* logits, int64_t row_stride, int rows, int V, void* workspace, size_t workspace_bytes,
+                   int64_t* tokens, const uint8_t* text_mask, int64_t total_len, int64_t* tok, int32_t* pos,
+                   int32_t* kv_len, uint8_t* eos, const int64_t* stop_tokens, int n_stop, void* stream);
+
+/*
  * Rotary embedding on adjacent pairs:
  *   y[b,t,h,2i]   = bf16( x[b,t,h,2i] * freq[t,2i] - x[b,t,h,2i+1] * freq[t,2i+1] )
  *   y[b,t,h,2i+1] = bf16( x[b,t,h,2i] * freq[t,2i+1] + x[b,t,h,2i+1] * freq[t,2i] )

@@ -458,6 +458,25 @@ int l3_argmax(const void* logits, int64_t row_stride, int rows, int V, void* wor
                          static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 
+int l3_greedy_step(const void* logits, int64_t row_stride, int rows, int V, void* workspace, size_t workspace_bytes,
+                   int64_t* tokens, const uint8_t* text_mask, int64_t total_len, int64_t* tok, int32_t* pos,
+                   int32_t* kv_len, uint8_t* eos, const int64_t* stop_tokens, int n_stop, void* stream) {
+    if (!logits || !workspace || !tokens || !text_mask || !tok || !pos || !kv_len || !eos || (n_stop > 0 && !stop_tokens))
+        return L3_ERR_NULL_POINTER;
+    if (rows <= 0 || V <= 0 || rows > 65535 || total_len <= 0 || n_stop < 0) return L3_ERR_SHAPE;
+    if (row_stride < V) return L3_ERR_STRIDE;
+    if (!aligned(logits, 2) || !aligned(workspace, 8) || !aligned(tokens, 8) || !aligned(tok, 8) || !aligned(pos, 4) ||
+        !aligned(kv_len, 4) || (stop_tokens && !aligned(stop_tokens, 8)))
+        return L3_ERR_ALIGNMENT;
+    if (workspace_bytes < l3_argmax_workspace_bytes(rows, V)) return L3_ERR_WORKSPACE;
+    const size_t parts = size_t(rows) * size_t(argmax_parts(V));
+    float* pv = static_cast<float*>(workspace);
+    int* pi = reinterpret_cast<int*>(pv + parts);
+    return launch_greedy_step(static_cast<const uint16_t*>(logits), row_stride, rows, V, pv, pi, tokens, text_mask,
+                              total_len, tok, pos, kv_len, eos, stop_tokens, n_stop,
+                              static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
 int l3_rot_embed(const void* x, const float* freq, void* y, int B, int T, int NH, int HD,
                  const int64_t x_strides[3], void* stream) {
     if (!x || !freq || !y || !x_strides) return L3_ERR_NULL_POINTER;

@@ -105,6 +105,9 @@ constexpr int kArgmaxChunk = 2048;  // logits one workgroup of the first argmax 
 int argmax_parts(int V);
 int launch_argmax(const uint16_t* logits, int64_t row_stride, int rows, int V, float* part_val, int* part_idx,
                   int64_t* out, hipStream_t stream);
+int launch_greedy_step(const uint16_t* logits, int64_t row_stride, int rows, int V, float* part_val, int* part_idx,
+                       int64_t* tokens, const uint8_t* text_mask, int64_t total_len, int64_t* tok, int* pos,
+                       int* kv_len, uint8_t* eos, const int64_t* stop, int n_stop, hipStream_t stream);
 int launch_rot_embed(const uint16_t* x, const float* freq, uint16_t* y, int B, int T, int NH, int HD,
                      int64_t sb, int64_t st, int64_t sh, bool vec_ok, hipStream_t stream);
 int launch_rot_embed_append(const uint16_t* qkv, const float* table, uint16_t* q_out, uint16_t* cache_k,

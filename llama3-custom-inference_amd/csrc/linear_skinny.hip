@@ -318,7 +318,7 @@ int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t s
         return stage ? launch_variant<16, 1, 8, false, true>(p, stream)
                      : launch_variant<16, 1, 8, false, false>(p, stream);
     }
-    return stage ? launch_variant<8, 1, 16, false, true>(p, stream) : launch_variant<8, 1, 16, false, false>(p, stream);
+    return stage ? launch_variant<8, 1, 8, false, true>(p, stream) : launch_variant<8, 1, 8, false, false>(p, stream);
 }
 
 }  // namespace l3

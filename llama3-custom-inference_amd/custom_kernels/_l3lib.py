@@ -102,6 +102,12 @@ SIGNATURES = {
          ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
          ctypes.c_void_p],
     ),
+    "l3_greedy_step": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p],
+    ),
     "l3_argmax_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "l3_argmax": (
         ctypes.c_int,

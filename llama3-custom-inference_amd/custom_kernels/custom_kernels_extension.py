@@ -471,6 +471,39 @@ def argmax(logits):
     return out
 
 
+def greedy_step(logits, tokens, text_mask, tok, pos, kv_len, eos, stop_tokens):
+    """The tail of one greedy decoding step, in place and on the device (model.py:371-378): pick
+    argmax(logits[b]) unless position pos + 1 still belongs to the prompt (text_mask), store the
+    token into tokens[:, pos + 1] and tok, mark rows that produced a stop token in eos, and
+    advance pos and kv_len by one.  logits (rows, V) bf16; tokens (rows, L) int64; text_mask
+    (rows, L) bool; tok (rows, 1) or (rows,) int64; pos, kv_len int32 scalars; eos (rows) bool;
+    stop_tokens int64.  An extension."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("logits", logits)
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise RuntimeError("greedy_step expects (rows, V) logits with a contiguous last dimension")
+    rows, V = logits.shape
+    L = tokens.shape[1]
+    ok = (tokens.dtype == torch.int64 and tokens.is_contiguous() and tokens.shape[0] == rows
+          and text_mask.dtype == torch.bool and text_mask.is_contiguous() and tuple(text_mask.shape) == (rows, L)
+          and tok.dtype == torch.int64 and tok.is_contiguous() and tok.numel() == rows
+          and pos.dtype == torch.int32 and pos.numel() == 1 and kv_len.dtype == torch.int32 and kv_len.numel() == 1
+          and eos.dtype == torch.bool and eos.is_contiguous() and eos.numel() == rows
+          and stop_tokens.dtype == torch.int64 and stop_tokens.is_contiguous())
+    if not ok or any(t.device != logits.device for t in (tokens, text_mask, tok, pos, kv_len, eos, stop_tokens)):
+        raise RuntimeError("greedy_step: state tensors have the wrong dtype, shape, layout or device")
+    with torch.cuda.device(logits.device):
+        ws_bytes = lib.l3_argmax_workspace_bytes(rows, V)
+        stream_ptr = _stream_ptr(logits.device)
+        ws = _workspace(logits.device, stream_ptr, ws_bytes)
+        rc = lib.l3_greedy_step(logits.data_ptr(), logits.stride(0), rows, V, ws.data_ptr(), ws_bytes,
+                                tokens.data_ptr(), text_mask.data_ptr(), L, tok.data_ptr(), pos.data_ptr(),
+                                kv_len.data_ptr(), eos.data_ptr(), stop_tokens.data_ptr(), stop_tokens.numel(),
+                                stream_ptr)
+    if rc != 0:
+        _fail(rc, f"rows={rows} V={V}")
+
+
 def rot_embed(input, freq):
     """input (B, T, NH, HD) bf16 (any strides on the first three dims), freq (T, HD) float32
     interleaved cos/sin -> contiguous (B, T, NH, HD) bf16 (model.py:100-101)."""

@@ -333,6 +333,10 @@ class GraphedDecodeLoop:
                 next_norm = m.layers[i + 1]["ln_1"] if i + 1 < len(m.layers) else m.ln_f
                 x, h = ops.add_rms_norm(x, mlp, next_norm, c.norm_eps)
             logits = m._linear(h[:, -1], m.wte)
+        if hasattr(ops, "greedy_step"):
+            # argmax and generate()'s bookkeeping (model.py:371-378) in two launches
+            ops.greedy_step(logits, self.tokens, self.text_mask, self.tok, self.pos, self.kv_len, self.eos, self.stop)
+            return
         nxt = ops.argmax(logits)   # first maximum of the bf16 logits = argmax of their float copy
         # generate() bookkeeping (model.py:373-378) at position pos + 1, all on the device
         cur = (self.pos + 1).long().clamp_(max=self.total_len - 1)

@@ -201,3 +201,18 @@ def test_linear_decode_fused_argument_checks():
     assert call(M=3, K=8192) == _l3lib.L3_ERR_SHAPE
     assert call(norm=FAKE + 2) == _l3lib.L3_ERR_ALIGNMENT
     assert call(res=FAKE + 4) == _l3lib.L3_ERR_ALIGNMENT
+
+
+def test_greedy_step_argument_checks():
+    lib = _l3lib.load()
+
+    def call(logits=FAKE, ws=FAKE, ws_bytes=1 << 20, rows=4, V=1000, stride=1000, L=16, eos=FAKE, pos=FAKE, n_stop=1):
+        return lib.l3_greedy_step(logits, stride, rows, V, ws, ws_bytes, FAKE, FAKE, L, FAKE, pos, FAKE, eos, FAKE,
+                                  n_stop, None)
+
+    assert call(eos=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert call(rows=0) == _l3lib.L3_ERR_SHAPE
+    assert call(L=0) == _l3lib.L3_ERR_SHAPE
+    assert call(stride=999) == _l3lib.L3_ERR_STRIDE
+    assert call(pos=FAKE + 2) == _l3lib.L3_ERR_ALIGNMENT
+    assert call(ws_bytes=8) == _l3lib.L3_ERR_WORKSPACE

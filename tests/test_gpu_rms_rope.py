@@ -253,3 +253,37 @@ def test_argmax_first_maximum(gpu, rows, V):
     wide = randn_bf16((rows, V + 9), 92).to(gpu)
     np.testing.assert_array_equal(cke.argmax(wide[:, :V]).cpu().numpy(),
                                   torch.argmax(wide[:, :V].float(), dim=-1).cpu().numpy())
+
+
+@pytest.mark.parametrize("rows,V,L,pos0", [(1, 128256, 256, 127), (64, 128256, 256, 200), (5, 1000, 20, 7), (3, 50, 9, 8)])
+def test_greedy_step_matches_generate_bookkeeping(gpu, rows, V, L, pos0):
+    """argmax + the per-token bookkeeping of generate() (model.py:371-378) in place on the device,
+    against the same steps written with torch operators; two steps in a row."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    g = torch.Generator().manual_seed(rows * 1000 + V)
+    tokens = torch.randint(0, V, (rows, L), generator=g)
+    text_mask = torch.rand((rows, L), generator=g) < 0.5
+    eos = torch.zeros(rows, dtype=torch.bool)
+    state = dict(tokens=tokens.to(gpu), text_mask=text_mask.to(gpu), tok=torch.zeros((rows, 1), dtype=torch.long, device=gpu),
+                 pos=torch.tensor([pos0], dtype=torch.int32, device=gpu),
+                 kv_len=torch.tensor([pos0 + 1], dtype=torch.int32, device=gpu), eos=eos.to(gpu))
+    ref_tokens, ref_eos, ref_pos = tokens.clone(), eos.clone(), pos0
+    for step in range(2):
+        logits = randn_bf16((rows, V), 7 + step)
+        want = torch.argmax(logits.float(), dim=-1)
+        # every second row's pick is declared a stop token
+        stop = torch.unique(torch.cat([want[::2], torch.tensor([V + 5])]))
+        cke.greedy_step(logits.to(gpu), state["tokens"], state["text_mask"], state["tok"], state["pos"],
+                        state["kv_len"], state["eos"], stop.to(gpu))
+        torch.cuda.synchronize()
+        cur = min(ref_pos + 1, L - 1)
+        keep = text_mask[:, cur]
+        nxt = torch.where(keep, ref_tokens[:, cur], want)
+        ref_tokens[:, cur] = nxt
+        ref_eos |= ~keep & torch.isin(nxt, stop)
+        ref_pos += 1
+        assert torch.equal(state["tokens"].cpu(), ref_tokens), f"tokens after step {step}"
+        assert torch.equal(state["tok"].cpu().view(-1), nxt)
+        assert torch.equal(state["eos"].cpu(), ref_eos)
+        assert state["pos"].item() == ref_pos and state["kv_len"].item() == ref_pos + 1
