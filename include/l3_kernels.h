@@ -237,6 +237,23 @@ int l3_linear_decode_fused(const void* x, const void* norm_weight, float norm_ep
                            int64_t y_stride, void* stream);
 
 /*
+ * The fused qkv projection of a decode step with what follows it folded in (model.py:95-106 for
+ * one new token per sequence): qkv = [rms_norm(x, norm_weight)] . w_qkv^T with N = (NH + 2 KVH) HD
+ * outputs in q | k | v order, rounded to bf16; the query and key heads are rotated with row *pos_dev
+ * of freq_table ((table_rows, HD) float32, interleaved cos/sin); rotated keys and the values go
+ * into cache_k / cache_v at token *pos_dev (element strides cache_strides = {batch, token},
+ * (KVH, HD) contiguous), the rotated queries to q_out (B, NH, HD).  One launch where the separate
+ * operators take l3_linear_decode_fused and l3_rot_embed_append, with the same bits.  Constraints
+ * of both apply (B <= L3_LINEAR_MAX_ROWS, K % 32 == 0, HD % 8 == 0, norm limits as above); an
+ * out-of-range position writes nothing.
+ */
+int l3_linear_qkv_rope_append(const void* x, const void* norm_weight, float norm_eps, const void* w_qkv,
+                              const float* freq_table, void* q_out, void* cache_k, void* cache_v,
+                              const int32_t* pos_dev, int B, int NH, int KVH, int HD, int K, int64_t x_stride,
+                              int64_t w_stride, const int64_t cache_strides[2], int cache_len, int table_rows,
+                              void* stream);
+
+/*
  * out[r] = index of the first maximum of the bf16 row logits[r*row_stride : r*row_stride + V]
  * (int64, like torch.argmax; a row of NaNs gives 0): the greedy pick of model.py:371.  Two small
  * launches (per-chunk maxima into the caller's workspace of l3_argmax_workspace_bytes(rows, V)

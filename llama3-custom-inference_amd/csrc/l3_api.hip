@@ -391,16 +391,24 @@ int l3_silu_mul(const void* a, const void* b, void* y, int64_t n, void* stream) 
 
 namespace {
 
+struct QkvTarget {
+    const float* table;
+    const int* pos;
+    uint16_t *q_out, *cache_k, *cache_v;
+    int NH, KVH, HD, cache_len, table_rows;
+    int64_t c_sb, c_st;
+};
+
 int linear_decode_impl(const void* x, const void* norm_w, float norm_eps, const void* w0, const void* w1,
                        const void* res, void* y, int M, int N, int K, int64_t x_stride, int64_t w_stride,
-                       int64_t y_stride, bool swiglu, void* stream) {
-    if (!x || !w0 || !y || (swiglu && !w1)) return L3_ERR_NULL_POINTER;
+                       int64_t y_stride, bool swiglu, void* stream, const QkvTarget* qkv = nullptr) {
+    if (!x || !w0 || (!y && !qkv) || (swiglu && !w1)) return L3_ERR_NULL_POINTER;
     if (M <= 0 || M > L3_LINEAR_MAX_ROWS || N <= 0 || K <= 0 || N % 4 != 0 || K % 32 != 0) return L3_ERR_SHAPE;
     if (N > (1 << 24) || K > (1 << 24)) return L3_ERR_SHAPE;
     if (norm_w && !linear_skinny_can_stage(M, K)) return L3_ERR_SHAPE;
     if (x_stride < K || w_stride < K || y_stride < N || x_stride % 8 || w_stride % 8 || y_stride % 4)
         return L3_ERR_STRIDE;
-    if (!aligned(x, 16) || !aligned(w0, 16) || (swiglu && !aligned(w1, 16)) || !aligned(y, 8) ||
+    if (!aligned(x, 16) || !aligned(w0, 16) || (swiglu && !aligned(w1, 16)) || (y && !aligned(y, 8)) ||
         (norm_w && !aligned(norm_w, 16)) || (res && !aligned(res, 8)))
         return L3_ERR_ALIGNMENT;
     LinearParams p;
@@ -414,6 +422,16 @@ int linear_decode_impl(const void* x, const void* norm_w, float norm_eps, const 
     p.M = M; p.N = N; p.K = K;
     p.x_stride = x_stride; p.w_stride = w_stride; p.y_stride = y_stride;
     p.sk = 1;
+    if (qkv) {
+        p.rope_table = qkv->table; p.rope_pos = qkv->pos; p.q_out = qkv->q_out;
+        p.cache_k = qkv->cache_k; p.cache_v = qkv->cache_v;
+        p.NH = qkv->NH; p.KVH = qkv->KVH; p.HD = qkv->HD; p.cache_len = qkv->cache_len; p.table_rows = qkv->table_rows;
+        p.c_sb = qkv->c_sb; p.c_st = qkv->c_st;
+    } else {
+        p.rope_table = nullptr; p.rope_pos = nullptr; p.q_out = p.cache_k = p.cache_v = nullptr;
+        p.NH = p.KVH = p.HD = p.cache_len = p.table_rows = 0;
+        p.c_sb = p.c_st = 0;
+    }
     return launch_linear_skinny(p, swiglu, current_device_cus(), static_cast<hipStream_t>(stream)) == 0 ? L3_OK
                                                                                                         : L3_ERR_HIP;
 }
@@ -437,6 +455,31 @@ int l3_linear_decode_fused(const void* x, const void* norm_weight, float norm_ep
                            int64_t y_stride, void* stream) {
     return linear_decode_impl(x, norm_weight, norm_eps, w, w_up, residual, y, M, N, K, x_stride, w_stride, y_stride,
                               w_up != nullptr, stream);
+}
+
+int l3_linear_qkv_rope_append(const void* x, const void* norm_weight, float norm_eps, const void* w_qkv,
+                              const float* freq_table, void* q_out, void* cache_k, void* cache_v,
+                              const int32_t* pos_dev, int B, int NH, int KVH, int HD, int K, int64_t x_stride,
+                              int64_t w_stride, const int64_t cache_strides[2], int cache_len, int table_rows,
+                              void* stream) {
+    if (!freq_table || !q_out || !cache_k || !cache_v || !pos_dev || !cache_strides) return L3_ERR_NULL_POINTER;
+    if (NH <= 0 || KVH <= 0 || HD <= 0 || HD % 8 != 0 || cache_len <= 0 || table_rows <= 0) return L3_ERR_SHAPE;
+    if (int64_t(NH + 2 * KVH) * HD > (1 << 24)) return L3_ERR_SHAPE;
+    if (cache_strides[0] < 0 || cache_strides[1] < 0 || cache_strides[1] % 8 || (B > 1 && cache_strides[0] % 8))
+        return L3_ERR_STRIDE;
+    if (!aligned(q_out, 16) || !aligned(cache_k, 16) || !aligned(cache_v, 16) || !aligned(freq_table, 16) ||
+        !aligned(pos_dev, 4))
+        return L3_ERR_ALIGNMENT;
+    QkvTarget t;
+    t.table = freq_table; t.pos = pos_dev;
+    t.q_out = static_cast<uint16_t*>(q_out);
+    t.cache_k = static_cast<uint16_t*>(cache_k);
+    t.cache_v = static_cast<uint16_t*>(cache_v);
+    t.NH = NH; t.KVH = KVH; t.HD = HD; t.cache_len = cache_len; t.table_rows = table_rows;
+    t.c_sb = cache_strides[0]; t.c_st = cache_strides[1];
+    const int N = (NH + 2 * KVH) * HD;
+    return linear_decode_impl(x, norm_weight, norm_eps, w_qkv, nullptr, nullptr, nullptr, B, N, K, x_stride, w_stride,
+                              N, false, stream, &t);
 }
 
 size_t l3_argmax_workspace_bytes(int rows, int V) {

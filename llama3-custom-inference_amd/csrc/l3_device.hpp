@@ -101,6 +101,24 @@ __device__ __forceinline__ float wave_max(float x) {
 // 2^x through the hardware v_exp_f32 (inputs here are <= 0 or small; no denormal fix-up).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Rotation of one adjacent bf16 pair (packed in a word) by (cos, sin): the rotary embedding of
+// custom_kernels.cu:400-414, float32 arithmetic, one rounding.
+__device__ __forceinline__ uint32_t rotate_pair(uint32_t xw, float c, float s) {
+    const float x0 = bf16lo_to_f32(xw);
+    const float x1 = bf16hi_to_f32(xw);
+    // x0*c - x1*s can cancel; a plain float32 evaluation then carries the rounding error of
+    // the larger product into a much smaller result and can miss the exact answer by more
+    // than one bf16 ulp.  The second product's rounding error is recovered exactly with an
+    // fma (e = x1*s - p) so that the error stays relative to the result itself.
+    const float p0 = x1 * s;
+    const float e0 = fmaf(x1, s, -p0);
+    const float y0 = fmaf(x0, c, -p0) - e0;
+    const float p1 = x1 * c;
+    const float e1 = fmaf(x1, c, -p1);
+    const float y1 = fmaf(x0, s, p1) + e1;
+    return pack_bf16x2(y0, y1);
+}
+
 // bf16(silu(a)) as a float: torch's F.silu(a) * b materialises silu's bf16 result before the
 // multiplication (model.py:134), and so does every kernel here that fuses the product.
 __device__ __forceinline__ float silu_rounded(float a) {

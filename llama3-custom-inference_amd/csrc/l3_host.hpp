@@ -82,6 +82,15 @@ struct LinearParams {
     int M, N, K;
     int64_t x_stride, w_stride, y_stride;
     int sk;               // wavefronts that split K for one block of 16 weight rows (set by the launcher)
+    // fused qkv projection of a decode step (rope_table != null): the N = (NH + 2 KVH) HD outputs of
+    // activation row b are rotated at position *rope_pos and go to q_out / the KV cache instead of y
+    const float* rope_table;   // (table_rows, HD) interleaved cos/sin
+    const int* rope_pos;
+    uint16_t* q_out;           // (M, NH, HD)
+    uint16_t* cache_k;         // element strides c_sb (batch), c_st (token); (KVH, HD) contiguous
+    uint16_t* cache_v;
+    int NH, KVH, HD, cache_len, table_rows;
+    int64_t c_sb, c_st;
 };
 
 // Launchers: return a hipError_t cast to int (0 = success).

@@ -24,6 +24,27 @@ namespace l3 {
 
 namespace {
 
+// Epilogue of the fused qkv projection: features n, n + 1 (n even) of activation row m, already
+// rounded to bf16 and packed in xw.  Query and key pairs are rotated at the device-side position,
+// keys and values land in the KV cache row of that position (model.py:100-106).
+__device__ __forceinline__ void store_qkv_pair(const LinearParams& p, int m, int n, uint32_t xw) {
+    const int pos = *p.rope_pos;
+    if (pos < 0 || pos >= p.cache_len || pos >= p.table_rows) return;   // never write outside the cache
+    const int slot = n / p.HD;
+    const int d = n % p.HD;
+    if (slot >= p.NH + p.KVH) {
+        *reinterpret_cast<uint32_t*>(p.cache_v + m * p.c_sb + pos * p.c_st + (slot - p.NH - p.KVH) * p.HD + d) = xw;
+        return;
+    }
+    const float2 cs = *reinterpret_cast<const float2*>(p.rope_table + int64_t(pos) * p.HD + d);
+    const uint32_t yw = rotate_pair(xw, cs.x, cs.y);
+    if (slot < p.NH) {
+        *reinterpret_cast<uint32_t*>(p.q_out + (int64_t(m) * p.NH + slot) * p.HD + d) = yw;
+    } else {
+        *reinterpret_cast<uint32_t*>(p.cache_k + m * p.c_sb + pos * p.c_st + (slot - p.NH) * p.HD + d) = yw;
+    }
+}
+
 // Elements of LDS the staged activations may take (rows are padded by 8 elements).
 constexpr int kXldsMaxElems = 24576;
 
@@ -194,12 +215,17 @@ linear_skinny_kernel(const LinearParams p) {
         if (kslice != 0 || lane >= 16) return;
         const int m = lane >> 2, t = lane & 3;             // activation row, weight row within the group
         const int n = n0 + t;
-        if (m >= p.M || n >= p.N) return;
         float o = 0.f;
         for (int w = 0; w < sk; ++w) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) o += s_red[wave + w][0][0][(q * 4 + m) * 4 + t];
         }
+        if (p.rope_table) {   // the even lane of a pair takes its partner's value and stores both
+            const float o1 = __shfl_xor(o, 1, kWaveSize);
+            if ((t & 1) == 0 && m < p.M && n < p.N) store_qkv_pair(p, m, n, pack_bf16x2(o, o1));
+            return;
+        }
+        if (m >= p.M || n >= p.N) return;
         if (p.res) o = bf16_to_f32(p.res[int64_t(m) * p.y_stride + n]) + __uint_as_float(f32_to_bf16_bits(o) << 16);
         p.y[int64_t(m) * p.y_stride + n] = uint16_t(f32_to_bf16_bits(o));
         return;
@@ -248,6 +274,11 @@ linear_skinny_kernel(const LinearParams p) {
             } else {
                 o[r] = acc[0][cb][r];
             }
+        }
+        if (p.rope_table) {
+            store_qkv_pair(p, m, n, pack_bf16x2(o[0], o[1]));
+            store_qkv_pair(p, m, n + 2, pack_bf16x2(o[2], o[3]));
+            continue;
         }
         if (p.res) {   // bf16(residual + bf16(product)), as the separate addition would give
             const uint2 rv = *reinterpret_cast<const uint2*>(p.res + int64_t(m) * p.y_stride + n);

@@ -13,22 +13,6 @@ namespace {
 
 constexpr int kRopeThreads = 256;
 
-__device__ __forceinline__ uint32_t rotate_pair(uint32_t xw, float c, float s) {
-    const float x0 = bf16lo_to_f32(xw);
-    const float x1 = bf16hi_to_f32(xw);
-    // x0*c - x1*s can cancel; a plain float32 evaluation then carries the rounding error of
-    // the larger product into a much smaller result and can miss the exact answer by more
-    // than one bf16 ulp.  The second product's rounding error is recovered exactly with an
-    // fma (e = x1*s - p) so that the error stays relative to the result itself.
-    const float p0 = x1 * s;
-    const float e0 = fmaf(x1, s, -p0);
-    const float y0 = fmaf(x0, c, -p0) - e0;
-    const float p1 = x1 * c;
-    const float e1 = fmaf(x1, c, -p1);
-    const float y1 = fmaf(x0, s, p1) + e1;
-    return pack_bf16x2(y0, y1);
-}
-
 // One 16-byte item (8 values = 4 pairs) per thread.  VPR = HD / 8 items per (b, t, h) row.
 __global__ void __launch_bounds__(kRopeThreads)
 rot_embed_vec_kernel(const uint16_t* __restrict__ x, const float* __restrict__ freq, uint16_t* __restrict__ y,

@@ -289,6 +289,46 @@ def rot_embed_append(qkv, freq_table, cache_k, cache_v, pos, n_head: int, out=No
     return out
 
 
+def linear_qkv_rope_append(x, w_qkv, freq_table, cache_k, cache_v, pos, n_head: int, norm_weight=None,
+                           eps: float = 1e-5):
+    """linear_decode_fused(x, w_qkv, norm_weight) followed by rot_embed_append in one launch: the
+    whole of model.py:95-106 for one new token per sequence.  x (B, 1, K); returns the rotated
+    queries (B, 1, n_head, HD); keys and values are written into the caches at ``pos``."""
+    lib = _l3lib.load()
+    x2, rows, N, K = _linear_args(x, (w_qkv,))
+    _require_gpu_bf16("cache_k", cache_k)
+    _require_gpu_bf16("cache_v", cache_v)
+    if cache_k.dim() != 4 or cache_k.shape != cache_v.shape or cache_k.stride() != cache_v.stride():
+        raise RuntimeError("cache_k and cache_v must be (maxB, L, KVH, HD) tensors of the same layout")
+    maxB, L, KVH, HD = cache_k.shape
+    if N != (n_head + 2 * KVH) * HD or rows > maxB:
+        raise RuntimeError(f"w_qkv {tuple(w_qkv.shape)} does not match n_head={n_head}, cache {tuple(cache_k.shape)}")
+    if cache_k.stride(3) != 1 or cache_k.stride(2) != HD:
+        raise RuntimeError("the (KVH, HD) dimensions of the cache must be contiguous")
+    if not freq_table.is_cuda or freq_table.dtype != torch.float32 or freq_table.dim() != 2 \
+            or freq_table.size(1) != HD or not freq_table.is_contiguous():
+        raise RuntimeError("freq_table must be a contiguous (rows, HD) float32 GPU tensor")
+    if not pos.is_cuda or pos.dtype != torch.int32 or pos.numel() != 1:
+        raise RuntimeError("pos must be a one-element int32 GPU tensor")
+    if norm_weight is not None:
+        _require_gpu_bf16("norm_weight", norm_weight)
+        if tuple(norm_weight.shape) != (K,) or not norm_weight.is_contiguous() \
+                or rows > linear_decode_fused_max_rows(K):
+            raise RuntimeError(f"linear_qkv_rope_append: norm_weight {tuple(norm_weight.shape)} / {rows} rows "
+                               f"do not fit the fused input norm (K={K})")
+    out = torch.empty((rows, 1, n_head, HD), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.l3_linear_qkv_rope_append(x2.data_ptr(), None if norm_weight is None else norm_weight.data_ptr(),
+                                           float(eps), w_qkv.data_ptr(), freq_table.data_ptr(), out.data_ptr(),
+                                           cache_k.data_ptr(), cache_v.data_ptr(), pos.data_ptr(), rows, n_head, KVH,
+                                           HD, K, x2.stride(0), w_qkv.stride(0),
+                                           _l3lib.i64_array((cache_k.stride(0), cache_k.stride(1))), L,
+                                           freq_table.size(0), _stream_ptr(x.device))
+    if rc != 0:
+        _fail(rc, f"B={rows} NH={n_head} KVH={KVH} HD={HD} K={K}")
+    return out
+
+
 def rms_norm(input, weight, eps):
     """input (B, T, C) bf16, weight (C,) bf16 -> (B, T, C) bf16 (model.py:70-72)."""
     lib = _l3lib.load()

@@ -305,11 +305,12 @@ class GraphedDecodeLoop:
         ops = m.ops
         x = F.embedding(self.tok, m.wte)
         if 0 < B <= m._fused_rows():
-            # five launches per layer: norms and residual additions ride with the linears
+            # five launches per layer: norms, rotary embedding, cache append and residual additions ride
+            # with the linears
             lin = ops.linear_decode_fused
             for L in m.layers:
-                qkv = lin(x, L["c_attn"], norm_weight=L["ln_1"], eps=c.norm_eps)
-                q = ops.rot_embed_append(qkv, m.freqs_cis, L["cache_k"], L["cache_v"], self.pos, c.n_head)
+                q = ops.linear_qkv_rope_append(x, L["c_attn"], m.freqs_cis, L["cache_k"], L["cache_v"], self.pos,
+                                               c.n_head, norm_weight=L["ln_1"], eps=c.norm_eps)
                 y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
                                                       L["cache_v"][:B].transpose(1, 2), self.kv_len)
                 x = lin(y.transpose(1, 2).reshape(B, 1, c.n_embd), L["c_proj"], residual=x)

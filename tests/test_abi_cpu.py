@@ -216,3 +216,20 @@ def test_greedy_step_argument_checks():
     assert call(stride=999) == _l3lib.L3_ERR_STRIDE
     assert call(pos=FAKE + 2) == _l3lib.L3_ERR_ALIGNMENT
     assert call(ws_bytes=8) == _l3lib.L3_ERR_WORKSPACE
+
+
+def test_linear_qkv_rope_append_argument_checks():
+    lib = _l3lib.load()
+    cs = _l3lib.i64_array((256 * 512, 512))
+
+    def call(table=FAKE, q_out=FAKE, B=1, HD=64, K=2048, strides=cs, norm=None):
+        return lib.l3_linear_qkv_rope_append(FAKE, norm, 1e-5, FAKE, table, q_out, FAKE, FAKE, FAKE, B, 32, 8, HD, K,
+                                             K, K, strides, 256, 16384, None)
+
+    assert call(table=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert call(HD=60) == _l3lib.L3_ERR_SHAPE
+    assert call(B=65) == _l3lib.L3_ERR_SHAPE
+    assert call(K=2040) == _l3lib.L3_ERR_SHAPE
+    assert call(B=12, norm=FAKE) == _l3lib.L3_ERR_SHAPE
+    assert call(strides=_l3lib.i64_array((256 * 512, 516))) == _l3lib.L3_ERR_STRIDE
+    assert call(q_out=FAKE + 8) == _l3lib.L3_ERR_ALIGNMENT

@@ -162,3 +162,40 @@ def test_linear_fused_whole_mlp_and_limits(gpu):
     with pytest.raises(RuntimeError):                                                  # width not a multiple of 512
         cke.linear_decode_fused(randn_bf16((2, 1056), 1).to(gpu), randn_bf16((64, 1056), 2).to(gpu),
                                 norm_weight=randn_bf16((1056,), 3).to(gpu))
+
+
+@pytest.mark.parametrize("B,NH,KVH,HD,K,norm", [(1, 32, 8, 64, 2048, True), (8, 32, 8, 64, 2048, True),
+                                                (16, 32, 8, 64, 2048, False), (3, 8, 2, 128, 512, True),
+                                                (64, 32, 8, 64, 2048, False), (2, 4, 4, 64, 96, False)])
+def test_linear_qkv_rope_append_equals_the_separate_operators(gpu, B, NH, KVH, HD, K, norm):
+    from custom_kernels import custom_kernels_extension as cke
+    from custom_kernels import precompute_freqs_cis
+
+    print(f"linear_qkv_rope_append B={B} NH={NH} KVH={KVH} HD={HD} K={K} norm={norm}", flush=True)
+    L, pos_val = 40, 17
+    x = randn_bf16((B, 1, K), 71).to(gpu)
+    w = randn_bf16(((NH + 2 * KVH) * HD, K), 72, scale=0.05).to(gpu)
+    nw = randn_bf16((K,), 73, scale=0.1, mean=1.0).to(gpu) if norm else None
+    table = precompute_freqs_cis(HD, 64, 500000.0, True, scale_factor=32.0, device=gpu)
+    pos = torch.tensor([pos_val], dtype=torch.int32, device=gpu)
+    base_k = randn_bf16((B + 1, L, KVH, HD), 74).to(gpu)
+    base_v = randn_bf16((B + 1, L, KVH, HD), 75).to(gpu)
+
+    ck1, cv1 = base_k.clone(), base_v.clone()
+    q1 = cke.linear_qkv_rope_append(x, w, table, ck1, cv1, pos, NH, norm_weight=nw, eps=1e-5)
+    ck2, cv2 = base_k.clone(), base_v.clone()
+    qkv = cke.linear_decode_fused(x, w, norm_weight=nw, eps=1e-5) if norm else cke.linear_decode(x, w)
+    q2 = cke.rot_embed_append(qkv, table, ck2, cv2, pos, NH)
+    torch.cuda.synchronize()
+    assert q1.shape == (B, 1, NH, HD)
+    assert torch.equal(q1, q2)
+    assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+    # only token `pos` of the first B cache rows changed
+    changed_k = (ck1 != base_k).any(dim=-1).any(dim=-1)
+    assert changed_k[:B, pos_val].all() and changed_k.sum().item() == B
+    # a position outside the cache writes nothing
+    ck3, cv3 = base_k.clone(), base_v.clone()
+    cke.linear_qkv_rope_append(x, w, table, ck3, cv3, torch.tensor([L], dtype=torch.int32, device=gpu), NH,
+                               norm_weight=nw, eps=1e-5)
+    torch.cuda.synchronize()
+    assert torch.equal(ck3, base_k) and torch.equal(cv3, base_v)
