@@ -398,7 +398,7 @@ def run_prefill(args, torch, lib, l3, dev):
         "config": {"workload": "causal prefill attention: B2 QH32 KVH8 HD64 bf16, 2048 tokens (the 2x2048-token "
                                "prefill of the 1B shape)", "accumulate": "f32", "launch": "hip graph", "seed": SEED},
         "roofline": {"bound": "mfma", "achieved": rec["TFLOPs"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": rec["frac"], "traffic": None, "kernel": "attn_prefill_mfma_kernel",
+                     "frac": rec["frac"], "traffic": None, "kernel": "attn_prefill_tiled_kernel",
                      "algorithmic_flops_per_launch": rec["flops"]},
         "cpu_baseline": cpu, "per_shape": detail,
     }
