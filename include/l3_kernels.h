@@ -200,6 +200,15 @@ int l3_add_rms_norm(const void* x, const void* residual, const void* w, void* su
 int l3_silu_mul(const void* a, const void* b, void* y, int64_t n, void* stream);
 
 /*
+ * l3_silu_mul on row-strided operands: y[r][j] = silu(a[r][j]) * b[r][j] for rows x cols elements,
+ * a and b with the given row strides (elements), y dense.  For the two halves of one fused
+ * gate|up projection (a = first half, b = second half, both strides 2 * cols).  cols and the
+ * strides multiples of 8, pointers 16-byte aligned.
+ */
+int l3_silu_mul_rows(const void* a, const void* b, void* y, int64_t rows, int64_t cols, int64_t a_row_stride,
+                     int64_t b_row_stride, void* stream);
+
+/*
  * y[M, N] = x[M, K] . w[N, K]^T for the few activation rows of a decode step: bf16 in and out,
  * float32 accumulation, one rounding.  Stands where the reference calls nn.Linear with T == 1
  * (model.py:95 c_attn, :121 c_proj, :134 mlp c_proj, :225 lm_head); hipBLASLt treats these as
@@ -252,6 +261,40 @@ int l3_linear_qkv_rope_append(const void* x, const void* norm_weight, float norm
                               const int32_t* pos_dev, int B, int NH, int KVH, int HD, int K, int64_t x_stride,
                               int64_t w_stride, const int64_t cache_strides[2], int cache_len, int table_rows,
                               void* stream);
+
+/*
+ * Split-K form of l3_linear_decode for 17 .. 64 activation rows (hipBLASLt's territory in the
+ * reference: nn.Linear at batch 64, model.py:95,121,134).  Eight wavefronts of a workgroup share
+ * the activations of one k range through LDS and take 128 weight rows; K is split `ksplit` ways
+ * across workgroups, each covering at most 512 k, and split s writes its float32 partial products
+ * to part[s][m][n] (M x N floats per split, contiguous).  The splits are NOT added up here: the
+ * elementwise operator that follows the linear in a decode step does that on its way
+ * (l3_add_rms_norm_partials, l3_rot_embed_append_partials), in split order, without atomics.
+ * l3_linear_splitk_plan returns the split count for a device with num_cus compute units (<= 0: the
+ * current device); l3_linear_splitk_workspace_bytes the size of `part`.  N % 8 == 0, K % 128 == 0,
+ * ceil((K / 128) / ksplit) <= 4; strides and alignment as for l3_linear_decode.
+ */
+int l3_linear_splitk_plan(int N, int K, int num_cus);
+size_t l3_linear_splitk_workspace_bytes(int M, int N, int ksplit);
+int l3_linear_splitk(const void* x, const void* w, void* part, size_t part_bytes, int M, int N, int K,
+                     int64_t x_stride, int64_t w_stride, int ksplit, void* stream);
+
+/*
+ * l3_add_rms_norm whose residual operand is a split-K linear's partial products (`part`,
+ * ksplit x rows x C floats): r = bf16(sum of the splits), sum_out = bf16(x + r),
+ * y = rms_norm(sum_out) -- the bits of the unsplit sequence given the same r.  C % 8 == 0,
+ * C <= 8192; all pointers 16-byte aligned.
+ */
+int l3_add_rms_norm_partials(const void* x, const void* part, int ksplit, const void* w, void* sum_out, void* y,
+                             int rows, int C, float eps, void* stream);
+
+/*
+ * l3_rot_embed_append whose fused qkv projection is a split-K linear's partial products (`part`,
+ * ksplit x B x (NH + 2 KVH) HD floats), added up and rounded to bf16 first.
+ */
+int l3_rot_embed_append_partials(const void* part, int ksplit, const float* freq_table, void* q_out, void* cache_k,
+                                 void* cache_v, const int32_t* pos_dev, int B, int NH, int KVH, int HD,
+                                 const int64_t cache_strides[2], int cache_len, int table_rows, void* stream);
 
 /*
  * out[r] = index of the first maximum of the bf16 row logits[r*row_stride : r*row_stride + V]

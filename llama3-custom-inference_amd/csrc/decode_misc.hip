@@ -15,12 +15,14 @@ constexpr int kMiscThreads = 256;
 
 __global__ void __launch_bounds__(kMiscThreads)
 silu_mul_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ y,
-                int64_t nvec) {
+                int64_t nvec, int64_t vec_per_row, int64_t a_row_stride, int64_t b_row_stride) {
     const int64_t i = int64_t(blockIdx.x) * kMiscThreads + threadIdx.x;
     if (i >= nvec) return;
+    // rows of a and b may be strided (the two halves of one fused gate|up projection); y is dense
+    const int64_t row = i / vec_per_row, col = i % vec_per_row;
     float fa[8], fb[8];
-    unpack8(load16(a + i * 8), fa);
-    unpack8(load16(b + i * 8), fb);
+    unpack8(load16(a + row * a_row_stride + col * 8), fa);
+    unpack8(load16(b + row * b_row_stride + col * 8), fb);
     uint4 o;
     o.x = pack_bf16x2(silu_rounded(fa[0]) * fb[0], silu_rounded(fa[1]) * fb[1]);
     o.y = pack_bf16x2(silu_rounded(fa[2]) * fb[2], silu_rounded(fa[3]) * fb[3]);
@@ -152,11 +154,19 @@ int launch_greedy_step(const uint16_t* logits, int64_t row_stride, int rows, int
     return int(hipGetLastError());
 }
 
+int launch_silu_mul_rows(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t rows, int64_t cols,
+                         int64_t a_row_stride, int64_t b_row_stride, hipStream_t stream) {
+    const int64_t nvec = rows * (cols / 8);
+    hipLaunchKernelGGL(silu_mul_kernel, dim3(unsigned((nvec + kMiscThreads - 1) / kMiscThreads)), dim3(kMiscThreads), 0,
+                       stream, a, b, y, nvec, cols / 8, a_row_stride, b_row_stride);
+    return int(hipGetLastError());
+}
+
 int launch_silu_mul(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n, bool vec_ok, hipStream_t stream) {
     if (vec_ok) {
         const int64_t nvec = n / 8;
         hipLaunchKernelGGL(silu_mul_kernel, dim3(unsigned((nvec + kMiscThreads - 1) / kMiscThreads)),
-                           dim3(kMiscThreads), 0, stream, a, b, y, nvec);
+                           dim3(kMiscThreads), 0, stream, a, b, y, nvec, nvec, int64_t(0), int64_t(0));
     } else {
         hipLaunchKernelGGL(silu_mul_scalar_kernel, dim3(unsigned((n + kMiscThreads - 1) / kMiscThreads)),
                            dim3(kMiscThreads), 0, stream, a, b, y, n);

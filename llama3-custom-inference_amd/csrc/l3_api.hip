@@ -482,6 +482,77 @@ int l3_linear_qkv_rope_append(const void* x, const void* norm_weight, float norm
                               N, false, stream, &t);
 }
 
+int l3_silu_mul_rows(const void* a, const void* b, void* y, int64_t rows, int64_t cols, int64_t a_row_stride,
+                     int64_t b_row_stride, void* stream) {
+    if (!a || !b || !y) return L3_ERR_NULL_POINTER;
+    if (rows <= 0 || cols <= 0 || cols % 8 != 0 || rows * cols >= (int64_t(1) << 38)) return L3_ERR_SHAPE;
+    if (a_row_stride < cols || b_row_stride < cols || a_row_stride % 8 || b_row_stride % 8) return L3_ERR_STRIDE;
+    if (!aligned(a, 16) || !aligned(b, 16) || !aligned(y, 16)) return L3_ERR_ALIGNMENT;
+    return launch_silu_mul_rows(static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b),
+                                static_cast<uint16_t*>(y), rows, cols, a_row_stride, b_row_stride,
+                                static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_linear_splitk_plan(int N, int K, int num_cus) {
+    if (N <= 0 || K <= 0 || K % 128 != 0) return L3_ERR_SHAPE;
+    if (num_cus <= 0) num_cus = current_device_cus();
+    return linear_splitk_plan(N, K, num_cus);
+}
+
+size_t l3_linear_splitk_workspace_bytes(int M, int N, int ksplit) {
+    if (M <= 0 || N <= 0 || ksplit <= 0) return 0;
+    return size_t(ksplit) * size_t(M) * size_t(N) * sizeof(float);
+}
+
+int l3_linear_splitk(const void* x, const void* w, void* part, size_t part_bytes, int M, int N, int K,
+                     int64_t x_stride, int64_t w_stride, int ksplit, void* stream) {
+    if (!x || !w || !part) return L3_ERR_NULL_POINTER;
+    if (M <= 0 || M > L3_LINEAR_MAX_ROWS || N <= 0 || K <= 0 || N % 8 != 0 || K % 128 != 0) return L3_ERR_SHAPE;
+    if (N > (1 << 24) || K > (1 << 24)) return L3_ERR_SHAPE;
+    if (ksplit <= 0 || ksplit > K / 128 || (K / 128 + ksplit - 1) / ksplit > 4) return L3_ERR_SPLITS;
+    if (x_stride < K || w_stride < K || x_stride % 8 || w_stride % 8) return L3_ERR_STRIDE;
+    if (!aligned(x, 16) || !aligned(w, 16) || !aligned(part, 16)) return L3_ERR_ALIGNMENT;
+    if (part_bytes < l3_linear_splitk_workspace_bytes(M, N, ksplit)) return L3_ERR_WORKSPACE;
+    return launch_linear_splitk(static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w),
+                                static_cast<float*>(part), M, N, K, x_stride, w_stride, ksplit,
+                                static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_add_rms_norm_partials(const void* x, const void* part, int ksplit, const void* w, void* sum_out, void* y,
+                             int rows, int C, float eps, void* stream) {
+    if (!x || !part || !w || !sum_out || !y) return L3_ERR_NULL_POINTER;
+    if (rows <= 0 || rows > 65535 || C <= 0 || C % 8 != 0 || C > 8192) return L3_ERR_SHAPE;
+    if (ksplit <= 0 || ksplit > L3_ATTN_MAX_SPLITS) return L3_ERR_SPLITS;
+    if (!aligned(x, 16) || !aligned(part, 16) || !aligned(w, 16) || !aligned(sum_out, 16) || !aligned(y, 16))
+        return L3_ERR_ALIGNMENT;
+    return launch_add_rms_norm_partials(static_cast<const uint16_t*>(x), static_cast<const float*>(part), ksplit,
+                                        int64_t(rows) * C, static_cast<const uint16_t*>(w),
+                                        static_cast<uint16_t*>(sum_out), static_cast<uint16_t*>(y), rows, C, eps,
+                                        static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_rot_embed_append_partials(const void* part, int ksplit, const float* freq_table, void* q_out, void* cache_k,
+                                 void* cache_v, const int32_t* pos_dev, int B, int NH, int KVH, int HD,
+                                 const int64_t cache_strides[2], int cache_len, int table_rows, void* stream) {
+    if (!part || !freq_table || !q_out || !cache_k || !cache_v || !pos_dev || !cache_strides)
+        return L3_ERR_NULL_POINTER;
+    if (B <= 0 || NH <= 0 || KVH <= 0 || HD <= 0 || HD % 8 != 0 || cache_len <= 0 || table_rows <= 0)
+        return L3_ERR_SHAPE;
+    if (int64_t(B) * (NH + 2 * KVH) * (HD / 8) >= (int64_t(1) << 31)) return L3_ERR_SHAPE;
+    if (ksplit <= 0 || ksplit > L3_ATTN_MAX_SPLITS) return L3_ERR_SPLITS;
+    if (cache_strides[0] < 0 || cache_strides[1] < 0 || cache_strides[1] % 8 || (B > 1 && cache_strides[0] % 8))
+        return L3_ERR_STRIDE;
+    if (!aligned(part, 16) || !aligned(q_out, 16) || !aligned(cache_k, 16) || !aligned(cache_v, 16) ||
+        !aligned(freq_table, 16) || !aligned(pos_dev, 4))
+        return L3_ERR_ALIGNMENT;
+    return launch_rot_embed_append_partials(static_cast<const float*>(part), ksplit,
+                                            int64_t(B) * (NH + 2 * KVH) * HD, freq_table,
+                                            static_cast<uint16_t*>(q_out), static_cast<uint16_t*>(cache_k),
+                                            static_cast<uint16_t*>(cache_v), pos_dev, B, NH, KVH, HD, cache_strides[0],
+                                            cache_strides[1], cache_len, table_rows,
+                                            static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
 size_t l3_argmax_workspace_bytes(int rows, int V) {
     if (rows <= 0 || V <= 0) return 0;
     return size_t(rows) * size_t(argmax_parts(V)) * (sizeof(float) + sizeof(int));

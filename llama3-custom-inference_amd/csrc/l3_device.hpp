@@ -101,6 +101,26 @@ __device__ __forceinline__ float wave_max(float x) {
 // 2^x through the hardware v_exp_f32 (inputs here are <= 0 or small; no denormal fix-up).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Sum over the K splits of a split-K linear (float32 partial products part[s][...], element
+// stride split_stride between splits) for 8 consecutive outputs, in split order, rounded to bf16
+// once: what the unsplit linear would have written.
+__device__ __forceinline__ uint4 sum_splits_bf16x8(const float* p, int ksplit, int64_t split_stride) {
+    float4 a = *reinterpret_cast<const float4*>(p);
+    float4 b = *reinterpret_cast<const float4*>(p + 4);
+    for (int s = 1; s < ksplit; ++s) {
+        const float4 c = *reinterpret_cast<const float4*>(p + s * split_stride);
+        const float4 d = *reinterpret_cast<const float4*>(p + s * split_stride + 4);
+        a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
+        b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
+    }
+    uint4 o;
+    o.x = pack_bf16x2(a.x, a.y);
+    o.y = pack_bf16x2(a.z, a.w);
+    o.z = pack_bf16x2(b.x, b.y);
+    o.w = pack_bf16x2(b.z, b.w);
+    return o;
+}
+
 // Rotation of one adjacent bf16 pair (packed in a word) by (cos, sin): the rotary embedding of
 // custom_kernels.cu:400-414, float32 arithmetic, one rounding.
 __device__ __forceinline__ uint32_t rotate_pair(uint32_t xw, float c, float s) {

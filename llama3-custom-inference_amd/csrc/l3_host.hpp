@@ -96,6 +96,16 @@ struct LinearParams {
 // Launchers: return a hipError_t cast to int (0 = success).
 int linear_skinny_plan(int N, int K, int waves_per_wg, int num_cus, int rows_per_wave, int kstep);
 bool linear_skinny_can_stage(int M, int K);
+int linear_splitk_plan(int N, int K, int num_cus);
+int launch_add_rms_norm_partials(const uint16_t* x, const float* part, int ksplit, int64_t split_stride,
+                                 const uint16_t* w, uint16_t* sum_out, uint16_t* y, int rows, int C, float eps,
+                                 hipStream_t stream);
+int launch_rot_embed_append_partials(const float* part, int ksplit, int64_t split_stride, const float* table,
+                                     uint16_t* q_out, uint16_t* cache_k, uint16_t* cache_v, const int* pos_dev, int B,
+                                     int NH, int KVH, int HD, int64_t c_sb, int64_t c_st, int cache_len,
+                                     int table_rows, hipStream_t stream);
+int launch_linear_splitk(const uint16_t* x, const uint16_t* w, float* part, int M, int N, int K, int64_t x_stride,
+                         int64_t w_stride, int ksplit, hipStream_t stream);
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream);
 int launch_attn_prefill(const PrefillParams& p, int HD, hipStream_t stream);        // a wavefront per column group
 constexpr int kPrefillTiledWaves = 8;      // wavefronts per workgroup of the tiled prefill kernel
@@ -109,6 +119,8 @@ int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t r
                     bool vec_ok, hipStream_t stream);
 int launch_add_rms_norm(const uint16_t* x, const uint16_t* res, const uint16_t* w, uint16_t* sum_out, uint16_t* y,
                         int64_t rows, int C, float eps, bool vec_ok, hipStream_t stream);
+int launch_silu_mul_rows(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t rows, int64_t cols,
+                         int64_t a_row_stride, int64_t b_row_stride, hipStream_t stream);
 int launch_silu_mul(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n, bool vec_ok, hipStream_t stream);
 constexpr int kArgmaxChunk = 2048;  // logits one workgroup of the first argmax stage scans
 int argmax_parts(int V);

@@ -1,0 +1,140 @@
+// y[M, N] = x[M, K] . W[N, K]^T for 17 .. 64 activation rows, split over K across workgroups.
+//
+// With this many rows the activation operand of a k step (64 rows x 32 k = 4 KiB) is four times
+// the weight operand of a wavefront (16 rows x 32 k), so the activations must be shared: the eight
+// wavefronts of a workgroup take eight consecutive blocks of 16 weight rows over the SAME k range,
+// the workgroup stages the activations of that range in LDS, and every wavefront reads its B
+// operands from there while its weights come straight from global memory into operand registers.
+// A workgroup covers at most 512 k, so all its loads are requested at once and a single barrier
+// separates staging from arithmetic.  K is split across workgroups (which also gives a matrix
+// with few rows enough workgroups to fill the device): workgroup (row group g, split s) writes
+// the float32 partial products of its k range to part[s][m][n], and whatever elementwise kernel
+// follows the linear in the decode step adds the splits up (residual + norm, SwiGLU product,
+// rotary embedding), in a fixed order, without atomics.
+#include "attn_mfma_core.hpp"
+
+namespace l3 {
+
+namespace {
+
+constexpr int kSplitkWaves = 8;
+constexpr int kSplitkChunk = 128;                    // k per staged activation chunk (4 k steps)
+constexpr int kSplitkPitch = kSplitkChunk * 2 + 16;  // bytes per staged activation row
+constexpr int kSplitkMaxChunks = 4;                  // chunks (of 128 k) one workgroup covers at most
+
+__global__ void __launch_bounds__(kSplitkWaves * kWaveSize)
+linear_splitk_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ part, int M,
+                     int N, int K, int64_t x_stride, int64_t w_stride, int chunks_per_split) {
+    constexpr int NW = kSplitkWaves, KC = kSplitkChunk, PITCH = kSplitkPitch, CB = 4;
+    constexpr int STAGE = 64 * PITCH;
+    __shared__ __align__(16) unsigned char s_x[kSplitkMaxChunks * STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid / kWaveSize;
+    const int fn = lane & 15;
+    const int fg = lane >> 4;
+
+    const int row_groups = (N + 16 * NW - 1) / (16 * NW);
+    const int g = int(blockIdx.x) % row_groups;
+    const int split = int(blockIdx.x) / row_groups;
+    const int n0 = (g * NW + wave) * 16;
+    const int total_chunks = K / KC;
+    const int c0 = split * chunks_per_split;
+    const int c1 = min(total_chunks, c0 + chunks_per_split);
+
+    const int64_t row = min(n0 + fn, N - 1);
+    const uint16_t* wp = w + row * w_stride + fg * 8;
+    constexpr int SPC = KC / 32;        // k steps per chunk
+    constexpr int MAXC = kSplitkMaxChunks;
+    const int nch = c1 - c0;            // 1 .. MAXC chunks, all in flight at once
+
+    // everything this workgroup needs is requested up front: the weights of every k step into
+    // operand registers, the activations of the whole k range into registers and on to LDS
+    uint4 rw[MAXC][SPC];
+#pragma unroll
+    for (int j = 0; j < MAXC; ++j) {
+        if (j < nch) {
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) rw[j][s] = load16(wp + ((c0 + j) * SPC + s) * 32);
+        }
+    }
+    // staging roles: 64 rows x 16 chunks of 16 bytes = 1024 pieces over 512 threads
+    const int st_row = tid / 16, st_col = tid % 16;           // rows st_row and st_row + 32
+    const bool st_valid0 = st_row < M, st_valid1 = st_row + 32 < M;
+    const uint16_t* xs0 = x + int64_t(st_valid0 ? st_row : 0) * x_stride + st_col * 8;
+    const uint16_t* xs1 = x + int64_t(st_valid1 ? st_row + 32 : 0) * x_stride + st_col * 8;
+    uint4 xr[MAXC][2];
+#pragma unroll
+    for (int j = 0; j < MAXC; ++j) {
+        if (j < nch) {
+            xr[j][0] = st_valid0 ? load16(xs0 + (c0 + j) * KC) : make_uint4(0u, 0u, 0u, 0u);
+            xr[j][1] = st_valid1 ? load16(xs1 + (c0 + j) * KC) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < MAXC; ++j) {
+        if (j < nch) {
+            *reinterpret_cast<uint4*>(s_x + j * STAGE + st_row * PITCH + st_col * 16) = xr[j][0];
+            *reinterpret_cast<uint4*>(s_x + j * STAGE + (st_row + 32) * PITCH + st_col * 16) = xr[j][1];
+        }
+    }
+    __syncthreads();
+
+    f32x4_t acc[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) acc[cb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < MAXC; ++j) {
+        if (j < nch) {   // workgroup-uniform
+            const unsigned char* rd = s_x + j * STAGE + fn * PITCH + fg * 16;
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) {
+                const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, rw[j][s]);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const uint4 xv = *reinterpret_cast<const uint4*>(rd + cb * 16 * PITCH + s * 64);
+                    acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, __builtin_bit_cast(bf16x8_t, xv), acc[cb],
+                                                                      0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // acc[cb][r]: weight row n0 + 4*fg + r against activation row cb*16 + fn
+    const int n = n0 + 4 * fg;
+    if (n >= N) return;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        const int m = cb * 16 + fn;
+        if (m < M) {
+            *reinterpret_cast<float4*>(part + (int64_t(split) * M + m) * N + n) =
+                make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
+        }
+    }
+}
+
+}  // namespace
+
+// Splits of K: a workgroup covers 128, 256 or 512 k; the largest of these that still gives about
+// one workgroup per CU (fewer splits mean less partial-product traffic).
+int linear_splitk_plan(int N, int K, int num_cus) {
+    const int row_groups = (N + 16 * kSplitkWaves - 1) / (16 * kSplitkWaves);
+    const int total_chunks = K / kSplitkChunk;
+    int per = kSplitkMaxChunks;
+    while (per > 1 && int64_t(row_groups) * ((total_chunks + per - 1) / per) < (3 * int64_t(num_cus)) / 4) per /= 2;
+    return (total_chunks + per - 1) / per;
+}
+
+int launch_linear_splitk(const uint16_t* x, const uint16_t* w, float* part, int M, int N, int K, int64_t x_stride,
+                         int64_t w_stride, int ksplit, hipStream_t stream) {
+    const int row_groups = (N + 16 * kSplitkWaves - 1) / (16 * kSplitkWaves);
+    const int total_chunks = K / kSplitkChunk;
+    const int chunks_per_split = (total_chunks + ksplit - 1) / ksplit;   // <= kSplitkMaxChunks, checked by the caller
+    hipLaunchKernelGGL(linear_splitk_kernel, dim3(unsigned(row_groups * ksplit)),
+                       dim3(kSplitkWaves * kWaveSize), 0, stream, x, w, part, M, N, K, x_stride, w_stride,
+                       chunks_per_split);
+    return int(hipGetLastError());
+}
+
+}  // namespace l3

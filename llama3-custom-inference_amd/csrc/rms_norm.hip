@@ -120,7 +120,69 @@ rms_norm_generic_kernel(const uint16_t* __restrict__ x, const uint16_t* __restri
     }
 }
 
+// add_rms_norm whose residual operand is the output of a split-K linear that has not been added
+// up yet: r = bf16(sum over splits of part[s][row][:]) first (what the unsplit linear would have
+// written), then exactly the ADD path above.  One workgroup per row (decode steps have few rows);
+// C % 8 == 0 and C / 8 <= 256 * 4.
+__global__ void __launch_bounds__(kRmsThreads)
+add_rms_norm_partials_kernel(const uint16_t* __restrict__ x, const float* __restrict__ part, int ksplit,
+                             int64_t split_stride, const uint16_t* __restrict__ w, uint16_t* __restrict__ sum_out,
+                             uint16_t* __restrict__ y, int C, float eps) {
+    constexpr int MAXV = 4;
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const int nvec = C / 8;
+    uint4 xv[MAXV];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int vi = tid + j * kRmsThreads;
+        if (vi < nvec) {
+            float f[8], r[8];
+            unpack8(load16(x + row * C + vi * 8), f);
+            unpack8(sum_splits_bf16x8(part + row * C + vi * 8, ksplit, split_stride), r);
+            xv[j].x = pack_bf16x2(f[0] + r[0], f[1] + r[1]);
+            xv[j].y = pack_bf16x2(f[2] + r[2], f[3] + r[3]);
+            xv[j].z = pack_bf16x2(f[4] + r[4], f[5] + r[5]);
+            xv[j].w = pack_bf16x2(f[6] + r[6], f[7] + r[7]);
+            store16(sum_out + row * C + vi * 8, xv[j]);
+            unpack8(xv[j], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+        }
+    }
+    ss = wave_sum(ss);
+    __shared__ float s_part[kRmsThreads / kWaveSize];
+    if ((tid & (kWaveSize - 1)) == 0) s_part[tid / kWaveSize] = ss;
+    __syncthreads();
+    ss = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+    const float inv = rsqrtf(ss / float(C) + eps);
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int vi = tid + j * kRmsThreads;
+        if (vi < nvec) {
+            float f[8], g[8];
+            unpack8(xv[j], f);
+            unpack8(load16(w + vi * 8), g);
+            uint4 o;
+            o.x = pack_bf16x2(f[0] * inv * g[0], f[1] * inv * g[1]);
+            o.y = pack_bf16x2(f[2] * inv * g[2], f[3] * inv * g[3]);
+            o.z = pack_bf16x2(f[4] * inv * g[4], f[5] * inv * g[5]);
+            o.w = pack_bf16x2(f[6] * inv * g[6], f[7] * inv * g[7]);
+            store16(y + row * C + vi * 8, o);
+        }
+    }
+}
+
 }  // namespace
+
+int launch_add_rms_norm_partials(const uint16_t* x, const float* part, int ksplit, int64_t split_stride,
+                                 const uint16_t* w, uint16_t* sum_out, uint16_t* y, int rows, int C, float eps,
+                                 hipStream_t stream) {
+    hipLaunchKernelGGL(add_rms_norm_partials_kernel, dim3(unsigned(rows)), dim3(kRmsThreads), 0, stream, x, part,
+                       ksplit, split_stride, w, sum_out, y, C, eps);
+    return int(hipGetLastError());
+}
 
 namespace {
 

@@ -63,8 +63,12 @@ rot_embed_pair_kernel(const uint16_t* __restrict__ x, const float* __restrict__ 
 // in place of two rot_embed calls plus the two cache slice assignments of model.py:100-106;
 // because the position is read on the device the launch can be replayed from a HIP graph.
 // One 16-byte item per thread over (batch, q|k|v head slot, chunk).
+// PART: the fused projection comes as the float32 partial products of a split-K linear
+// (part[s][b][:], `ksplit` splits `split_stride` elements apart) and is added up here first.
+template <bool PART>
 __global__ void __launch_bounds__(kRopeThreads)
-rot_embed_append_kernel(const uint16_t* __restrict__ qkv, const float* __restrict__ table, uint16_t* __restrict__ q_out,
+rot_embed_append_kernel(const uint16_t* __restrict__ qkv, const float* __restrict__ part, int ksplit,
+                        int64_t split_stride, const float* __restrict__ table, uint16_t* __restrict__ q_out,
                         uint16_t* __restrict__ cache_k, uint16_t* __restrict__ cache_v,
                         const int* __restrict__ pos_dev, int total_items, int NH, int KVH, int HD, int64_t qkv_sb,
                         int64_t c_sb, int64_t c_st, int cache_len, int table_rows) {
@@ -77,7 +81,12 @@ rot_embed_append_kernel(const uint16_t* __restrict__ qkv, const float* __restric
     const int c = item % vpr;
     const int slot = (item / vpr) % slots;
     const int b = item / (vpr * slots);
-    const uint4 xv = load16(qkv + b * qkv_sb + slot * HD + c * 8);
+    uint4 xv;
+    if constexpr (PART) {
+        xv = sum_splits_bf16x8(part + b * qkv_sb + slot * HD + c * 8, ksplit, split_stride);
+    } else {
+        xv = load16(qkv + b * qkv_sb + slot * HD + c * 8);
+    }
     if (slot >= NH + KVH) {  // value head: plain copy into the cache
         store16(cache_v + b * c_sb + pos * c_st + (slot - NH - KVH) * HD + c * 8, xv);
         return;
@@ -104,8 +113,21 @@ int launch_rot_embed_append(const uint16_t* qkv, const float* table, uint16_t* q
                             int64_t c_sb, int64_t c_st, int cache_len, int table_rows, hipStream_t stream) {
     const int items = B * (NH + 2 * KVH) * (HD / 8);
     const unsigned blocks = unsigned((items + kRopeThreads - 1) / kRopeThreads);
-    hipLaunchKernelGGL(rot_embed_append_kernel, dim3(blocks), dim3(kRopeThreads), 0, stream, qkv, table, q_out,
-                       cache_k, cache_v, pos_dev, items, NH, KVH, HD, qkv_sb, c_sb, c_st, cache_len, table_rows);
+    hipLaunchKernelGGL(rot_embed_append_kernel<false>, dim3(blocks), dim3(kRopeThreads), 0, stream, qkv, nullptr, 1,
+                       int64_t(0), table, q_out, cache_k, cache_v, pos_dev, items, NH, KVH, HD, qkv_sb, c_sb, c_st,
+                       cache_len, table_rows);
+    return int(hipGetLastError());
+}
+
+int launch_rot_embed_append_partials(const float* part, int ksplit, int64_t split_stride, const float* table,
+                                     uint16_t* q_out, uint16_t* cache_k, uint16_t* cache_v, const int* pos_dev, int B,
+                                     int NH, int KVH, int HD, int64_t c_sb, int64_t c_st, int cache_len,
+                                     int table_rows, hipStream_t stream) {
+    const int items = B * (NH + 2 * KVH) * (HD / 8);
+    const unsigned blocks = unsigned((items + kRopeThreads - 1) / kRopeThreads);
+    hipLaunchKernelGGL(rot_embed_append_kernel<true>, dim3(blocks), dim3(kRopeThreads), 0, stream, nullptr, part,
+                       ksplit, split_stride, table, q_out, cache_k, cache_v, pos_dev, items, NH, KVH, HD,
+                       int64_t(NH + 2 * KVH) * HD, c_sb, c_st, cache_len, table_rows);
     return int(hipGetLastError());
 }
 

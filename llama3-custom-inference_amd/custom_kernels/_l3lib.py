@@ -109,6 +109,29 @@ SIGNATURES = {
          ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_int,
          ctypes.c_void_p],
     ),
+    "l3_silu_mul_rows": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+         ctypes.c_int64, ctypes.c_void_p],
+    ),
+    "l3_linear_splitk_plan": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "l3_linear_splitk_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "l3_linear_splitk": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p],
+    ),
+    "l3_add_rms_norm_partials": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_void_p],
+    ),
+    "l3_rot_embed_append_partials": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int64),
+         ctypes.c_int, ctypes.c_int, ctypes.c_void_p],
+    ),
     "l3_greedy_step": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,

@@ -391,6 +391,23 @@ def silu_mul(a, b):
     _require_gpu_bf16("b", b)
     if tuple(a.shape) != tuple(b.shape):
         raise RuntimeError(f"silu_mul: shapes differ: {tuple(a.shape)} vs {tuple(b.shape)}")
+    C = a.shape[-1] if a.dim() else 1
+    rows = a.numel() // max(C, 1)
+    strided = (a.dim() >= 1 and a.numel() > 0 and C % 8 == 0 and a.stride(-1) == 1 and b.stride(-1) == 1
+               and not (a.is_contiguous() and b.is_contiguous()))
+    if strided:
+        # rows with a stride (the two halves of a fused gate|up projection): no copies
+        a2, b2 = a.reshape(rows, C), b.reshape(rows, C)
+        if a2.stride(1) == 1 and b2.stride(1) == 1 and a2.data_ptr() % 16 == 0 and b2.data_ptr() % 16 == 0 \
+                and a2.stride(0) % 8 == 0 and b2.stride(0) % 8 == 0 and a2.data_ptr() == a.data_ptr() \
+                and b2.data_ptr() == b.data_ptr():
+            y = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+            with torch.cuda.device(a.device):
+                rc = lib.l3_silu_mul_rows(a2.data_ptr(), b2.data_ptr(), y.data_ptr(), rows, C, max(a2.stride(0), C),
+                                          max(b2.stride(0), C), _stream_ptr(a.device))
+            if rc != 0:
+                _fail(rc, f"rows={rows} cols={C}")
+            return y
     ac = a if a.is_contiguous() else a.contiguous()
     bc = b if b.is_contiguous() else b.contiguous()
     y = torch.empty(ac.shape, dtype=ac.dtype, device=ac.device)
@@ -486,6 +503,84 @@ def linear_decode_fused(x, weight, norm_weight=None, eps: float = 1e-5, w_up=Non
     if rc != 0:
         _fail(rc, f"M={rows} N={N} K={K}")
     return y.view(*x.shape[:-1], N)
+
+
+def linear_splitk(x, weight, ksplit: int = 0):
+    """x (..., K) with 17..64 rows times weight (N, K)^T as float32 partial products
+    (ksplit, rows, N) -- NOT added up: hand them to add_rms_norm_partials or
+    rot_embed_append_partials, which sum the splits on their way (or sum them yourself).
+    ksplit 0 lets the library choose.  Stands for nn.Linear at batch sizes where the activations no
+    longer fit one matrix-instruction column block (model.py:95,121,134).  An extension."""
+    lib = _l3lib.load()
+    x2, rows, N, K = _linear_args(x, (weight,))
+    with torch.cuda.device(x.device):
+        if ksplit <= 0:
+            ksplit = lib.l3_linear_splitk_plan(N, K, _cus(x.device))
+            if ksplit < 0:
+                _fail(ksplit, f"N={N} K={K}")
+        part = torch.empty((ksplit, rows, N), dtype=torch.float32, device=x.device)
+        rc = lib.l3_linear_splitk(x2.data_ptr(), weight.data_ptr(), part.data_ptr(), part.numel() * 4, rows, N, K,
+                                  x2.stride(0), weight.stride(0), ksplit, _stream_ptr(x.device))
+    if rc != 0:
+        _fail(rc, f"M={rows} N={N} K={K} ksplit={ksplit}")
+    return part
+
+
+def add_rms_norm_partials(input, part, weight, eps):
+    """add_rms_norm(input, r, weight, eps) with r = bf16(part.sum(0)) formed inside the kernel:
+    ``part`` is linear_splitk's output for the linear whose result is the residual branch
+    (model.py:147-148).  Returns (input + r, rms_norm(input + r))."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("input", input)
+    _require_gpu_bf16("weight", weight)
+    C = input.shape[-1]
+    rows = input.numel() // C
+    if not part.is_cuda or part.dtype != torch.float32 or part.dim() != 3 or not part.is_contiguous() \
+            or tuple(part.shape[1:]) != (rows, C):
+        raise RuntimeError(f"add_rms_norm_partials: partials {tuple(part.shape)} do not fit input {tuple(input.shape)}")
+    if weight.numel() != C or not weight.is_contiguous():
+        raise RuntimeError(f"weight has {weight.numel()} elements, expected {C}")
+    x = input if input.is_contiguous() else input.contiguous()
+    s = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.l3_add_rms_norm_partials(x.data_ptr(), part.data_ptr(), part.shape[0], weight.data_ptr(),
+                                          s.data_ptr(), y.data_ptr(), rows, C, float(eps), _stream_ptr(x.device))
+    if rc != 0:
+        _fail(rc, f"rows={rows} C={C} ksplit={part.shape[0]}")
+    return s, y
+
+
+def rot_embed_append_partials(part, freq_table, cache_k, cache_v, pos, n_head: int):
+    """rot_embed_append on a fused qkv projection that is still in linear_splitk's partial
+    products (ksplit, B, (n_head + 2*KVH)*HD): summed, rounded to bf16, rotated, appended."""
+    lib = _l3lib.load()
+    _require_gpu_bf16("cache_k", cache_k)
+    _require_gpu_bf16("cache_v", cache_v)
+    if cache_k.dim() != 4 or cache_k.shape != cache_v.shape or cache_k.stride() != cache_v.stride():
+        raise RuntimeError("cache_k and cache_v must be (maxB, L, KVH, HD) tensors of the same layout")
+    maxB, L, KVH, HD = cache_k.shape
+    if not part.is_cuda or part.dtype != torch.float32 or part.dim() != 3 or not part.is_contiguous():
+        raise RuntimeError("rot_embed_append_partials: expected contiguous float32 (ksplit, B, N) partials")
+    ksplit, B, N = part.shape
+    if N != (n_head + 2 * KVH) * HD or B > maxB:
+        raise RuntimeError(f"partials {tuple(part.shape)} do not match n_head={n_head}, cache {tuple(cache_k.shape)}")
+    if cache_k.stride(3) != 1 or cache_k.stride(2) != HD:
+        raise RuntimeError("the (KVH, HD) dimensions of the cache must be contiguous")
+    if not freq_table.is_cuda or freq_table.dtype != torch.float32 or freq_table.dim() != 2 \
+            or freq_table.size(1) != HD or not freq_table.is_contiguous():
+        raise RuntimeError("freq_table must be a contiguous (rows, HD) float32 GPU tensor")
+    if not pos.is_cuda or pos.dtype != torch.int32 or pos.numel() != 1:
+        raise RuntimeError("pos must be a one-element int32 GPU tensor")
+    out = torch.empty((B, 1, n_head, HD), dtype=cache_k.dtype, device=part.device)
+    with torch.cuda.device(part.device):
+        rc = lib.l3_rot_embed_append_partials(part.data_ptr(), ksplit, freq_table.data_ptr(), out.data_ptr(),
+                                              cache_k.data_ptr(), cache_v.data_ptr(), pos.data_ptr(), B, n_head, KVH,
+                                              HD, _l3lib.i64_array((cache_k.stride(0), cache_k.stride(1))), L,
+                                              freq_table.size(0), _stream_ptr(part.device))
+    if rc != 0:
+        _fail(rc, f"B={B} NH={n_head} KVH={KVH} HD={HD} ksplit={ksplit}")
+    return out
 
 
 def argmax(logits):

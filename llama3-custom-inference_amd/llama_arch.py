@@ -139,6 +139,32 @@ class LlamaDecoder:
             y = self.ops.flash_attention_decode(q, k, v)
         return y.transpose(1, 2).contiguous().view(B, T, c.n_embd)
 
+    def _splitk(self, rows: int) -> bool:
+        """17..64 activation rows: the split-K linears (activations shared through LDS, splits added
+        up by the operator that follows) stand for F.linear on the three smaller matrices."""
+        return self.decode_linear_rows > 0 and 16 < rows <= 64 and hasattr(self.ops, "linear_splitk")
+
+    def _gate_up(self, L):
+        """c_fc2 and c_fc stacked into one (2 * hidden, C) matrix: one GEMM instead of two."""
+        if "c_fc_cat" not in L:
+            L["c_fc_cat"] = torch.cat([L["c_fc2"], L["c_fc"]], dim=0)
+        return L["c_fc_cat"]
+
+    def _decode_layers_splitk(self, x, append_and_attend):
+        """The layers of one decode step (T == 1) at 17..64 rows; returns the final hidden state.
+        append_and_attend(L, qkv partial products) -> attention output (B, 1, C)."""
+        c, ops = self.config, self.ops
+        H = c.hidden_dim
+        h = ops.rms_norm(x, self.layers[0]["ln_1"], c.norm_eps)
+        for i, L in enumerate(self.layers):
+            y = append_and_attend(L, ops.linear_splitk(h, L["c_attn"]))
+            x, h = ops.add_rms_norm_partials(x, ops.linear_splitk(y, L["c_proj"]), L["ln_2"], c.norm_eps)
+            gu = F.linear(h, self._gate_up(L))
+            t = ops.silu_mul(gu[..., :H], gu[..., H:])
+            next_norm = self.layers[i + 1]["ln_1"] if i + 1 < len(self.layers) else self.ln_f
+            x, h = ops.add_rms_norm_partials(x, ops.linear_splitk(t, L["mlp_proj"]), next_norm, c.norm_eps)
+        return h
+
     def _fused_rows(self) -> int:
         """Rows up to which the decode step uses linear_decode_fused (norms and residual additions
         folded into the linears); 0 when the operator module has no such operator."""
@@ -172,6 +198,17 @@ class LlamaDecoder:
                 t = lin(x, L["c_fc2"], norm_weight=L["ln_2"], eps=c.norm_eps, w_up=L["c_fc"])
                 x = lin(t, L["mlp_proj"], residual=x)
             return lin(x, self.wte, norm_weight=self.ln_f, eps=c.norm_eps).float()
+        if T == 1 and self._splitk(B):
+            pos = torch.tensor([start_pos], dtype=torch.int32, device=self.device)
+
+            def append_and_attend(L, part):
+                q = self.ops.rot_embed_append_partials(part, self.freqs_cis, L["cache_k"], L["cache_v"], pos, c.n_head)
+                y = self.ops.flash_attention_decode(q.transpose(1, 2), L["cache_k"][:B, :start_pos + 1].transpose(1, 2),
+                                                    L["cache_v"][:B, :start_pos + 1].transpose(1, 2))
+                return y.transpose(1, 2).reshape(B, 1, c.n_embd)
+
+            h = self._decode_layers_splitk(x, append_and_attend)
+            return F.linear(h, self.wte).float()
         for L in self.layers:
             x = x + self._attention(L, self.ops.rms_norm(x, L["ln_1"], c.norm_eps), freqs_cis, start_pos)
             h = self.ops.rms_norm(x, L["ln_2"], c.norm_eps)
@@ -317,6 +354,14 @@ class GraphedDecodeLoop:
                 t = lin(x, L["c_fc2"], norm_weight=L["ln_2"], eps=c.norm_eps, w_up=L["c_fc"])
                 x = lin(t, L["mlp_proj"], residual=x)
             logits = lin(x[:, -1], m.wte, norm_weight=m.ln_f, eps=c.norm_eps)
+        elif m._splitk(B):
+            def append_and_attend(L, part):
+                q = ops.rot_embed_append_partials(part, m.freqs_cis, L["cache_k"], L["cache_v"], self.pos, c.n_head)
+                y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
+                                                      L["cache_v"][:B].transpose(1, 2), self.kv_len)
+                return y.transpose(1, 2).reshape(B, 1, c.n_embd)
+
+            logits = F.linear(m._decode_layers_splitk(x, append_and_attend)[:, -1], m.wte)
         else:
             h = ops.rms_norm(x, m.layers[0]["ln_1"], c.norm_eps)
             for i, L in enumerate(m.layers):
@@ -427,7 +472,9 @@ def bench_e2e(args, torch_mod, dev):
         rec["graphed_torch_linear"] = {"tok_per_s": round(best, 1)}
         # ... then the library's weight-streaming linear kernels where they apply (up to 16 rows)
         model.set_decode_linear_rows(16)
-        rec["decode_linear"] = "l3_linear_decode" if 0 < batch <= model.decode_linear_rows else "torch F.linear"
+        rec["decode_linear"] = ("l3_linear_decode (fused)" if 0 < batch <= model.decode_linear_rows else
+                                "l3_linear_splitk for c_attn / c_proj / mlp c_proj, F.linear for gate|up and lm_head"
+                                if model._splitk(batch) else "torch F.linear")
         for mode in ("eager", "graphed"):
             graphed = mode == "graphed"
             # warm-up generate, as llama3_inference.py:31-36 does (for the graphed loop it also records the graph)

@@ -233,3 +233,33 @@ def test_linear_qkv_rope_append_argument_checks():
     assert call(B=12, norm=FAKE) == _l3lib.L3_ERR_SHAPE
     assert call(strides=_l3lib.i64_array((256 * 512, 516))) == _l3lib.L3_ERR_STRIDE
     assert call(q_out=FAKE + 8) == _l3lib.L3_ERR_ALIGNMENT
+
+
+def test_linear_splitk_plan_and_argument_checks():
+    lib = _l3lib.load()
+    # 1B-architecture matrices on a 256-CU device: enough workgroups (128 weight rows x one split each)
+    for (N, K) in ((3072, 2048), (2048, 2048), (2048, 8192), (16384, 2048), (128256, 2048)):
+        ks = lib.l3_linear_splitk_plan(N, K, 256)
+        chunks = K // 128
+        per = -(-chunks // ks)
+        assert 1 <= ks <= chunks and per <= 4
+        assert per == 4 or -(-N // 128) * ks >= 192
+    assert lib.l3_linear_splitk_plan(2048, 2000, 256) == _l3lib.L3_ERR_SHAPE
+    assert lib.l3_linear_splitk_workspace_bytes(64, 2048, 16) == 16 * 64 * 2048 * 4
+
+    def call(M=64, N=2048, K=2048, ks=4, nbytes=1 << 30, part=FAKE):
+        return lib.l3_linear_splitk(FAKE, FAKE, part, nbytes, M, N, K, K, K, ks, None)
+
+    assert call(part=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert call(M=65) == _l3lib.L3_ERR_SHAPE
+    assert call(N=2044) == _l3lib.L3_ERR_SHAPE
+    assert call(ks=2) == _l3lib.L3_ERR_SPLITS          # 1024 k per workgroup
+    assert call(ks=17) == _l3lib.L3_ERR_SPLITS
+    assert call(nbytes=1024) == _l3lib.L3_ERR_WORKSPACE
+    assert lib.l3_add_rms_norm_partials(FAKE, FAKE, 0, FAKE, FAKE, FAKE, 64, 2048, 1e-5, None) == _l3lib.L3_ERR_SPLITS
+    assert lib.l3_add_rms_norm_partials(FAKE, FAKE, 4, FAKE, FAKE, FAKE, 64, 2044, 1e-5, None) == _l3lib.L3_ERR_SHAPE
+    cs = _l3lib.i64_array((256 * 512, 512))
+    assert lib.l3_rot_embed_append_partials(FAKE, 4, FAKE, FAKE, FAKE, None, FAKE, 64, 32, 8, 64, cs, 256, 512, None) \
+        == _l3lib.L3_ERR_NULL_POINTER
+    assert lib.l3_rot_embed_append_partials(FAKE, 4, FAKE, FAKE, FAKE, FAKE, FAKE, 64, 32, 8, 60, cs, 256, 512, None) \
+        == _l3lib.L3_ERR_SHAPE

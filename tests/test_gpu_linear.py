@@ -199,3 +199,83 @@ def test_linear_qkv_rope_append_equals_the_separate_operators(gpu, B, NH, KVH, H
                                norm_weight=nw, eps=1e-5)
     torch.cuda.synchronize()
     assert torch.equal(ck3, base_k) and torch.equal(cv3, base_v)
+
+
+# ---- split-K linear for 17..64 rows and the operators that add its splits up
+def _sum_in_split_order(part):
+    acc = part[0].clone()
+    for s in range(1, part.shape[0]):
+        acc += part[s]
+    return acc
+
+
+@pytest.mark.parametrize("M,N,K,ksplit", [(64, 3072, 2048, 0), (64, 2048, 2048, 0), (64, 2048, 8192, 0), (17, 2048, 2048, 4),
+                                          (40, 264, 384, 1), (33, 8, 128, 1), (64, 16384, 2048, 4), (64, 2048, 2048, 16),
+                                          (20, 1000, 1280, 3)])
+def test_linear_splitk_against_oracle(gpu, M, N, K, ksplit):
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"linear_splitk M={M} N={N} K={K} ksplit={ksplit}", flush=True)
+    x = randn_bf16((M, K), 81)
+    w = randn_bf16((N, K), 82, scale=0.05)
+    part = cke.linear_splitk(x.to(gpu), w.to(gpu), ksplit)
+    torch.cuda.synchronize()
+    assert part.dtype == torch.float32 and part.shape[1:] == (M, N) and (ksplit == 0 or part.shape[0] == ksplit)
+    y = _sum_in_split_order(part).to(torch.bfloat16)
+    assert_linear_close(y, linear_ref(t2f32(x), t2f32(w)), f"splitk {M}x{N}x{K}")
+    # every split alone is the product over its own k range
+    per = -(-(K // 128) // part.shape[0]) * 128
+    s = part.shape[0] - 1
+    ref_last = linear_ref(t2f32(x)[:, s * per:], t2f32(w)[:, s * per:])
+    assert np.abs(part[s].cpu().numpy() - ref_last).max() <= 1e-4 * max(1.0, np.abs(ref_last).max())
+
+
+def test_linear_splitk_errors(gpu):
+    from custom_kernels import custom_kernels_extension as cke
+
+    w = randn_bf16((256, 2048), 1).to(gpu)
+    with pytest.raises(RuntimeError):
+        cke.linear_splitk(randn_bf16((64, 2048), 2).to(gpu), w, 2)        # 1024 k per workgroup: more than it stages
+    with pytest.raises(RuntimeError):
+        cke.linear_splitk(randn_bf16((64, 2048), 2).to(gpu), w, 17)       # more splits than 128-k chunks
+    with pytest.raises(RuntimeError):
+        cke.linear_splitk(randn_bf16((64, 96), 2).to(gpu), randn_bf16((256, 96), 3).to(gpu))   # K % 128 != 0
+    with pytest.raises(RuntimeError):
+        cke.linear_splitk(randn_bf16((65, 2048), 2).to(gpu), w)
+
+
+@pytest.mark.parametrize("rows,C,ksplit", [(64, 2048, 16), (17, 2048, 4), (64, 4096, 8), (3, 8, 1), (5, 8192, 2)])
+def test_add_rms_norm_partials_equals_sum_then_add_rms_norm(gpu, rows, C, ksplit):
+    from custom_kernels import custom_kernels_extension as cke
+
+    x = randn_bf16((rows, 1, C), 91).to(gpu)
+    w = randn_bf16((C,), 92, scale=0.1, mean=1.0).to(gpu)
+    part = (torch.randn((ksplit, rows, C), generator=torch.Generator().manual_seed(93)) * 0.7).to(gpu)
+    s1, y1 = cke.add_rms_norm_partials(x, part, w, 1e-5)
+    r = _sum_in_split_order(part).to(torch.bfloat16).view(rows, 1, C)
+    s2, y2 = cke.add_rms_norm(x, r, w, 1e-5)
+    torch.cuda.synchronize()
+    assert torch.equal(s1, s2)
+    d = bf16_ulp_distance(t2bits(y1), t2bits(y2))     # the two kernels add the squares in different orders
+    assert d.max() <= 1 and (d > 0).mean() < 0.02
+
+
+@pytest.mark.parametrize("B,NH,KVH,HD,ksplit", [(64, 32, 8, 64, 8), (17, 8, 2, 128, 3), (2, 4, 4, 64, 1)])
+def test_rot_embed_append_partials_equals_sum_then_rot_embed_append(gpu, B, NH, KVH, HD, ksplit):
+    from custom_kernels import custom_kernels_extension as cke
+    from custom_kernels import precompute_freqs_cis
+
+    L, pos_val = 24, 11
+    N = (NH + 2 * KVH) * HD
+    part = torch.randn((ksplit, B, N), generator=torch.Generator().manual_seed(95)).to(gpu)
+    table = precompute_freqs_cis(HD, 64, 500000.0, True, scale_factor=32.0, device=gpu)
+    pos = torch.tensor([pos_val], dtype=torch.int32, device=gpu)
+    base_k = randn_bf16((B, L, KVH, HD), 96).to(gpu)
+    base_v = randn_bf16((B, L, KVH, HD), 97).to(gpu)
+    ck1, cv1 = base_k.clone(), base_v.clone()
+    q1 = cke.rot_embed_append_partials(part, table, ck1, cv1, pos, NH)
+    ck2, cv2 = base_k.clone(), base_v.clone()
+    qkv = _sum_in_split_order(part).to(torch.bfloat16).view(B, 1, N)
+    q2 = cke.rot_embed_append(qkv, table, ck2, cv2, pos, NH)
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
