@@ -500,6 +500,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "prefill", "linear", "e2e", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="default workload only: skip the end-to-end tokens/s summary that rides along")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall time spent on the CPU baseline sample")
     ap.add_argument("--e2e-batch", type=int, default=1)
     ap.add_argument("--attn-kernel", default="default", choices=["default", "mfma", "fma"],
@@ -552,6 +554,12 @@ def main():
     line.update(res)
     if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):
         line["config"].update(attn_opts)
+    if args.workload == "c2" and not args.no_e2e and not args.lengths:
+        # the second half of the headline metric: greedy decode tokens/s of the 1B architecture
+        # (128 prompt ids + 128 generated tokens, graph-replayed loop; --workload e2e has the detail)
+        import llama_arch
+
+        line["e2e_tokens_per_s"] = llama_arch.e2e_summary(torch, dev)
     line["device"] = torch.cuda.get_device_name(0)
     print(json.dumps(line), flush=True)
 

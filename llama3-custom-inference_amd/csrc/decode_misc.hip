@@ -101,37 +101,56 @@ argmax_final_kernel(const float* __restrict__ part_val, const int* __restrict__ 
 //   tokens[b, next] = nxt;  tok[b] = nxt (the token fed to the next step)
 //   eos[b] |= !text_mask[b, next] && nxt is a stop token
 // and, once every row is done, pos += 1 and kv_len += 1.  One workgroup handles all rows (a
-// wavefront per row in turn), so the two counters are read by everybody before one thread bumps
+// wavefront per four rows in turn), so the two counters are read by everybody before one thread bumps
 // them.  In a graph-replayed decode step this stands for the second argmax stage plus about a
 // dozen tiny elementwise launches.
-__global__ void __launch_bounds__(kMiscThreads)
+constexpr int kGreedyThreads = 1024;
+constexpr int kGreedyRowsPerPass = 4;   // rows a wavefront takes per pass, loads of all of them in flight together
+__global__ void __launch_bounds__(kGreedyThreads)
 greedy_step_kernel(const float* __restrict__ part_val, const int* __restrict__ part_idx, int nparts, int rows,
                    int64_t* __restrict__ tokens, const uint8_t* __restrict__ text_mask, int64_t total_len,
                    int64_t* __restrict__ tok, int* __restrict__ pos, int* __restrict__ kv_len,
                    uint8_t* __restrict__ eos, const int64_t* __restrict__ stop, int n_stop) {
+    constexpr int NWAVES = kGreedyThreads / kWaveSize;
+    constexpr int RP = kGreedyRowsPerPass;
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int wave = threadIdx.x / kWaveSize;
     const int p0 = *pos;
     const int64_t next = min(int64_t(p0) + 1, total_len - 1);
-    for (int row = wave; row < rows; row += kMiscThreads / kWaveSize) {
-        float v = -INFINITY;
-        int idx = 0x7fffffff;
-        for (int i = lane; i < nparts; i += kWaveSize) {
-            argmax_merge(v, idx, part_val[row * nparts + i], part_idx[row * nparts + i]);
-        }
+    for (int base = wave * RP; base < rows; base += NWAVES * RP) {
+        // everything that is only read first, for all rows of the pass (independent loads) ...
+        float v[RP];
+        int idx[RP];
+        bool keep[RP];
+        int64_t prompt_tok[RP];
 #pragma unroll
-        for (int off = 1; off < kWaveSize; off <<= 1) {
-            argmax_merge(v, idx, __shfl_xor(v, off, kWaveSize), __shfl_xor(idx, off, kWaveSize));
+        for (int j = 0; j < RP; ++j) {
+            const int row = min(base + j, rows - 1);
+            v[j] = -INFINITY;
+            idx[j] = 0x7fffffff;
+            for (int i = lane; i < nparts; i += kWaveSize) {
+                argmax_merge(v[j], idx[j], part_val[row * nparts + i], part_idx[row * nparts + i]);
+            }
+            keep[j] = text_mask[row * total_len + next] != 0;
+            prompt_tok[j] = tokens[row * total_len + next];
         }
-        if (lane == 0) {
-            int64_t nxt = (idx == 0x7fffffff) ? 0 : idx;
-            const bool keep = text_mask[row * total_len + next] != 0;
-            if (keep) nxt = tokens[row * total_len + next];
-            tokens[row * total_len + next] = nxt;
-            tok[row] = nxt;
-            bool is_stop = false;
-            for (int i = 0; i < n_stop; ++i) is_stop |= (stop[i] == nxt);
-            if (!keep && is_stop) eos[row] = 1;
+        // ... then the reductions and the stores
+#pragma unroll
+        for (int j = 0; j < RP; ++j) {
+#pragma unroll
+            for (int off = 1; off < kWaveSize; off <<= 1) {
+                argmax_merge(v[j], idx[j], __shfl_xor(v[j], off, kWaveSize), __shfl_xor(idx[j], off, kWaveSize));
+            }
+            const int row = base + j;
+            if (lane == 0 && row < rows) {
+                int64_t nxt = (idx[j] == 0x7fffffff) ? 0 : idx[j];
+                if (keep[j]) nxt = prompt_tok[j];
+                tokens[row * total_len + next] = nxt;
+                tok[row] = nxt;
+                bool is_stop = false;
+                for (int i = 0; i < n_stop; ++i) is_stop |= (stop[i] == nxt);
+                if (!keep[j] && is_stop) eos[row] = 1;
+            }
         }
     }
     __syncthreads();
@@ -149,7 +168,7 @@ int launch_greedy_step(const uint16_t* logits, int64_t row_stride, int rows, int
     const int parts = argmax_parts(V);
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(unsigned(parts), unsigned(rows)), dim3(kMiscThreads), 0, stream,
                        logits, row_stride, V, kArgmaxChunk, part_val, part_idx);
-    hipLaunchKernelGGL(greedy_step_kernel, dim3(1), dim3(kMiscThreads), 0, stream, part_val, part_idx, parts, rows,
+    hipLaunchKernelGGL(greedy_step_kernel, dim3(1), dim3(kGreedyThreads), 0, stream, part_val, part_idx, parts, rows,
                        tokens, text_mask, total_len, tok, pos, kv_len, eos, stop, n_stop);
     return int(hipGetLastError());
 }

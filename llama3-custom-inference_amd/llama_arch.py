@@ -450,6 +450,25 @@ def timed_generate(model, batch, input_len, gen_len, seed=42, sync=None, graphed
     return gen_len * batch / dt, dt, out
 
 
+def e2e_summary(torch_mod, dev, batches=(1, 64), input_len=128, gen_len=128, repeats=2):
+    """Graph-replayed greedy decode of the end-to-end configuration, tokens/s per batch size (best of
+    `repeats` after one warm-up generation that also records the graph): the short form that rides
+    along with the default attention benchmark."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    out = {}
+    for batch in batches:
+        cfg = LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=batch)
+        model = LlamaDecoder(cfg, cke, dev)
+        timed_generate(model, batch, input_len, gen_len, seed=1, graphed=True)
+        best = max(timed_generate(model, batch, input_len, gen_len, sync=torch_mod.cuda.synchronize, graphed=True)[0]
+                   for _ in range(repeats))
+        out[f"bs{batch}"] = round(best, 1)
+        del model
+        torch_mod.cuda.empty_cache()
+    return out
+
+
 def bench_e2e(args, torch_mod, dev):
     """bench.py --workload e2e: the end-to-end configuration (16 layers, hidden 2048, 32/8 heads, head_dim 64,
     FFN 8192, vocab 128256 tied, N(0, 0.02) weights, 128 random prompt ids + 128 greedy tokens) at
