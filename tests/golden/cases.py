@@ -44,6 +44,22 @@ FREQ_CASES = {
 }
 
 
+PREFILL_CASES = {
+    # name: (B, QH, KVH, T, S, HD, seed)
+    "prompt_r4_hd64": (1, 32, 8, 40, 40, 64, 70),
+    "chunk_after_cache_hd128": (2, 8, 2, 9, 21, 128, 71),         # 9 new tokens on top of 12 cached ones
+    "r1_hd64_t17": (1, 4, 4, 17, 17, 64, 72),
+}
+
+LINEAR_CASES = {
+    # name: (M, N, K, swiglu, seed)
+    "gemv_qkv": (1, 96, 256, False, 80),
+    "rows5": (5, 40, 128, False, 81),
+    "swiglu_rows3": (3, 64, 192, True, 82),
+    "rows40": (40, 24, 384, False, 83),
+}
+
+
 def crc(*arrays) -> int:
     c = 0
     for a in arrays:
@@ -71,3 +87,19 @@ def rope_inputs(name):
 
 def bits_crc(*tensors) -> int:
     return crc(*[t2bits(t) for t in tensors])
+
+
+def prefill_inputs(name):
+    B, QH, KVH, T, S, HD, seed = PREFILL_CASES[name]
+    q = randn_bf16((B, T, QH, HD), seed).transpose(1, 2)
+    k = randn_bf16((B, S, KVH, HD), seed + 100).transpose(1, 2)
+    v = randn_bf16((B, S, KVH, HD), seed + 200).transpose(1, 2)
+    return q, k, v
+
+
+def linear_inputs(name):
+    M, N, K, swiglu, seed = LINEAR_CASES[name]
+    x = randn_bf16((M, K), seed)
+    w = randn_bf16((N, K), seed + 100, scale=0.1)
+    w2 = randn_bf16((N, K), seed + 200, scale=0.1) if swiglu else None
+    return x, w, w2

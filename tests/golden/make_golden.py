@@ -20,8 +20,8 @@ for p in (ROOT, os.path.join(ROOT, "llama3-custom-inference_amd"), os.path.dirna
 
 import cases  # noqa: E402
 from helpers import t2f32  # noqa: E402
-from oracle import (attention_decode_ref, f32_to_bf16_bits, precompute_freqs_cis_ref, rms_norm_ref,  # noqa: E402
-                    rot_embed_ref)
+from oracle import (attention_decode_ref, attention_prefill_ref, f32_to_bf16_bits, linear_ref,  # noqa: E402
+                    precompute_freqs_cis_ref, rms_norm_ref, rot_embed_ref, swiglu_linear_ref)
 
 
 def main():
@@ -46,6 +46,15 @@ def main():
     for name, (HD, factor, positions) in cases.FREQ_CASES.items():
         tab = precompute_freqs_cis_ref(HD, max(positions) + 1, theta=500000.0, use_scaled=True, scale_factor=factor)
         out[f"freq/{name}/rows"] = tab[list(positions)]
+    for name in cases.PREFILL_CASES:
+        q, k, v = cases.prefill_inputs(name)
+        out[f"prefill/{name}/expected_f32"] = attention_prefill_ref(t2f32(q), t2f32(k), t2f32(v)).astype(np.float32)
+        out[f"prefill/{name}/input_crc"] = np.uint32(cases.bits_crc(q, k, v))
+    for name in cases.LINEAR_CASES:
+        x, w, w2 = cases.linear_inputs(name)
+        ref = linear_ref(t2f32(x), t2f32(w)) if w2 is None else swiglu_linear_ref(t2f32(x), t2f32(w), t2f32(w2))
+        out[f"linear/{name}/expected_f32"] = ref.astype(np.float32)
+        out[f"linear/{name}/input_crc"] = np.uint32(cases.bits_crc(*([x, w] + ([w2] if w2 is not None else []))))
     path = os.path.join(HERE, "hot_path_golden.npz")
     np.savez_compressed(path, **out)
     print(f"wrote {path}: {len(out)} arrays, {os.path.getsize(path)} bytes")

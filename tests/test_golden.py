@@ -15,8 +15,8 @@ sys.path.insert(0, os.path.join(HERE, "golden"))
 import cases  # noqa: E402
 from helpers import (assert_attn_close, assert_within_ulps, bf16_bits_to_f32, t2bits, t2f32,  # noqa: E402
                      to_device_like)
-from oracle import (attention_decode_ref, f32_to_bf16_bits, precompute_freqs_cis_ref, rms_norm_ref,  # noqa: E402
-                    rot_embed_ref)
+from oracle import (attention_decode_ref, attention_prefill_ref, f32_to_bf16_bits, linear_ref,  # noqa: E402
+                    precompute_freqs_cis_ref, rms_norm_ref, rot_embed_ref, swiglu_linear_ref)
 
 GOLD = np.load(os.path.join(HERE, "golden", "hot_path_golden.npz"))
 
@@ -44,6 +44,22 @@ def test_oracle_rope_golden(name):
     assert cases.bits_crc(x) == int(GOLD[f"rope/{name}/input_crc"])
     ref = rot_embed_ref(t2f32(x), GOLD[f"rope/{name}/freq"])
     np.testing.assert_array_equal(f32_to_bf16_bits(ref.astype(np.float32)), GOLD[f"rope/{name}/expected_bits"])
+
+
+@pytest.mark.parametrize("name", list(cases.PREFILL_CASES))
+def test_oracle_prefill_golden(name):
+    q, k, v = cases.prefill_inputs(name)
+    assert cases.bits_crc(q, k, v) == int(GOLD[f"prefill/{name}/input_crc"]), "seeded inputs drifted"
+    ref = attention_prefill_ref(t2f32(q), t2f32(k), t2f32(v))
+    np.testing.assert_allclose(ref, GOLD[f"prefill/{name}/expected_f32"], rtol=2e-7, atol=1e-8)
+
+
+@pytest.mark.parametrize("name", list(cases.LINEAR_CASES))
+def test_oracle_linear_golden(name):
+    x, w, w2 = cases.linear_inputs(name)
+    assert cases.bits_crc(*([x, w] + ([w2] if w2 is not None else []))) == int(GOLD[f"linear/{name}/input_crc"])
+    ref = linear_ref(t2f32(x), t2f32(w)) if w2 is None else swiglu_linear_ref(t2f32(x), t2f32(w), t2f32(w2))
+    np.testing.assert_allclose(ref, GOLD[f"linear/{name}/expected_f32"], rtol=2e-7, atol=1e-8)
 
 
 @pytest.mark.parametrize("name", list(cases.FREQ_CASES))
@@ -103,3 +119,33 @@ def test_gpu_rope_golden(gpu, name):
     torch.cuda.synchronize()
     assert out.is_contiguous() and out.shape == x.shape
     assert_within_ulps(out, bf16_bits_to_f32(GOLD[f"rope/{name}/expected_bits"]), 1, what=name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(cases.PREFILL_CASES))
+def test_gpu_prefill_golden(gpu, name):
+    from custom_kernels import custom_kernels_extension as cke
+
+    q, k, v = cases.prefill_inputs(name)
+    out = cke.flash_attention_prefill(q.to(gpu), k.to(gpu), v.to(gpu))
+    torch.cuda.synchronize()
+    assert_attn_close(out, GOLD[f"prefill/{name}/expected_f32"], what=name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(cases.LINEAR_CASES))
+def test_gpu_linear_golden(gpu, name):
+    from custom_kernels import custom_kernels_extension as cke
+
+    x, w, w2 = cases.linear_inputs(name)
+    if w2 is None:
+        y = cke.linear_decode(x.to(gpu), w.to(gpu))
+    else:
+        y = cke.linear_swiglu_decode(x.to(gpu), w.to(gpu), w2.to(gpu))
+    torch.cuda.synchronize()
+    ref = GOLD[f"linear/{name}/expected_f32"].astype(np.float64)
+    got = t2f32(y).astype(np.float64)
+    # 1 bf16 ulp of the result plus the float32 accumulation slack of a cancelling sum; the SwiGLU
+    # form may also flip the rounding of its gate or up factor (one more ulp of that factor)
+    tol = (2.0 ** -7 if w2 is not None else 2.0 ** -8) * np.abs(ref) + 2.0 ** -16 * max(1.0, np.abs(ref).max())
+    assert np.all(np.abs(got - ref) <= tol), f"{name}: max excess {(np.abs(got - ref) - tol).max():.3e}"
