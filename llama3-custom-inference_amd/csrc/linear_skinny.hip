@@ -111,65 +111,62 @@ linear_skinny_kernel(const LinearParams p) {
             }
         }
     };
+    // RMSNorm of the activations into LDS (XLDS).  The workgroup shares the 16-byte chunks of all
+    // rows; K % 512 == 0, so the 64 chunks of a wavefront lie in one row and the row's sum of squares
+    // is a fixed-order sum of per-wavefront parts.  A thread's first chunk stays in registers and
+    // its loads are issued BEFORE the weight ring is filled (loads return in order, and the norm
+    // must not wait behind kilobytes of weights coming from HBM); with more than two rows the
+    // further chunks go through LDS, one at a time, so that the prologue costs few registers.
+    constexpr int NT = NW * kWaveSize;
+    const int KP = p.K + 8;                                // LDS row pitch in elements
+    const int cpr = p.K / 8;                               // chunks per row
+    const int nchunks = p.M * cpr;
+    uint4 xv0 = make_uint4(0u, 0u, 0u, 0u), gv0 = xv0;
+    if constexpr (XLDS) {
+        const int c = int(threadIdx.x);
+        if (c < nchunks) {                                 // wave-uniform
+            xv0 = load16(p.x + int64_t(c / cpr) * p.x_stride + (c % cpr) * 8);
+            gv0 = load16(p.norm_w + (c % cpr) * 8);
+        }
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         if (ks0 + u < ks1) fill(u, ks0 + u);
     }
 
-    const int KP = p.K + 8;                                // LDS row pitch in elements
     if constexpr (XLDS) {
-        // RMSNorm of the activations into LDS while the first weight loads are in flight.  The
-        // workgroup shares the 16-byte chunks of all rows; K % 512 == 0, so the 64 chunks of a
-        // wavefront lie in one row and the row's sum of squares is a fixed-order sum of
-        // per-wavefront parts.
-        constexpr int NT = NW * kWaveSize;
-        constexpr int MAXC = (kXldsMaxElems / 8 + NT - 1) / NT;
         __shared__ float s_part[kXldsMaxElems / 8 / kWaveSize];
-        const int cpr = p.K / 8;                           // chunks per row
-        const int nchunks = p.M * cpr;
         const int parts_per_row = cpr / kWaveSize;
-        uint4 xv[MAXC], gv[MAXC];
-#pragma unroll
-        for (int j = 0; j < MAXC; ++j) {
-            const int c = int(threadIdx.x) + j * NT;
-            if (c < nchunks) {                             // wave-uniform
-                const int r = c / cpr, col = c % cpr;
-                xv[j] = load16(p.x + int64_t(r) * p.x_stride + col * 8);
-                gv[j] = load16(p.norm_w + col * 8);
+        for (int c = int(threadIdx.x), it = 0; c < nchunks; c += NT, ++it) {
+            const int r = c / cpr, col = c % cpr;
+            uint4 v = xv0;
+            if (it > 0) {
+                v = load16(p.x + int64_t(r) * p.x_stride + col * 8);
+                *reinterpret_cast<uint4*>(s_x + r * KP + col * 8) = v;   // raw, re-read by this thread below
             }
-        }
+            float f[8];
+            unpack8(v, f);
+            float ss = 0.f;
 #pragma unroll
-        for (int j = 0; j < MAXC; ++j) {
-            const int c = int(threadIdx.x) + j * NT;
-            if (c < nchunks) {
-                float f[8];
-                unpack8(xv[j], f);
-                float ss = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
-                ss = wave_sum(ss);
-                if (lane == 0) s_part[c / kWaveSize] = ss;
-            }
+            for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+            ss = wave_sum(ss);
+            if (lane == 0) s_part[c / kWaveSize] = ss;
         }
         __syncthreads();
-#pragma unroll
-        for (int j = 0; j < MAXC; ++j) {
-            const int c = int(threadIdx.x) + j * NT;
-            if (c < nchunks) {
-                const int r = c / cpr, col = c % cpr;
-                float ss = 0.f;
-                for (int q = 0; q < parts_per_row; ++q) ss += s_part[r * parts_per_row + q];
-                const float inv = rsqrtf(ss / float(p.K) + p.norm_eps);
-                float f[8], g[8];
-                unpack8(xv[j], f);
-                unpack8(gv[j], g);
-                uint4 o;
-                o.x = pack_bf16x2(f[0] * inv * g[0], f[1] * inv * g[1]);
-                o.y = pack_bf16x2(f[2] * inv * g[2], f[3] * inv * g[3]);
-                o.z = pack_bf16x2(f[4] * inv * g[4], f[5] * inv * g[5]);
-                o.w = pack_bf16x2(f[6] * inv * g[6], f[7] * inv * g[7]);
-                *reinterpret_cast<uint4*>(s_x + r * KP + col * 8) = o;
-            }
+        for (int c = int(threadIdx.x), it = 0; c < nchunks; c += NT, ++it) {
+            const int r = c / cpr, col = c % cpr;
+            float ss = 0.f;
+            for (int q = 0; q < parts_per_row; ++q) ss += s_part[r * parts_per_row + q];
+            const float inv = rsqrtf(ss / float(p.K) + p.norm_eps);
+            float f[8], g[8];
+            unpack8(it == 0 ? xv0 : *reinterpret_cast<const uint4*>(s_x + r * KP + col * 8), f);
+            unpack8(it == 0 ? gv0 : load16(p.norm_w + col * 8), g);
+            uint4 o;
+            o.x = pack_bf16x2(f[0] * inv * g[0], f[1] * inv * g[1]);
+            o.y = pack_bf16x2(f[2] * inv * g[2], f[3] * inv * g[3]);
+            o.z = pack_bf16x2(f[4] * inv * g[4], f[5] * inv * g[5]);
+            o.w = pack_bf16x2(f[6] * inv * g[6], f[7] * inv * g[7]);
+            *reinterpret_cast<uint4*>(s_x + r * KP + col * 8) = o;
         }
         __syncthreads();
     }
