@@ -129,12 +129,7 @@ linear_skinny_kernel(const LinearParams p) {
             gv0 = load16(p.norm_w + (c % cpr) * 8);
         }
     }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        if (ks0 + u < ks1) fill(u, ks0 + u);
-    }
-
-    if constexpr (XLDS) {
+    auto norm_prologue = [&]() {
         __shared__ float s_part[kXldsMaxElems / 8 / kWaveSize];
         const int parts_per_row = cpr / kWaveSize;
         for (int c = int(threadIdx.x), it = 0; c < nchunks; c += NT, ++it) {
@@ -169,6 +164,26 @@ linear_skinny_kernel(const LinearParams p) {
             *reinterpret_cast<uint4*>(s_x + r * KP + col * 8) = o;
         }
         __syncthreads();
+    };
+    // Initial ring fill, then the norm.  The weight loads sit BEHIND the activation loads in the
+    // wavefront's in-order memory queue; when their number is known at compile time (a full ring
+    // or half of one: the common cases) the compiler waits for the activations alone, otherwise
+    // it has to wait for everything.
+    const int nst = ks1 - ks0;
+    if (nst >= U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) fill(u, ks0 + u);
+        if constexpr (XLDS) norm_prologue();
+    } else if (nst == U / 2) {
+#pragma unroll
+        for (int u = 0; u < U / 2; ++u) fill(u, ks0 + u);
+        if constexpr (XLDS) norm_prologue();
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (ks0 + u < ks1) fill(u, ks0 + u);
+        }
+        if constexpr (XLDS) norm_prologue();
     }
     const uint16_t* lx = s_x + (xvalid[0] ? fn % RW : 0) * KP + koff;
 
