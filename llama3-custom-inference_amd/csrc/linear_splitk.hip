@@ -11,6 +11,8 @@
 // the float32 partial products of its k range to part[s][m][n], and whatever elementwise kernel
 // follows the linear in the decode step adds the splits up (residual + norm, SwiGLU product,
 // rotary embedding), in a fixed order, without atomics.
+#include <type_traits>
+
 #include "attn_mfma_core.hpp"
 
 namespace l3 {
@@ -49,35 +51,44 @@ linear_splitk_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
     constexpr int MAXC = kSplitkMaxChunks;
     const int nch = c1 - c0;            // 1 .. MAXC chunks, all in flight at once
 
-    // everything this workgroup needs is requested up front: the weights of every k step into
-    // operand registers, the activations of the whole k range into registers and on to LDS
-    uint4 rw[MAXC][SPC];
-#pragma unroll
-    for (int j = 0; j < MAXC; ++j) {
-        if (j < nch) {
-#pragma unroll
-            for (int s = 0; s < SPC; ++s) rw[j][s] = load16(wp + ((c0 + j) * SPC + s) * 32);
-        }
-    }
+    // Everything this workgroup needs is requested up front: first the activations of the whole k
+    // range (registers, then LDS), behind them the weights of every k step into operand registers.
+    // Loads return in order, so the activations are staged while the weights are still on their
+    // way -- provided the compiler knows how many weight loads follow, hence one copy of the
+    // sequence per chunk count.
     // staging roles: 64 rows x 16 chunks of 16 bytes = 1024 pieces over 512 threads
     const int st_row = tid / 16, st_col = tid % 16;           // rows st_row and st_row + 32
     const bool st_valid0 = st_row < M, st_valid1 = st_row + 32 < M;
     const uint16_t* xs0 = x + int64_t(st_valid0 ? st_row : 0) * x_stride + st_col * 8;
     const uint16_t* xs1 = x + int64_t(st_valid1 ? st_row + 32 : 0) * x_stride + st_col * 8;
+    uint4 rw[MAXC][SPC];
     uint4 xr[MAXC][2];
+    auto request_and_stage = [&](auto count) {
+        constexpr int NCH = decltype(count)::value;
 #pragma unroll
-    for (int j = 0; j < MAXC; ++j) {
-        if (j < nch) {
+        for (int j = 0; j < NCH; ++j) {
             xr[j][0] = st_valid0 ? load16(xs0 + (c0 + j) * KC) : make_uint4(0u, 0u, 0u, 0u);
             xr[j][1] = st_valid1 ? load16(xs1 + (c0 + j) * KC) : make_uint4(0u, 0u, 0u, 0u);
         }
-    }
 #pragma unroll
-    for (int j = 0; j < MAXC; ++j) {
-        if (j < nch) {
+        for (int j = 0; j < NCH; ++j) {
+#pragma unroll
+            for (int s = 0; s < SPC; ++s) rw[j][s] = load16(wp + ((c0 + j) * SPC + s) * 32);
+        }
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
             *reinterpret_cast<uint4*>(s_x + j * STAGE + st_row * PITCH + st_col * 16) = xr[j][0];
             *reinterpret_cast<uint4*>(s_x + j * STAGE + (st_row + 32) * PITCH + st_col * 16) = xr[j][1];
         }
+    };
+    if (nch == 4) {
+        request_and_stage(std::integral_constant<int, 4>{});
+    } else if (nch == 3) {
+        request_and_stage(std::integral_constant<int, 3>{});
+    } else if (nch == 2) {
+        request_and_stage(std::integral_constant<int, 2>{});
+    } else if (nch == 1) {
+        request_and_stage(std::integral_constant<int, 1>{});
     }
     __syncthreads();
 
