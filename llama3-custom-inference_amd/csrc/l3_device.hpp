@@ -107,7 +107,23 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ uint4 sum_splits_bf16x8(const float* p, int ksplit, int64_t split_stride) {
     float4 a = *reinterpret_cast<const float4*>(p);
     float4 b = *reinterpret_cast<const float4*>(p + 4);
-    for (int s = 1; s < ksplit; ++s) {
+    int s = 1;
+    // four splits per round: their loads are independent and go out together, the additions keep
+    // the split order
+    for (; s + 4 <= ksplit; s += 4) {
+        float4 c[4], d[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            c[i] = *reinterpret_cast<const float4*>(p + (s + i) * split_stride);
+            d[i] = *reinterpret_cast<const float4*>(p + (s + i) * split_stride + 4);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a.x += c[i].x; a.y += c[i].y; a.z += c[i].z; a.w += c[i].w;
+            b.x += d[i].x; b.y += d[i].y; b.z += d[i].z; b.w += d[i].w;
+        }
+    }
+    for (; s < ksplit; ++s) {
         const float4 c = *reinterpret_cast<const float4*>(p + s * split_stride);
         const float4 d = *reinterpret_cast<const float4*>(p + s * split_stride + 4);
         a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
