@@ -27,13 +27,17 @@ namespace {
 // through LDS at the end; with a single split per head the workgroup writes the final output and
 // no combine kernel runs.  It trades the contiguous-row access of the streaming form for eight
 // times the parallelism per head, which is what a latency-bound call (a few tiles per head) needs.
-template <int HD, bool COOP>
+// LOADS = 4 (head size 64, cooperative form, at most 512 tokens): half-size tiles of 32 tokens, so
+// that a short sequence still gives every wavefront a tile, and slabs small enough for two
+// workgroups per CU.
+template <int HD, bool COOP, int LOADS = 8>
 __global__ void __launch_bounds__(kMfmaWaves * kWaveSize, 2)
 attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg) {
-    using T = MfmaTile<HD>;
+    using T = MfmaTile<HD, LOADS>;
     constexpr int WT = T::WT, KC = T::KC, NB = T::NB, SLAB = T::SLAB;
     constexpr int STEP = COOP ? kMfmaWaves * WT : WT;  // token stride between a wavefront's tiles
-    static_assert(WT == attn_tile_tokens(HD, kAttnImplMfma), "host plan and kernel tile disagree");
+    static_assert(LOADS != 8 || WT == attn_tile_tokens(HD, kAttnImplMfma), "host plan and kernel tile disagree");
+    static_assert(LOADS == 8 || COOP, "the split plan counts full tiles");
 
     __shared__ __align__(16) unsigned char s_slab[kMfmaWaves][SLAB];
 
@@ -88,8 +92,8 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     for (int nb = 0; nb < NB; ++nb) O[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = kMaskedScore;  // running maximum of the raw scores (common to the four k groups of a head)
     float l_part = 0.f;          // this lane's share of the softmax denominator
-    mfma_tile_loop<HD>(kbase, vbase, p.k_st, p.v_st, s_slab[wave], qfrag, t_begin + (COOP ? wave * WT : 0), t_end,
-                       STEP, t_end, t_end, c, O, m_run, l_part);
+    mfma_tile_loop<HD, LOADS>(kbase, vbase, p.k_st, p.v_st, s_slab[wave], qfrag, t_begin + (COOP ? wave * WT : 0),
+                              t_end, STEP, t_end, t_end, c, O, m_run, l_part);
 
     // ---- this wavefront's result.  O[nb][r] is dim 16*nb + 4*fg + r of head fn; the softmax
     //      denominator is still spread over the four k groups.
@@ -178,7 +182,9 @@ int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipS
     const dim3 block(kMfmaWaves * kWaveSize);
     if (coop) {
         const dim3 grid(unsigned(p.B) * unsigned(p.KVH) * unsigned(p.num_splits));
-        if (HD == 64) {
+        if (HD == 64 && p.tokens_per_split <= 2 * kMfmaWaves * 32) {
+            hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, true, 4>), grid, block, 0, stream, p, R, 1);
+        } else if (HD == 64) {
             hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, true>), grid, block, 0, stream, p, R, 1);
         } else {
             hipLaunchKernelGGL((attn_splitkv_mfma_kernel<128, true>), grid, block, 0, stream, p, R, 1);

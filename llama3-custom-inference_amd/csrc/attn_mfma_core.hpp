@@ -31,11 +31,11 @@ typedef __attribute__((ext_vector_type(8))) short s16x8_t;
 // hardware already executes one wavefront's LDS accesses in order).
 __device__ __forceinline__ void lds_phase_fence() { asm volatile("" ::: "memory"); }
 
-template <int HD>
+template <int HD, int LOADS = 8>
 struct MfmaTile {
     static constexpr int LPR = HD / 8;            // lanes per token row in a global load
     static constexpr int G = kWaveSize / LPR;     // token rows per wavefront-wide load
-    static constexpr int U = 8;                   // loads of K (and of V) per tile and lane
+    static constexpr int U = LOADS;               // loads of K (and of V) per tile and lane (8; 4 = a half tile)
     static constexpr int WT = U * G;              // tokens per wavefront tile: 32 (HD 128) or 64 (HD 64)
     static constexpr int NG = WT / 16;            // 16-token groups per tile (rows of one S tile)
     static constexpr int KC = HD / 32;            // 32-dim chunks of the head dimension
@@ -54,13 +54,14 @@ struct MfmaTile {
 // wave-uniform; tiles below it skip the masking).  On return O[nb][r] is dim 16*nb + 4*fg + r of
 // column fn (unnormalised), m_run the column's running maximum of the raw scores (shared by its
 // four k groups) and l_part this lane's share of the column's softmax denominator.
-template <int HD>
+template <int HD, int LOADS = 8>
 __device__ __forceinline__ void mfma_tile_loop(const uint16_t* kbase, const uint16_t* vbase, int64_t k_st,
                                                int64_t v_st, unsigned char* slab,
                                                const bf16x8_t (&qfrag)[MfmaTile<HD>::KC], int t_first, int t_end,
                                                int step, int col_limit, int col_limit_min, float c,
                                                f32x4_t (&O)[MfmaTile<HD>::NB], float& m_run, float& l_part) {
-    using T = MfmaTile<HD>;
+    using T = MfmaTile<HD, LOADS>;
+    static_assert(T::WT % 32 == 0, "a tile is a whole number of 32-token steps of the second product");
     constexpr int LPR = T::LPR, G = T::G, U = T::U, WT = T::WT, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
     constexpr int KPITCH = T::KPITCH, VPITCH = T::VPITCH;
     const int lane = threadIdx.x & (kWaveSize - 1);
