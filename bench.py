@@ -188,6 +188,25 @@ def run_attention(args, torch, lib, l3, dev, name):
         for c in cases:
             c.launch(slot, sp)
 
+    if args.single_shot:
+        # one eager call per length on cold copies, for use under a profiler (the reference's
+        # --use_ncu mode, benchmark_kernel.py:175-176); no graph, no repetition
+        one_pass(0)
+        torch.cuda.synchronize()
+        detail = []
+        for c in cases:
+            ms = event_time_ms(torch, lambda c=c: c.launch(1, torch.cuda.current_stream().cuda_stream), 1)
+            detail.append({"kv_len": c.S, "splits": c.num_splits, "us": round(ms * 1e3, 3),
+                           "GBps": round(c.bytes / ms / 1e6, 1)})
+        total_ms = sum(d["us"] for d in detail) / 1e3
+        return {
+            "metric": "decode_attn_hbm_GBps", "value": round(pass_bytes / total_ms / 1e6, 1), "unit": "GB/s",
+            "steps": 1, "ms_per_step": round(total_ms, 5), "dtype": "bf16",
+            "config": {"workload": label + " [single shot: one eager call per length, launch latency included]",
+                       "seed": SEED},
+            "roofline": None, "cpu_baseline": None, "per_length": detail,
+        }
+
     passes_per_graph = slots
     graph = capture_graph(torch, lambda: [one_pass(s) for s in range(passes_per_graph)])
 
@@ -500,6 +519,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "prefill", "linear", "e2e", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--single-shot", action="store_true",
+                    help="attention workloads: one eager call per length (for profilers), no graph replay")
     ap.add_argument("--no-e2e", action="store_true",
                     help="default workload only: skip the end-to-end tokens/s summary that rides along")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall time spent on the CPU baseline sample")
@@ -554,7 +575,7 @@ def main():
     line.update(res)
     if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):
         line["config"].update(attn_opts)
-    if args.workload == "c2" and not args.no_e2e and not args.lengths:
+    if args.workload == "c2" and not args.no_e2e and not args.lengths and not args.single_shot:
         # the second half of the headline metric: greedy decode tokens/s of the 1B architecture
         # (128 prompt ids + 128 generated tokens, graph-replayed loop; --workload e2e has the detail)
         import llama_arch
