@@ -5,7 +5,8 @@
 // this but reads split 0's (max, sum) for every split (:184,201,209) and so returns the plain
 // mean of the per-split outputs; here every split contributes its own statistics.
 //
-// One workgroup of eight wavefronts per (batch, query head).  The kernel is short and
+// One workgroup of eight wavefronts per (batch, query head), or four of them (one per quarter
+// of the head dimension) when there are few heads with many splits each.  The kernel is short and
 // latency-bound, so it is built around a single round trip to memory: a wavefront issues the
 // loads of its (max, sum) pairs AND of its partial rows back to back, before it knows any
 // weight, and only then reduces.  Each wavefront merges up to 32 splits per pass with its own
@@ -19,13 +20,17 @@ namespace {
 constexpr int kCombineWaves = 8;
 constexpr int kCombineRows = 32;  // splits a wavefront merges per pass (their loads are all in flight at once)
 
-template <int HD>
+// CG = column groups: with few (batch, query head) pairs the head dimension is dealt to CG
+// workgroups (blockIdx.y), each merging HD / CG columns of every split, so that more than
+// B * QH compute units pull the partial rows.
+template <int HD, int CG>
 __global__ void __launch_bounds__(kCombineWaves * kWaveSize)
 attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
                     uint16_t* __restrict__ out, int QH, int n_rows, int64_t o_sb, int64_t o_sh,
                     const int* __restrict__ seqlen_dev, int tokens_per_split) {
-    constexpr int TPR = HD / 4;             // lanes covering one partial row with float4 loads
-    constexpr int RPL = kWaveSize / TPR;    // rows per wavefront-wide load (2 or 4)
+    constexpr int TPR = HD / CG / 4;        // lanes covering this workgroup's part of a partial row with float4 loads
+    constexpr int RQ = HD / 4;              // float4 per whole partial row
+    constexpr int RPL = kWaveSize / TPR;    // rows per wavefront-wide load (2 to 16)
     constexpr int NLD = kCombineRows / RPL; // row loads per pass
 
     __shared__ float s_m[kCombineWaves];
@@ -40,7 +45,7 @@ attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__
     if (seqlen_dev) n = min(n_rows, max(1, (*seqlen_dev + tokens_per_split - 1) / tokens_per_split));
     const float2* ml = part_ml + int64_t(bq) * n_rows;
     const float4* po = reinterpret_cast<const float4*>(part_o + int64_t(bq) * n_rows * HD);
-    const int dq = lane % TPR;
+    const int dq = int(blockIdx.y) * TPR + lane % TPR;
     const int sub = lane / TPR;
 
     float m_w = kMaskedScore, l_w = 0.f;
@@ -54,7 +59,7 @@ attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__
 #pragma unroll
         for (int u = 0; u < NLD; ++u) {
             const int r = min(r0 + u * RPL + sub, n - 1);  // rows past the end get weight 0 below
-            x[u] = po[int64_t(r) * TPR + dq];
+            x[u] = po[int64_t(r) * RQ + dq];
         }
         const float m_new = fmaxf(m_w, wave_max(st.x));
         const float alpha = fast_exp2(m_w - m_new);
@@ -107,20 +112,28 @@ attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__
         packed.y = pack_bf16x2(t.z * inv, t.w * inv);
         const int b = bq / QH;
         const int qh = bq % QH;
-        *reinterpret_cast<uint2*>(out + b * o_sb + int64_t(qh) * o_sh + threadIdx.x * 4) = packed;
+        *reinterpret_cast<uint2*>(out + b * o_sb + int64_t(qh) * o_sh + (int(blockIdx.y) * TPR + threadIdx.x) * 4) =
+            packed;
     }
 }
 
 }  // namespace
 
 int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream) {
-    const dim3 grid(unsigned(p.B) * unsigned(p.QH));
+    const bool few = int64_t(p.B) * p.QH <= 64 && p.num_splits > kCombineRows;   // few heads, many rows each
+    const dim3 grid(unsigned(p.B) * unsigned(p.QH), few ? 4u : 1u);
     const dim3 block(kCombineWaves * kWaveSize);
-    if (HD == 64) {
-        hipLaunchKernelGGL((attn_combine_kernel<64>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
+    if (HD == 64 && few) {
+        hipLaunchKernelGGL((attn_combine_kernel<64, 4>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
+                           p.num_splits, p.o_sb, p.o_sh, p.seqlen_dev, p.tokens_per_split);
+    } else if (HD == 64) {
+        hipLaunchKernelGGL((attn_combine_kernel<64, 1>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
+                           p.num_splits, p.o_sb, p.o_sh, p.seqlen_dev, p.tokens_per_split);
+    } else if (few) {
+        hipLaunchKernelGGL((attn_combine_kernel<128, 4>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
                            p.num_splits, p.o_sb, p.o_sh, p.seqlen_dev, p.tokens_per_split);
     } else {
-        hipLaunchKernelGGL((attn_combine_kernel<128>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
+        hipLaunchKernelGGL((attn_combine_kernel<128, 1>), grid, block, 0, stream, p.part_o, p.part_ml, p.out, p.QH,
                            p.num_splits, p.o_sb, p.o_sh, p.seqlen_dev, p.tokens_per_split);
     }
     return int(hipGetLastError());
