@@ -378,7 +378,7 @@ def run_prefill(args, torch, lib, l3, dev):
         reps = 8
         forms = {}
         for fname, form in (("auto", l3.L3_ATTN_PREFILL_AUTO), ("wave", l3.L3_ATTN_PREFILL_WAVE),
-                            ("tiled", l3.L3_ATTN_PREFILL_TILED)):
+                            ("tiled", l3.L3_ATTN_PREFILL_TILED), ("pipelined", l3.L3_ATTN_PREFILL_PIPELINED)):
             prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, form)
             cke.flash_attention_prefill(q, k, v)
             gph = capture_graph(torch, lambda: [cke.flash_attention_prefill(q, k, v) for _ in range(reps)])
@@ -398,6 +398,7 @@ def run_prefill(args, torch, lib, l3, dev):
                "TFLOPs": round(flops / ms / 1e9, 1), "frac": round(flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4),
                "flops": flops, "wave_form_us": round(forms["wave"] * 1e3, 2),
                "tiled_form_us": round(forms["tiled"] * 1e3, 2),
+               "pipelined_form_us": round(forms["pipelined"] * 1e3, 2),
                "torch_sdpa_us": None if sd_ms is None else round(sd_ms * 1e3, 2)}
         detail.append(rec)
         if (B, T, HD) == (2, 2048, 64):
@@ -417,7 +418,7 @@ def run_prefill(args, torch, lib, l3, dev):
         "config": {"workload": "causal prefill attention: B2 QH32 KVH8 HD64 bf16, 2048 tokens (the 2x2048-token "
                                "prefill of the 1B shape)", "accumulate": "f32", "launch": "hip graph", "seed": SEED},
         "roofline": {"bound": "mfma", "achieved": rec["TFLOPs"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": rec["frac"], "traffic": None, "kernel": "attn_prefill_tiled_kernel",
+                     "frac": rec["frac"], "traffic": None, "kernel": "attn_prefill_pipe_kernel",
                      "algorithmic_flops_per_launch": rec["flops"]},
         "cpu_baseline": cpu, "per_shape": detail,
     }

@@ -58,7 +58,9 @@ const char* l3_strerror(int code);
  * Split planning depends on the kernel, so choose before sizing workspaces.
  *
  * L3_ATTN_OPT_PREFILL chooses the form of l3_attn_prefill in the same way: AUTO (by prompt
- * length), WAVE (every wavefront streams K/V on its own) or TILED (a workgroup shares K/V tiles).
+ * length: WAVE for short prompts, PIPELINED for long ones), WAVE (every wavefront streams K/V on
+ * its own), TILED (a workgroup shares K/V tiles; a tile's three phases run in turn) or PIPELINED
+ * (the same tiling with the phases of three consecutive tiles interleaved).
  */
 #define L3_ATTN_OPT_KERNEL 0
 #define L3_ATTN_KERNEL_FMA 0
@@ -67,6 +69,7 @@ const char* l3_strerror(int code);
 #define L3_ATTN_PREFILL_AUTO 0
 #define L3_ATTN_PREFILL_WAVE 1
 #define L3_ATTN_PREFILL_TILED 2
+#define L3_ATTN_PREFILL_PIPELINED 3
 int l3_attn_set_option(int option, int value);
 
 /*

@@ -16,11 +16,25 @@
 // issued before the arithmetic on tile i and land in the other LDS buffer after it.
 //
 // Query i of T sits at absolute position S - T + i and attends to tokens 0 .. S - T + i.
+#include <type_traits>
+#include <utility>
+
 #include "attn_mfma_core.hpp"
 
 namespace l3 {
 
 namespace {
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop that is unrolled by
+// construction, with indices that are constant expressions inside the body.
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
 
 template <int HD, int CB, int NW>
 struct PrefillTile {
@@ -260,13 +274,345 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     }
 }
 
+// Software-pipelined form of the kernel above.  The three phases of a tile -- S = K Q^T, the
+// softmax of S, O^T += V^T P -- depend on each other, so a wavefront that runs them in turn
+// leaves the matrix pipe idle during the softmax and the vector pipe idle during the products
+// (and the wavefronts of a workgroup, held in step by the per-tile barrier, do so together).
+// Here iteration `it` multiplies K of tile it, takes the softmax of tile it - 1 and adds tile
+// it - 2 to the output: three independent pieces of work in one basic block, which the
+// scheduler interleaves.  An LDS stage therefore holds K of one tile and V of the tile two
+// before it.  The rescale that a softmax finds is applied to the output accumulators at the
+// start of the NEXT iteration (after the P of tile it - 2, which still refers to the previous
+// maximum, has been added); the two sets of score / probability registers swap roles every
+// iteration, hence the loop unrolled by two.
 template <int HD, int CB, int NW>
-int launch_tiled(const PrefillParams& p, hipStream_t stream) {
+__global__ void __launch_bounds__(NW * kWaveSize)
+attn_prefill_pipe_kernel(const PrefillParams p) {
+    using T = PrefillTile<HD, CB, NW>;
+    constexpr int NT = T::NT, TK = T::TK, LPR = T::LPR, U = T::U, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
+    constexpr int KPITCH = T::KPITCH, VPITCH = T::VPITCH, KBYTES = T::KBYTES, STAGE = T::STAGE;
+    __shared__ __align__(16) unsigned char s_tiles[2 * STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWaveSize - 1);
+    const int wave = tid / kWaveSize;
+    const int fn = lane & 15;
+    const int fg = lane >> 4;
+
+    const int R = p.QH / p.KVH;
+    const int ppw = 16 / R;
+    const int wg_pos = NW * CB * ppw;
+    const int wgs_per_head = (p.T + wg_pos - 1) / wg_pos;
+    const int heads = p.B * p.KVH;
+    const int wg = wgs_per_head - 1 - int(blockIdx.x) / heads;   // longest token ranges first
+    const int bh = int(blockIdx.x) % heads;
+    const int kvh = bh % p.KVH;
+    const int b = bh / p.KVH;
+
+    const int wg_first_qi = wg * wg_pos;
+    const int wg_last_qi = min(p.T, wg_first_qi + wg_pos) - 1;
+    const int wg_t_end = p.S - p.T + wg_last_qi + 1;
+    const int wave_first_qi = wg_first_qi + wave * CB * ppw;
+    const int wave_last_qi = min(p.T, wave_first_qi + CB * ppw) - 1;
+    const int wave_t_end = wave_first_qi < p.T ? p.S - p.T + wave_last_qi + 1 : 0;
+    const int wave_limit_min = p.S - p.T + wave_first_qi + 1;    // tokens below this are seen by every column
+    const int wg_tiles = (wg_t_end + TK - 1) / TK;
+    const int wt = (wave_t_end + TK - 1) / TK;                   // tiles this wavefront works on
+    const int n_it = wg_tiles + 2;                               // workgroup-uniform trip count
+
+    int col_limit[CB];
+    bf16x8_t qfrag[CB][KC];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        const int qi = wave_first_qi + cb * ppw + fn / R;
+        const int qh = kvh * R + fn % R;
+        const bool valid = (fn < ppw * R) && (qi < p.T);
+        col_limit[cb] = valid ? (p.S - p.T + qi + 1) : 0;
+#pragma unroll
+        for (int m = 0; m < KC; ++m) {
+            uint4 qv = make_uint4(0u, 0u, 0u, 0u);
+            if (valid) qv = load16(p.q + b * p.q_sb + int64_t(qh) * p.q_sh + int64_t(qi) * p.q_st + (m * 4 + fg) * 8);
+            qfrag[cb][m] = __builtin_bit_cast(bf16x8_t, qv);
+        }
+    }
+
+    const uint16_t* kbase = p.k + b * p.k_sb + kvh * p.k_sh + (tid % LPR) * 8;
+    const uint16_t* vbase = p.v + b * p.v_sb + kvh * p.v_sh + (tid % LPR) * 8;
+    const int ld_row = tid / LPR;
+    constexpr int ROWS_PER_LOAD = NT / LPR;
+    uint4 kr[U], vr[U];
+    // the stage of iteration `it`: K of tile it, V of tile it - 2 (rows outside the data are
+    // clamped to a valid row and never used)
+    auto issue = [&](int it) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int row = u * ROWS_PER_LOAD + ld_row;
+            const int tok_k = min(it * TK + row, p.S - 1);
+            const int tok_v = min(max((it - 2) * TK + row, 0), p.S - 1);
+            kr[u] = load16(kbase + int64_t(tok_k) * p.k_st);
+            vr[u] = load16(vbase + int64_t(tok_v) * p.v_st);
+        }
+    };
+    auto stash = [&](unsigned char* stage) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int row = u * ROWS_PER_LOAD + ld_row;
+            *reinterpret_cast<uint4*>(stage + row * KPITCH + (tid % LPR) * 16) = kr[u];
+            *reinterpret_cast<uint4*>(stage + KBYTES + row * VPITCH + (tid % LPR) * 16) = vr[u];
+        }
+    };
+
+    f32x4_t O[CB][NB];
+    float m_run[CB], l_part[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        m_run[cb] = kMaskedScore;
+        l_part[cb] = 0.f;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) O[cb][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    const float c = p.scale_log2e;
+    float alpha[CB];   // rescale found by an iteration's softmax; the accumulators meet it at the start of the next
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) alpha[cb] = 1.f;
+
+    static_assert(NG == 4, "the maximum tree below is written for 16 scores per column block and lane");
+    constexpr int GQ = NG * KC;         // LDS operands of the first product (each feeds CB matrix instructions)
+    constexpr int GP = KS * NB;         // LDS operands of the second product
+    constexpr int NM = CB * (GQ + GP);  // matrix instructions per tile
+    constexpr int NE = CB * NG * 4;     // scores per lane and tile
+    constexpr int MS = 11;              // steps of the maximum phase
+
+    // One iteration on its LDS stage.  STEADY: all three phases are live and the softmax tile needs no
+    // causal mask.
+    auto body = [&](auto steady_tag, int it, f32x4_t (&Sprod)[CB][NG], f32x4_t (&Scons)[CB][NG],
+                    uint4 (&Pcons)[CB][KS], uint4 (&Pprod)[CB][KS]) {
+        constexpr bool STEADY = decltype(steady_tag)::value;
+        const unsigned char* stage = s_tiles + (it & 1) * STAGE;
+        const unsigned char* rd_k = stage + fn * KPITCH + fg * 16;
+        const unsigned char* rd_v = stage + KBYTES + (4 * fg + (fn >> 2)) * VPITCH + (lane & 3) * 8;
+        const bool do_qk = STEADY || it < wt;
+        const bool do_sm = STEADY || (it >= 1 && it <= wt);
+        const bool do_pv = STEADY || (it >= 2 && it <= wt + 1);
+
+        // the accumulators (tiles <= it - 3) move to the maximum the previous iteration found; P(it - 2),
+        // added below, already refers to it
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            if (__builtin_amdgcn_ballot_w64(alpha[cb] != 1.f) != 0) {
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) O[cb][nb] *= alpha[cb];
+            }
+            alpha[cb] = 1.f;
+        }
+
+        // ---- the softmax of S(it - 1) as a list of small steps.
+        // Maximum phase: steps 0..7 reduce the lane's 16 scores of each column block with a tree of
+        // three-input maxima, 8 and 9 fold the four k groups of a column, 10 derives the factors.
+        float t1[CB][5], t2[CB][2], mloc[CB], mc[CB], psum[CB];
+        auto sc = [&](int cb, int idx) -> float { return Scons[cb][idx >> 2][idx & 3]; };
+        auto max_step = [&](int k) {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                if (k < 5) t1[cb][k] = fmaxf(fmaxf(sc(cb, 3 * k), sc(cb, 3 * k + 1)), sc(cb, 3 * k + 2));
+                else if (k == 5) t2[cb][0] = fmaxf(fmaxf(t1[cb][0], t1[cb][1]), t1[cb][2]);
+                else if (k == 6) t2[cb][1] = fmaxf(fmaxf(t1[cb][3], t1[cb][4]), sc(cb, 15));
+                else if (k == 7) mloc[cb] = fmaxf(t2[cb][0], t2[cb][1]);
+                else if (k == 8) mloc[cb] = fmaxf(mloc[cb], __shfl_xor(mloc[cb], 16, kWaveSize));
+                else if (k == 9) mloc[cb] = fmaxf(mloc[cb], __shfl_xor(mloc[cb], 32, kWaveSize));
+                else {
+                    const float m_new = fmaxf(m_run[cb], mloc[cb]);
+                    alpha[cb] = fast_exp2((m_run[cb] - m_new) * c);
+                    l_part[cb] *= alpha[cb];
+                    m_run[cb] = m_new;
+                    mc[cb] = m_new * c;
+                    psum[cb] = 0.f;
+                }
+            }
+        };
+        // Exponential phase in half steps: 2e turns score e into 2^(s c - m c), 2e + 1 adds it to the
+        // row sum and, for odd e, packs scores e - 1 and e into a word of P.
+        auto exp_half = [&](int hs) {
+            const int e = hs >> 1;
+            const int cb = e / (NG * 4), tg = (e >> 2) % NG, j = e & 3;
+            if ((hs & 1) == 0) {
+                Scons[cb][tg][j] = fast_exp2(fmaf(Scons[cb][tg][j], c, -mc[cb]));
+            } else {
+                psum[cb] += Scons[cb][tg][j];
+                if (j & 1) {
+                    const uint32_t w = pack_bf16x2(Scons[cb][tg][j - 1], Scons[cb][tg][j]);
+                    uint4& dst = Pprod[cb][tg >> 1];
+                    const int slot = (tg & 1) * 2 + (j >> 1);
+                    if (slot == 0) dst.x = w; else if (slot == 1) dst.y = w; else if (slot == 2) dst.z = w; else dst.w = w;
+                }
+            }
+        };
+        auto mask_scores = [&]() {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+                for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if ((it - 1) * TK + tg * 16 + 4 * fg + j >= col_limit[cb]) Scons[cb][tg][j] = kMaskedScore;
+                    }
+                }
+            }
+        };
+
+        auto qk_mfma = [&](const uint4& a, int g, int cb) {
+            const int tg = g / KC, m = g % KC;
+            const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : Sprod[cb][tg];
+            Sprod[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[cb][m], acc, 0, 0, 0);
+        };
+        auto pv_mfma = [&](const s16x8_t& vv, int h, int cb) {
+            const int ks = h / NB, nb = h % NB;
+            O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv),
+                                                                __builtin_bit_cast(bf16x8_t, Pcons[cb][ks]), O[cb][nb], 0, 0, 0);
+        };
+        auto read_k = [&](int g) {
+            return *reinterpret_cast<const uint4*>(rd_k + (g / KC) * 16 * KPITCH + (g % KC) * 64);
+        };
+        // the k slots of a 32-token step pair (fg, i) with token 4*fg + i of the step's first 16-token
+        // group for i < 4 and of its second group for i >= 4
+        auto read_v = [&](int h) {
+            const int ks = h / NB, nb = h % NB;
+            const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                L3_LDS_PTR(s16x4_t, rd_v + (2 * ks) * 16 * VPITCH + nb * 32));
+            const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                L3_LDS_PTR(s16x4_t, rd_v + (2 * ks + 1) * 16 * VPITCH + nb * 32));
+            return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+
+        if constexpr (STEADY) {
+            // Hand-placed order: O^T += V^T P(it - 2) first, then S(it) = K Q^T, so that the registers of
+            // P(it - 2) and of the exponentiated scores are free when S(it) needs its own.  Every matrix
+            // instruction is followed by the vector work that fits into the cycles it occupies the
+            // matrix pipe; an LDS operand is requested one group ahead.  Nothing moves across the fences.
+            // LDS operands travel through a ring of four register slots, requested three groups ahead.
+            constexpr int AHEAD = 3, PRE = 4;   // PRE: maximum-phase steps taken while the first operands are on their way
+            uint4 ring[AHEAD + 1];
+            auto request = [&](auto gc) {
+                constexpr int g = decltype(gc)::value;
+                if constexpr (g < GP) ring[g % (AHEAD + 1)] = __builtin_bit_cast(uint4, read_v(g));
+                else if constexpr (g < GP + GQ) ring[g % (AHEAD + 1)] = read_k(g - GP);
+            };
+            static_for<AHEAD>([&](auto gc) { request(gc); });
+            static_for<PRE>([&](auto kc) { max_step(decltype(kc)::value); });
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<GP + GQ>([&](auto gc) {
+                constexpr int g = decltype(gc)::value;
+                request(std::integral_constant<int, g + AHEAD>{});
+                static_for<CB>([&](auto cc) {
+                    constexpr int cb = decltype(cc)::value;
+                    constexpr int i = g * CB + cb;   // matrix instruction index
+                    if constexpr (g < GP) pv_mfma(__builtin_bit_cast(s16x8_t, ring[g % (AHEAD + 1)]), g, cb);
+                    else qk_mfma(ring[g % (AHEAD + 1)], g - GP, cb);
+                    if constexpr (i + PRE < MS) {
+                        max_step(i + PRE);
+                    } else {
+                        constexpr int n = NM - (MS - PRE), k = i - (MS - PRE);
+                        constexpr int h0 = k * (2 * NE) / n, h1 = (k + 1) * (2 * NE) / n;
+                        static_for<h1 - h0>([&](auto hc) { exp_half(h0 + decltype(hc)::value); });
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            });
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) l_part[cb] += psum[cb];
+        } else {
+            if (do_sm) {
+                mask_scores();
+#pragma unroll
+                for (int k = 0; k < MS; ++k) max_step(k);
+#pragma unroll
+                for (int hs = 0; hs < 2 * NE; ++hs) exp_half(hs);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) l_part[cb] += psum[cb];
+            }
+            if (do_pv) {
+#pragma unroll
+                for (int h = 0; h < GP; ++h) {
+                    const s16x8_t vv = read_v(h);
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) pv_mfma(vv, h, cb);
+                }
+            }
+            if (do_qk) {
+#pragma unroll
+                for (int g = 0; g < GQ; ++g) {
+                    const uint4 a = read_k(g);
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) qk_mfma(a, g, cb);
+                }
+            }
+        }
+    };
+
+    auto run = [&](int it, f32x4_t (&Sprod)[CB][NG], f32x4_t (&Scons)[CB][NG], uint4 (&Pcons)[CB][KS],
+                   uint4 (&Pprod)[CB][KS]) {
+        const bool more = it + 1 < n_it;   // workgroup-uniform
+        if (more) issue(it + 1);
+        if (it >= 2 && it < wt && it * TK <= wave_limit_min) {
+            body(std::true_type{}, it, Sprod, Scons, Pcons, Pprod);
+        } else {
+            body(std::false_type{}, it, Sprod, Scons, Pcons, Pprod);
+        }
+        // the other stage was last read before the previous barrier: refill it, then meet
+        if (more) stash(s_tiles + ((it + 1) & 1) * STAGE);
+        __syncthreads();
+    };
+
+    issue(0);
+    stash(s_tiles);
+    __syncthreads();
+
+    f32x4_t SA[CB][NG], SB[CB][NG];
+    uint4 PA[CB][KS], PB[CB][KS];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+        for (int tg = 0; tg < NG; ++tg) SA[cb][tg] = SB[cb][tg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) PA[cb][ks] = PB[cb][ks] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    for (int it = 0; it < n_it; it += 2) {
+        run(it, SA, SB, PA, PB);
+        if (it + 1 < n_it) run(it + 1, SB, SA, PB, PA);
+    }
+
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        float l = l_part[cb];
+        l += __shfl_xor(l, 16, kWaveSize);
+        l += __shfl_xor(l, 32, kWaveSize);
+        if (col_limit[cb] > 0) {
+            const int qi = wave_first_qi + cb * ppw + fn / R;
+            const int qh = kvh * R + fn % R;
+            const float inv = 1.0f / l;
+            uint16_t* orow = p.out + b * p.o_sb + int64_t(qh) * p.o_sh + int64_t(qi) * p.o_st + fg * 4;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                uint2 w;
+                w.x = pack_bf16x2(O[cb][nb][0] * inv, O[cb][nb][1] * inv);
+                w.y = pack_bf16x2(O[cb][nb][2] * inv, O[cb][nb][3] * inv);
+                *reinterpret_cast<uint2*>(orow + nb * 16) = w;
+            }
+        }
+    }
+}
+
+template <int HD, int CB, int NW>
+int launch_tiled(const PrefillParams& p, bool pipelined, hipStream_t stream) {
     const int R = p.QH / p.KVH;
     const int wg_pos = NW * CB * (16 / R);
     const int wgs_per_head = (p.T + wg_pos - 1) / wg_pos;
     const dim3 grid(unsigned(p.B) * unsigned(p.KVH) * unsigned(wgs_per_head));
-    hipLaunchKernelGGL((attn_prefill_tiled_kernel<HD, CB, NW>), grid, dim3(NW * kWaveSize), 0, stream, p);
+    if (pipelined) {
+        hipLaunchKernelGGL((attn_prefill_pipe_kernel<HD, CB, NW>), grid, dim3(NW * kWaveSize), 0, stream, p);
+    } else {
+        hipLaunchKernelGGL((attn_prefill_tiled_kernel<HD, CB, NW>), grid, dim3(NW * kWaveSize), 0, stream, p);
+    }
     return int(hipGetLastError());
 }
 
@@ -274,9 +620,9 @@ int launch_tiled(const PrefillParams& p, hipStream_t stream) {
 
 int prefill_tiled_positions_per_wg(int R) { return kPrefillTiledWaves * kPrefillTiledColBlocks * (16 / R); }
 
-int launch_attn_prefill_tiled(const PrefillParams& p, int HD, hipStream_t stream) {
-    if (HD == 64) return launch_tiled<64, kPrefillTiledColBlocks, kPrefillTiledWaves>(p, stream);
-    return launch_tiled<128, kPrefillTiledColBlocks, kPrefillTiledWaves>(p, stream);
+int launch_attn_prefill_tiled(const PrefillParams& p, int HD, bool pipelined, hipStream_t stream) {
+    if (HD == 64) return launch_tiled<64, kPrefillTiledColBlocks, kPrefillTiledWaves>(p, pipelined, stream);
+    return launch_tiled<128, kPrefillTiledColBlocks, kPrefillTiledWaves>(p, pipelined, stream);
 }
 
 }  // namespace l3

@@ -139,7 +139,8 @@ const char* l3_strerror(int code) {
 int l3_attn_set_option(int option, int value) {
     if (option == L3_ATTN_OPT_PREFILL) {
         const int prev_form = g_prefill_form.load(std::memory_order_relaxed);
-        if (value == L3_ATTN_PREFILL_AUTO || value == L3_ATTN_PREFILL_WAVE || value == L3_ATTN_PREFILL_TILED)
+        if (value == L3_ATTN_PREFILL_AUTO || value == L3_ATTN_PREFILL_WAVE || value == L3_ATTN_PREFILL_TILED ||
+            value == L3_ATTN_PREFILL_PIPELINED)
             g_prefill_form.store(value, std::memory_order_relaxed);
         return prev_form;
     }
@@ -306,11 +307,12 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     if (form == L3_ATTN_PREFILL_AUTO) {
         const int wg_pos = prefill_tiled_positions_per_wg(QH / KVH);
         const int64_t tiled_wgs = int64_t(B) * KVH * ((T + wg_pos - 1) / wg_pos);
-        form = (T >= 4 * wg_pos && tiled_wgs >= current_device_cus() / 2) ? L3_ATTN_PREFILL_TILED
+        form = (T >= 4 * wg_pos && tiled_wgs >= current_device_cus() / 2) ? L3_ATTN_PREFILL_PIPELINED
                                                                           : L3_ATTN_PREFILL_WAVE;
     }
-    const int rc = (form == L3_ATTN_PREFILL_TILED) ? launch_attn_prefill_tiled(p, HD, static_cast<hipStream_t>(stream))
-                                                   : launch_attn_prefill(p, HD, static_cast<hipStream_t>(stream));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int rc = (form == L3_ATTN_PREFILL_WAVE) ? launch_attn_prefill(p, HD, st)
+                                                  : launch_attn_prefill_tiled(p, HD, form == L3_ATTN_PREFILL_PIPELINED, st);
     return rc == 0 ? L3_OK : L3_ERR_HIP;
 }
 

@@ -111,7 +111,7 @@ int launch_attn_prefill(const PrefillParams& p, int HD, hipStream_t stream);    
 constexpr int kPrefillTiledWaves = 8;      // wavefronts per workgroup of the tiled prefill kernel
 constexpr int kPrefillTiledColBlocks = 2;  // 16-column blocks per wavefront
 int prefill_tiled_positions_per_wg(int R);
-int launch_attn_prefill_tiled(const PrefillParams& p, int HD, hipStream_t stream);  // K/V tiles shared by a workgroup
+int launch_attn_prefill_tiled(const PrefillParams& p, int HD, bool pipelined, hipStream_t stream);  // K/V tiles shared by a workgroup
 int launch_attn_splitkv_fma(const AttnParams& p, int HD, int R, hipStream_t stream);
 int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipStream_t stream);
 int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream);

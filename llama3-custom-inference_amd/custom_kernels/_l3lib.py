@@ -29,6 +29,7 @@ L3_ATTN_OPT_PREFILL = 1
 L3_ATTN_PREFILL_AUTO = 0
 L3_ATTN_PREFILL_WAVE = 1
 L3_ATTN_PREFILL_TILED = 2
+L3_ATTN_PREFILL_PIPELINED = 3
 
 # name -> (restype, argtypes); mirrors include/l3_kernels.h line by line
 _c_i64p = ctypes.POINTER(ctypes.c_int64)

@@ -44,13 +44,14 @@ def attn_kernel(request):
     lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL, prev)
 
 
-@pytest.fixture(params=["auto", "wave", "tiled"])
+@pytest.fixture(params=["auto", "wave", "tiled", "pipelined"])
 def prefill_form(request):
     """Run a prefill test once per form of the kernel (the library's own choice, and each forced)."""
     from custom_kernels import _l3lib as l3
 
     lib = l3.load()
-    value = {"auto": l3.L3_ATTN_PREFILL_AUTO, "wave": l3.L3_ATTN_PREFILL_WAVE, "tiled": l3.L3_ATTN_PREFILL_TILED}
+    value = {"auto": l3.L3_ATTN_PREFILL_AUTO, "wave": l3.L3_ATTN_PREFILL_WAVE, "tiled": l3.L3_ATTN_PREFILL_TILED,
+             "pipelined": l3.L3_ATTN_PREFILL_PIPELINED}
     prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, value[request.param])
     yield request.param
     lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, prev)

@@ -301,7 +301,7 @@ def test_prefill_against_oracle(gpu, prefill_form, HD, B, QH, KVH, T, S):
 
 
 def test_prefill_forms_agree_on_a_long_prompt(gpu):
-    """2048 tokens (the auto choice is the tiled form): tiled and wavefront-private forms against
+    """2048 tokens (the auto choice is the pipelined form): the tiled forms and the wavefront-private form against
     each other, and sampled rows against the float64 oracle."""
     from custom_kernels import _l3lib as l3
     from custom_kernels import custom_kernels_extension as cke
@@ -315,19 +315,21 @@ def test_prefill_forms_agree_on_a_long_prompt(gpu):
     qd, kd, vd = (t.to(gpu).transpose(1, 2) for t in (q, k, v))
     outs = {}
     for name, form in (("auto", l3.L3_ATTN_PREFILL_AUTO), ("wave", l3.L3_ATTN_PREFILL_WAVE),
-                       ("tiled", l3.L3_ATTN_PREFILL_TILED)):
+                       ("tiled", l3.L3_ATTN_PREFILL_TILED), ("pipelined", l3.L3_ATTN_PREFILL_PIPELINED)):
         print(f"long prefill form={name}", flush=True)
         prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, form)
         try:
             outs[name] = cke.flash_attention_prefill(qd, kd, vd).float().cpu()
         finally:
             lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, prev)
-    assert torch.equal(outs["auto"], outs["tiled"])
+    assert torch.equal(outs["auto"], outs["pipelined"])
     assert (outs["wave"] - outs["tiled"]).abs().max().item() <= 2.0 ** -6
+    assert (outs["pipelined"] - outs["tiled"]).abs().max().item() <= 2.0 ** -6
     for i in (0, 1, 63, 64, 65, 1000, 2047):
         ref = attention_decode_ref(t2f32(q[:, i:i + 1].transpose(1, 2)), t2f32(k[:, :i + 1].transpose(1, 2)),
                                    t2f32(v[:, :i + 1].transpose(1, 2)))
-        assert_attn_close(outs["tiled"][:, :, i:i + 1], ref, what=f"long prefill row {i}")
+        assert_attn_close(outs["tiled"][:, :, i:i + 1], ref, what=f"long prefill row {i} (tiled)")
+        assert_attn_close(outs["pipelined"][:, :, i:i + 1], ref, what=f"long prefill row {i} (pipelined)")
 
 
 def test_prefill_last_row_equals_decode(gpu):

@@ -55,7 +55,7 @@ def _draw_prefill_cases(n, seed):
         B = int(rng.integers(1, 4))
         T = int(rng.choice((int(rng.integers(2, 40)), int(rng.integers(40, 300)), int(rng.integers(300, 700)))))
         past = int(rng.choice((0, 0, 1, 50, 130)))          # tokens already in the cache
-        form = str(rng.choice(("auto", "wave", "tiled")))
+        form = str(rng.choice(("auto", "wave", "tiled", "pipelined")))
         cases.append((i, B, R * KVH, KVH, T, T + past, HD, form))
     return cases
 
@@ -71,7 +71,8 @@ def test_prefill_attention_random_shapes(gpu, case):
     k = randn_bf16((B, S, KVH, HD), 3000 + i)
     v = randn_bf16((B, S, KVH, HD), 4000 + i)
     lib = l3.load()
-    value = {"auto": l3.L3_ATTN_PREFILL_AUTO, "wave": l3.L3_ATTN_PREFILL_WAVE, "tiled": l3.L3_ATTN_PREFILL_TILED}[form]
+    value = {"auto": l3.L3_ATTN_PREFILL_AUTO, "wave": l3.L3_ATTN_PREFILL_WAVE, "tiled": l3.L3_ATTN_PREFILL_TILED,
+             "pipelined": l3.L3_ATTN_PREFILL_PIPELINED}[form]
     prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, value)
     try:
         out = cke.flash_attention_prefill(*(t.to(gpu).transpose(1, 2) for t in (q, k, v)))
