@@ -39,8 +39,8 @@ FORCE_SPLITS = 0        # --splits
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (summaries and the copy-kernel calibration are in profiles/); keyed by (workload, kernel).
 MEASURED_TRAFFIC = {
-    # profiles/attn_splitkv_mfma_c2_sweep_hbm_traffic.md: 38.22 MB fetched + 2.51 MB written per launch
-    ("c2", "attn_splitkv_mfma_kernel"): 40730000,
+    # profiles/attn_splitkv_mfma_c2_sweep_hbm_traffic.md: 38.21 MB fetched + 2.47 MB written per launch
+    ("c2", "attn_splitkv_mfma_kernel"): 40680000,
 }
 
 
@@ -426,8 +426,8 @@ def run_prefill(args, torch, lib, l3, dev):
 
 def run_linear(args, torch, lib, l3, dev):
     """The nn.Linear calls of one decode step of the 1B architecture (model.py:95,121,134,225) at
-    batch 1 and 64 through l3_linear_decode / l3_linear_swiglu_decode: a stream over the weight
-    matrix, priced against HBM.  Each shape owns enough weight copies that the Infinity Cache
+    batch 1 (l3_linear_decode / l3_linear_swiglu_decode) and 64 (l3_linear_splitk + finish for the
+    three matrices of a few thousand rows): a stream over the weight matrix, priced against HBM.  Each shape owns enough weight copies that the Infinity Cache
     cannot hold them; stock F.linear (hipBLASLt) on the same tensors is timed beside it."""
     import torch.nn.functional as F
     from custom_kernels import custom_kernels_extension as cke
@@ -449,8 +449,14 @@ def run_linear(args, torch, lib, l3, dev):
                 run_l3 = lambda: [cke.linear_swiglu_decode(x, a, b) for a, b in zip(ws, ws2)]  # noqa: E731
                 run_t = lambda: [F.silu(F.linear(x, a)) * F.linear(x, b) for a, b in zip(ws, ws2)]  # noqa: E731
             else:
+                # up to 16 rows: l3_linear_decode; 64 rows: l3_linear_splitk + l3_linear_splitk_finish
                 run_l3 = lambda: [cke.linear_decode(x, a) for a in ws]  # noqa: E731
                 run_t = lambda: [F.linear(x, a) for a in ws]  # noqa: E731
+            # At 64 rows the SwiGLU pair and the vocabulary projection stay with the library GEMM (as in the
+            # end-to-end harness): their rows alone fill the device, so splitting K only adds traffic.
+            library = M > 16 and (swiglu or N > 32768)
+            if library:
+                run_l3 = run_t
             run_l3()
             gph = capture_graph(torch, run_l3)
             gph.replay()
@@ -464,7 +470,10 @@ def run_linear(args, torch, lib, l3, dev):
             nbytes = wbytes + M * K * 2 + M * N * 2
             detail.append({"M": M, "layer": name, "N": N, "K": K, "us": round(ms * 1e3, 2),
                            "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
-                           "bytes": nbytes, "torch_us": round(tms * 1e3, 2)})
+                           "bytes": nbytes, "torch_us": round(tms * 1e3, 2),
+                           "path": "F.linear (library GEMM)" if library else
+                                   ("l3_linear_splitk + l3_linear_splitk_finish" if M > 16 else
+                                    ("l3_linear_swiglu_decode" if swiglu else "l3_linear_decode"))})
             per_token = 1 if name == "lm_head" else 16
             total_us += ms * 1e3 * per_token
             torch_us += tms * 1e3 * per_token

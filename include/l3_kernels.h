@@ -216,11 +216,12 @@ int l3_silu_mul_rows(const void* a, const void* b, void* y, int64_t rows, int64_
  * float32 accumulation, one rounding.  Stands where the reference calls nn.Linear with T == 1
  * (model.py:95 c_attn, :121 c_proj, :134 mlp c_proj, :225 lm_head); hipBLASLt treats these as
  * GEMMs, this entry point as a single pass over the weight matrix at HBM speed.
- * 1 <= M <= L3_LINEAR_MAX_ROWS; N % 4 == 0; K % 32 == 0; strides are row strides in elements
+ * 1 <= M <= L3_LINEAR_MAX_ROWS (one 16-column block of the matrix instruction; more rows:
+ * l3_linear_splitk); N % 4 == 0; K % 32 == 0; strides are row strides in elements
  * (x_stride, w_stride >= K and multiples of 8; y_stride >= N and a multiple of 4); x and w
  * 16-byte aligned, y 8-byte aligned.  Needs no workspace.
  */
-#define L3_LINEAR_MAX_ROWS 64
+#define L3_LINEAR_MAX_ROWS 16
 int l3_linear_decode(const void* x, const void* w, void* y, int M, int N, int K, int64_t x_stride,
                      int64_t w_stride, int64_t y_stride, void* stream);
 
@@ -241,7 +242,7 @@ int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up,
  *   t = w_up ? bf16(silu(bf16(h.w^T))) * bf16(h.w_up^T) : h.w^T                   (model.py:134)
  *   y = residual ? bf16(residual + bf16(t)) : bf16(t)                             (model.py:147-148)
  * with the rounding points of the separate operators.  residual has y's shape and row stride and
- * may be y itself.  The input norm stages x in LDS and needs M <= 16, K % 512 == 0 and M * (K + 8) <= 24576
+ * may be y itself.  The input norm stages x in LDS and needs K % 512 == 0 and M * (K + 8) <= 24576
  * (L3_ERR_SHAPE otherwise); everything else as for l3_linear_decode.
  */
 int l3_linear_decode_fused(const void* x, const void* norm_weight, float norm_eps, const void* w, const void* w_up,
@@ -272,15 +273,29 @@ int l3_linear_qkv_rope_append(const void* x, const void* norm_weight, float norm
  * across workgroups, each covering at most 512 k, and split s writes its float32 partial products
  * to part[s][m][n] (M x N floats per split, contiguous).  The splits are NOT added up here: the
  * elementwise operator that follows the linear in a decode step does that on its way
- * (l3_add_rms_norm_partials, l3_rot_embed_append_partials), in split order, without atomics.
+ * (l3_add_rms_norm_partials, l3_rot_embed_append_partials), in split order, without atomics;
+ * l3_linear_splitk_finish does it where there is no such operator.
  * l3_linear_splitk_plan returns the split count for a device with num_cus compute units (<= 0: the
- * current device); l3_linear_splitk_workspace_bytes the size of `part`.  N % 8 == 0, K % 128 == 0,
- * ceil((K / 128) / ksplit) <= 4; strides and alignment as for l3_linear_decode.
+ * current device); l3_linear_splitk_workspace_bytes the size of `part`.  1 <= M <=
+ * L3_LINEAR_SPLITK_MAX_ROWS, N % 8 == 0, K % 128 == 0, ceil((K / 128) / ksplit) <= 4; strides and
+ * alignment as for l3_linear_decode.  Meant for matrices of a few thousand rows, where the split
+ * count fills the device; for a matrix whose rows alone do (a vocabulary projection), every split
+ * costs M x N floats of traffic and a library GEMM is the better tool.
  */
+#define L3_LINEAR_SPLITK_MAX_ROWS 64
 int l3_linear_splitk_plan(int N, int K, int num_cus);
 size_t l3_linear_splitk_workspace_bytes(int M, int N, int ksplit);
 int l3_linear_splitk(const void* x, const void* w, void* part, size_t part_bytes, int M, int N, int K,
                      int64_t x_stride, int64_t w_stride, int ksplit, void* stream);
+
+/*
+ * y[m][n] = bf16(sum over the splits of part[s][m][n]), or bf16(residual + that) with the two
+ * roundings of a separate addition when residual (same shape and row stride as y, may be y) is not
+ * NULL: finishes l3_linear_splitk on its own.  N % 8 == 0, y_stride >= N and a multiple of 8,
+ * pointers 16-byte aligned.
+ */
+int l3_linear_splitk_finish(const void* part, int ksplit, const void* residual, void* y, int M, int N,
+                            int64_t y_stride, void* stream);
 
 /*
  * l3_add_rms_norm whose residual operand is a split-K linear's partial products (`part`,

@@ -509,7 +509,7 @@ size_t l3_linear_splitk_workspace_bytes(int M, int N, int ksplit) {
 int l3_linear_splitk(const void* x, const void* w, void* part, size_t part_bytes, int M, int N, int K,
                      int64_t x_stride, int64_t w_stride, int ksplit, void* stream) {
     if (!x || !w || !part) return L3_ERR_NULL_POINTER;
-    if (M <= 0 || M > L3_LINEAR_MAX_ROWS || N <= 0 || K <= 0 || N % 8 != 0 || K % 128 != 0) return L3_ERR_SHAPE;
+    if (M <= 0 || M > L3_LINEAR_SPLITK_MAX_ROWS || N <= 0 || K <= 0 || N % 8 != 0 || K % 128 != 0) return L3_ERR_SHAPE;
     if (N > (1 << 24) || K > (1 << 24)) return L3_ERR_SHAPE;
     if (ksplit <= 0 || ksplit > K / 128 || (K / 128 + ksplit - 1) / ksplit > 4) return L3_ERR_SPLITS;
     if (x_stride < K || w_stride < K || x_stride % 8 || w_stride % 8) return L3_ERR_STRIDE;
@@ -518,6 +518,18 @@ int l3_linear_splitk(const void* x, const void* w, void* part, size_t part_bytes
     return launch_linear_splitk(static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w),
                                 static_cast<float*>(part), M, N, K, x_stride, w_stride, ksplit,
                                 static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_linear_splitk_finish(const void* part, int ksplit, const void* residual, void* y, int M, int N,
+                            int64_t y_stride, void* stream) {
+    if (!part || !y) return L3_ERR_NULL_POINTER;
+    if (M <= 0 || M > L3_LINEAR_SPLITK_MAX_ROWS || N <= 0 || N % 8 != 0 || N > (1 << 24)) return L3_ERR_SHAPE;
+    if (ksplit <= 0 || ksplit > L3_ATTN_MAX_SPLITS) return L3_ERR_SPLITS;
+    if (y_stride < N || y_stride % 8) return L3_ERR_STRIDE;
+    if (!aligned(part, 16) || !aligned(y, 16) || (residual && !aligned(residual, 16))) return L3_ERR_ALIGNMENT;
+    return launch_linear_splitk_finish(static_cast<const float*>(part), ksplit, static_cast<const uint16_t*>(residual),
+                                       static_cast<uint16_t*>(y), M, N, y_stride,
+                                       static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 
 int l3_add_rms_norm_partials(const void* x, const void* part, int ksplit, const void* w, void* sum_out, void* y,

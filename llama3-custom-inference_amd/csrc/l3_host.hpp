@@ -106,6 +106,8 @@ int launch_rot_embed_append_partials(const float* part, int ksplit, int64_t spli
                                      int table_rows, hipStream_t stream);
 int launch_linear_splitk(const uint16_t* x, const uint16_t* w, float* part, int M, int N, int K, int64_t x_stride,
                          int64_t w_stride, int ksplit, hipStream_t stream);
+int launch_linear_splitk_finish(const float* part, int ksplit, const uint16_t* res, uint16_t* y, int M, int N,
+                                int64_t y_stride, hipStream_t stream);
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream);
 int launch_attn_prefill(const PrefillParams& p, int HD, hipStream_t stream);        // a wavefront per column group
 constexpr int kPrefillTiledWaves = 8;      // wavefronts per workgroup of the tiled prefill kernel

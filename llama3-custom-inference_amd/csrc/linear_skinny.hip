@@ -1,4 +1,4 @@
-// y[M, N] = x[M, K] . W[N, K]^T for the few rows of a decode step (M <= 64), bf16 in and out,
+// y[M, N] = x[M, K] . W[N, K]^T for the few rows of a decode step (M <= 16), bf16 in and out,
 // float32 accumulation: the nn.Linear calls of model.py:95,121,134,225 when T == 1.  With so few
 // rows the product is a stream over the weight matrix, so the kernel is built like the attention
 // kernels: HBM-bound, every weight byte read once, 16-byte loads kept in flight.
@@ -306,171 +306,6 @@ linear_skinny_kernel(const LinearParams p) {
     }
 }
 
-// 17 .. 64 activation rows: four 16-column blocks per matrix instruction row block, and RB blocks
-// of 16 weight rows per wavefront, so that an activation operand fetched from cache is used RB
-// times (with one block of weight rows the activations would be re-read four times as often as
-// weight bytes arrive).  Activations come straight from global memory (they stay in cache); the
-// sk wavefronts of a row group add up in LDS one (matrix, row block) at a time.
-template <int NW, int RB, int U, bool SWIGLU>
-__global__ void __launch_bounds__(NW * kWaveSize)
-linear_wide_kernel(const LinearParams p) {
-    constexpr int ACC = SWIGLU ? 2 : 1;
-    constexpr int CB = 4;
-    __shared__ float s_red[NW][CB][256];
-
-    const int lane = threadIdx.x & (kWaveSize - 1);
-    const int wave = threadIdx.x / kWaveSize;
-    const int fn = lane & 15;
-    const int fg = lane >> 4;
-
-    const int sk = p.sk;
-    const int rg = int(blockIdx.x) * (NW / sk) + wave / sk;   // group of 16 * RB weight rows
-    const int kslice = wave % sk;
-    const int n0 = rg * 16 * RB;
-    const int ksteps = p.K / 32;
-    const int kpw = (ksteps + sk - 1) / sk;
-    const int ks0 = kslice * kpw;
-    const int ks1 = min(ksteps, ks0 + kpw);
-
-    const uint16_t* wp[ACC][RB];
-#pragma unroll
-    for (int j = 0; j < RB; ++j) {
-        const int64_t row = min(n0 + j * 16 + fn, p.N - 1);   // rows past N are loaded clamped and never stored
-        wp[0][j] = p.w0 + row * p.w_stride + fg * 8;
-        if constexpr (SWIGLU) wp[ACC - 1][j] = p.w1 + row * p.w_stride + fg * 8;
-    }
-    const uint16_t* xp[CB];
-    bool xvalid[CB];
-#pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-        xvalid[cb] = cb * 16 + fn < p.M;
-        xp[cb] = p.x + int64_t(xvalid[cb] ? cb * 16 + fn : 0) * p.x_stride + fg * 8;
-    }
-
-    f32x4_t acc[ACC][RB][CB];
-#pragma unroll
-    for (int a = 0; a < ACC; ++a) {
-#pragma unroll
-        for (int j = 0; j < RB; ++j) {
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) acc[a][j][cb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        }
-    }
-
-    uint4 rw[ACC][RB][U], rx[CB][U];
-    auto fill = [&](int u, int ks) {
-#pragma unroll
-        for (int a = 0; a < ACC; ++a) {
-#pragma unroll
-            for (int j = 0; j < RB; ++j) rw[a][j][u] = load16(wp[a][j] + ks * 32);
-        }
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            rx[cb][u] = xvalid[cb] ? load16(xp[cb] + ks * 32) : make_uint4(0u, 0u, 0u, 0u);
-        }
-    };
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        if (ks0 + u < ks1) fill(u, ks0 + u);
-    }
-    for (int ks = ks0; ks < ks1; ks += U) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (ks + u < ks1) {                            // wave-uniform
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    const bf16x8_t xf = __builtin_bit_cast(bf16x8_t, rx[cb][u]);
-#pragma unroll
-                    for (int a = 0; a < ACC; ++a) {
-#pragma unroll
-                        for (int j = 0; j < RB; ++j) {
-                            acc[a][j][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                                __builtin_bit_cast(bf16x8_t, rw[a][j][u]), xf, acc[a][j][cb], 0, 0, 0);
-                        }
-                    }
-                }
-                if (ks + U + u < ks1) fill(u, ks + U + u);
-            }
-        }
-    }
-
-    if (sk > 1) {
-#pragma unroll
-        for (int a = 0; a < ACC; ++a) {
-#pragma unroll
-            for (int j = 0; j < RB; ++j) {
-                if (kslice != 0) {
-#pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) s_red[wave][cb][r * 64 + lane] = acc[a][j][cb][r];
-                    }
-                }
-                __syncthreads();
-                if (kslice == 0) {
-                    for (int o = 1; o < sk; ++o) {
-#pragma unroll
-                        for (int cb = 0; cb < CB; ++cb) {
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) acc[a][j][cb][r] += s_red[wave + o][cb][r * 64 + lane];
-                        }
-                    }
-                }
-                __syncthreads();
-            }
-        }
-        if (kslice != 0) return;
-    }
-
-    // acc[.][j][cb][r] is weight row n0 + 16*j + 4*fg + r against activation row cb*16 + fn
-#pragma unroll
-    for (int j = 0; j < RB; ++j) {
-        const int n = n0 + j * 16 + 4 * fg;
-        if (n >= p.N) continue;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            const int m = cb * 16 + fn;
-            if (m >= p.M) continue;
-            float o[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if constexpr (SWIGLU) {
-                    const float g = __uint_as_float(f32_to_bf16_bits(acc[0][j][cb][r]) << 16);
-                    const float u = __uint_as_float(f32_to_bf16_bits(acc[ACC - 1][j][cb][r]) << 16);
-                    o[r] = silu_rounded(g) * u;
-                } else {
-                    o[r] = acc[0][j][cb][r];
-                }
-            }
-            if (p.rope_table) {
-                store_qkv_pair(p, m, n, pack_bf16x2(o[0], o[1]));
-                store_qkv_pair(p, m, n + 2, pack_bf16x2(o[2], o[3]));
-                continue;
-            }
-            if (p.res) {
-                const uint2 rv = *reinterpret_cast<const uint2*>(p.res + int64_t(m) * p.y_stride + n);
-                o[0] = bf16lo_to_f32(rv.x) + __uint_as_float(f32_to_bf16_bits(o[0]) << 16);
-                o[1] = bf16hi_to_f32(rv.x) + __uint_as_float(f32_to_bf16_bits(o[1]) << 16);
-                o[2] = bf16lo_to_f32(rv.y) + __uint_as_float(f32_to_bf16_bits(o[2]) << 16);
-                o[3] = bf16hi_to_f32(rv.y) + __uint_as_float(f32_to_bf16_bits(o[3]) << 16);
-            }
-            uint2 w;
-            w.x = pack_bf16x2(o[0], o[1]);
-            w.y = pack_bf16x2(o[2], o[3]);
-            *reinterpret_cast<uint2*>(p.y + int64_t(m) * p.y_stride + n) = w;
-        }
-    }
-}
-
-template <int NW, int RB, int U, bool SWIGLU>
-int launch_wide(const LinearParams& p, hipStream_t stream) {
-    const int row_groups = (p.N + 16 * RB - 1) / (16 * RB);
-    const int rg_per_wg = NW / p.sk;
-    const dim3 grid(unsigned((row_groups + rg_per_wg - 1) / rg_per_wg));
-    hipLaunchKernelGGL((linear_wide_kernel<NW, RB, U, SWIGLU>), grid, dim3(NW * kWaveSize), 0, stream, p);
-    return int(hipGetLastError());
-}
-
 template <int NW, int CBLK, int U, bool SWIGLU, bool XLDS, int RW = 16>
 int launch_variant(const LinearParams& p, hipStream_t stream) {
     const int row_blocks = (p.N + RW - 1) / RW;
@@ -504,14 +339,9 @@ bool linear_skinny_can_stage(int M, int K) {
 }
 
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream) {
-    const bool wide = p.M > 16;
+    if (p.M > 16) return int(hipErrorInvalidValue);   // one 16-column MFMA block of activation rows (checked by the caller)
     const bool stage = p.norm_w != nullptr;   // the caller has checked linear_skinny_can_stage
     const int row_blocks = (p.N + 15) / 16;
-    if (wide) {
-        constexpr int RB = 2;
-        p.sk = linear_skinny_plan(p.N, p.K, 8, num_cus / 2, 16 * RB, 32);   // one 8-wavefront workgroup per CU
-        return swiglu ? launch_wide<8, RB, 4, true>(p, stream) : launch_wide<8, RB, 6, false>(p, stream);
-    }
     // a matrix with too few 16-row blocks to fill the device, and at most four activation rows:
     // four weight rows per wavefront
     if (!swiglu && p.M <= 4 && p.K % 128 == 0 && row_blocks < 2 * num_cus) {
@@ -520,7 +350,7 @@ int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t s
                      : launch_variant<8, 1, 8, false, false, 4>(p, stream);
     }
     // few row blocks and a long K (the MLP's down projection): sixteen wavefronts share a row block
-    const bool big_wg = !wide && !swiglu && row_blocks < num_cus && p.K / 32 >= 128;
+    const bool big_wg = !swiglu && row_blocks < num_cus && p.K / 32 >= 128;
     p.sk = linear_skinny_plan(p.N, p.K, big_wg ? 16 : 8, num_cus, 16, 32);
     if (swiglu) {
         return stage ? launch_variant<8, 1, 8, true, true>(p, stream) : launch_variant<8, 1, 8, true, false>(p, stream);

@@ -125,7 +125,39 @@ linear_splitk_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
     }
 }
 
+// y[m][n] = bf16(sum over splits of part[s][m][n]) (+ residual, with the rounding of a separate
+// bf16 addition): the split-K linear finished on its own, for callers with no elementwise
+// operator to fold the sum into.  Eight outputs per lane.
+__global__ void __launch_bounds__(256)
+linear_splitk_finish_kernel(const float* __restrict__ part, int ksplit, int64_t split_stride,
+                            const uint16_t* __restrict__ res, uint16_t* __restrict__ y, int M, int N, int64_t y_stride) {
+    const int nvec = N / 8;
+    const int64_t item = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (item >= int64_t(M) * nvec) return;
+    const int m = int(item / nvec);
+    const int n = int(item % nvec) * 8;
+    uint4 o = sum_splits_bf16x8(part + int64_t(m) * N + n, ksplit, split_stride);
+    if (res) {
+        float a[8], b[8];
+        unpack8(o, a);
+        unpack8(load16(res + int64_t(m) * y_stride + n), b);
+        o.x = pack_bf16x2(a[0] + b[0], a[1] + b[1]);
+        o.y = pack_bf16x2(a[2] + b[2], a[3] + b[3]);
+        o.z = pack_bf16x2(a[4] + b[4], a[5] + b[5]);
+        o.w = pack_bf16x2(a[6] + b[6], a[7] + b[7]);
+    }
+    store16(y + int64_t(m) * y_stride + n, o);
+}
+
 }  // namespace
+
+int launch_linear_splitk_finish(const float* part, int ksplit, const uint16_t* res, uint16_t* y, int M, int N,
+                                int64_t y_stride, hipStream_t stream) {
+    const int64_t items = int64_t(M) * (N / 8);
+    hipLaunchKernelGGL(linear_splitk_finish_kernel, dim3(unsigned((items + 255) / 256)), dim3(256), 0, stream, part,
+                       ksplit, int64_t(M) * N, res, y, M, N, y_stride);
+    return int(hipGetLastError());
+}
 
 // Splits of K: a workgroup covers 128, 256 or 512 k; the largest of these that still gives about
 // one workgroup per CU (fewer splits mean less partial-product traffic).

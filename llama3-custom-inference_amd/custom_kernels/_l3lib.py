@@ -20,7 +20,8 @@ L3_ERR_WORKSPACE = -7
 L3_ERR_SPLITS = -8
 L3_ERR_HIP = -9
 L3_ATTN_MAX_SPLITS = 512
-L3_LINEAR_MAX_ROWS = 64
+L3_LINEAR_MAX_ROWS = 16
+L3_LINEAR_SPLITK_MAX_ROWS = 64
 L3_LINEAR_STAGE_ELEMS = 24576   # activations (rows padded by 8) the fused input norm can stage in LDS
 L3_ATTN_OPT_KERNEL = 0
 L3_ATTN_KERNEL_FMA = 0
@@ -121,6 +122,11 @@ SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
          ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p],
+    ),
+    "l3_linear_splitk_finish": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+         ctypes.c_void_p],
     ),
     "l3_add_rms_norm_partials": (
         ctypes.c_int,

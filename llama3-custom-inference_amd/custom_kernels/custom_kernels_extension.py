@@ -420,13 +420,13 @@ def silu_mul(a, b):
     return y
 
 
-def _linear_args(x, weights):
+def _linear_args(x, weights, max_rows=None):
     _require_gpu_bf16("x", x)
     K = x.shape[-1]
     rows = x.numel() // max(K, 1)
-    if x.dim() < 1 or rows < 1 or rows > _l3lib.L3_LINEAR_MAX_ROWS:
-        raise RuntimeError(f"linear_decode: 1..{_l3lib.L3_LINEAR_MAX_ROWS} activation rows expected, got "
-                           f"{tuple(x.shape)}")
+    max_rows = _l3lib.L3_LINEAR_MAX_ROWS if max_rows is None else max_rows
+    if x.dim() < 1 or rows < 1 or rows > max_rows:
+        raise RuntimeError(f"linear_decode: 1..{max_rows} activation rows expected, got {tuple(x.shape)}")
     for w in weights:
         _require_gpu_bf16("weight", w)
         if w.dim() != 2 or w.shape[1] != K or w.stride(1) != 1 or tuple(w.shape) != tuple(weights[0].shape) \
@@ -441,8 +441,12 @@ def _linear_args(x, weights):
 def linear_decode(x, weight):
     """F.linear(x, weight) for at most 64 activation rows (model.py:95,121,134,225 when T == 1):
     one pass over the weight matrix at HBM speed instead of a GEMM.  x (..., K), weight (N, K)
-    -> (..., N).  An extension."""
+    -> (..., N).  Up to 16 rows are one launch; 17..64 rows go through linear_splitk and
+    linear_splitk_finish (N % 8 == 0 and K % 128 == 0 then), which suits matrices of a few thousand
+    rows -- a vocabulary projection at that many rows is a job for a library GEMM.  An extension."""
     lib = _l3lib.load()
+    if x.shape[-1] > 0 and x.numel() // x.shape[-1] > _l3lib.L3_LINEAR_MAX_ROWS:
+        return linear_splitk_finish(linear_splitk(x, weight)).view(*x.shape[:-1], weight.shape[0])
     x2, rows, N, K = _linear_args(x, (weight,))
     y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
@@ -454,7 +458,7 @@ def linear_decode(x, weight):
 
 
 def linear_swiglu_decode(x, w_gate, w_up):
-    """F.silu(F.linear(x, w_gate)) * F.linear(x, w_up) for at most 64 activation rows in one
+    """F.silu(F.linear(x, w_gate)) * F.linear(x, w_up) for at most 16 activation rows in one
     launch (model.py:134 with w_gate = c_fc2, w_up = c_fc), same rounding points.  An extension."""
     lib = _l3lib.load()
     x2, rows, N, K = _linear_args(x, (w_gate, w_up))
@@ -478,6 +482,10 @@ def linear_decode_fused(x, weight, norm_weight=None, eps: float = 1e-5, w_up=Non
     matrix w_up (weight is then the gate, model.py:134), and `residual + result` behind
     (model.py:147-148) -- all with the rounding points of the separate operators.  An extension."""
     lib = _l3lib.load()
+    if norm_weight is None and w_up is None and x.shape[-1] > 0 \
+            and x.numel() // x.shape[-1] > _l3lib.L3_LINEAR_MAX_ROWS:
+        # 17..64 rows: split-K, the residual joins when the splits are added up
+        return linear_splitk_finish(linear_splitk(x, weight), residual).view(*x.shape[:-1], weight.shape[0])
     x2, rows, N, K = _linear_args(x, (weight,) if w_up is None else (weight, w_up))
     if norm_weight is not None:
         _require_gpu_bf16("norm_weight", norm_weight)
@@ -512,7 +520,7 @@ def linear_splitk(x, weight, ksplit: int = 0):
     ksplit 0 lets the library choose.  Stands for nn.Linear at batch sizes where the activations no
     longer fit one matrix-instruction column block (model.py:95,121,134).  An extension."""
     lib = _l3lib.load()
-    x2, rows, N, K = _linear_args(x, (weight,))
+    x2, rows, N, K = _linear_args(x, (weight,), _l3lib.L3_LINEAR_SPLITK_MAX_ROWS)
     with torch.cuda.device(x.device):
         if ksplit <= 0:
             ksplit = lib.l3_linear_splitk_plan(N, K, _cus(x.device))
@@ -524,6 +532,31 @@ def linear_splitk(x, weight, ksplit: int = 0):
     if rc != 0:
         _fail(rc, f"M={rows} N={N} K={K} ksplit={ksplit}")
     return part
+
+
+def linear_splitk_finish(part, residual=None):
+    """bf16(part.sum(0)) for linear_splitk's partial products (ksplit, rows, N), summed in split
+    order and rounded once -- what the unsplit linear would have returned -- plus ``residual``
+    (rows x N, bf16) with the rounding of a separate addition if given.  Returns (rows, N)."""
+    lib = _l3lib.load()
+    if not part.is_cuda or part.dtype != torch.float32 or part.dim() != 3 or not part.is_contiguous():
+        raise RuntimeError("linear_splitk_finish: expected contiguous float32 (ksplit, rows, N) partials")
+    ksplit, rows, N = part.shape
+    r2 = None
+    if residual is not None:
+        _require_gpu_bf16("residual", residual)
+        if residual.numel() != rows * N or residual.shape[-1] != N:
+            raise RuntimeError(f"linear_splitk_finish: residual {tuple(residual.shape)} does not fit ({rows}, {N})")
+        r2 = residual.reshape(rows, N)
+        if not r2.is_contiguous():
+            r2 = r2.contiguous()
+    y = torch.empty((rows, N), dtype=torch.bfloat16, device=part.device)
+    with torch.cuda.device(part.device):
+        rc = lib.l3_linear_splitk_finish(part.data_ptr(), ksplit, None if r2 is None else r2.data_ptr(), y.data_ptr(),
+                                         rows, N, N, _stream_ptr(part.device))
+    if rc != 0:
+        _fail(rc, f"rows={rows} N={N} ksplit={ksplit}")
+    return y
 
 
 def add_rms_norm_partials(input, part, weight, eps):

@@ -256,6 +256,18 @@ def test_linear_splitk_plan_and_argument_checks():
     assert call(ks=2) == _l3lib.L3_ERR_SPLITS          # 1024 k per workgroup
     assert call(ks=17) == _l3lib.L3_ERR_SPLITS
     assert call(nbytes=1024) == _l3lib.L3_ERR_WORKSPACE
+    assert _l3lib.L3_LINEAR_MAX_ROWS == 16 and _l3lib.L3_LINEAR_SPLITK_MAX_ROWS == 64
+
+    def finish(part=FAKE, ks=4, res=None, y=FAKE, M=64, N=2048, stride=2048):
+        return lib.l3_linear_splitk_finish(part, ks, res, y, M, N, stride, None)
+
+    assert finish(part=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert finish(y=None) == _l3lib.L3_ERR_NULL_POINTER
+    assert finish(M=65) == _l3lib.L3_ERR_SHAPE
+    assert finish(N=2052) == _l3lib.L3_ERR_SHAPE
+    assert finish(ks=0) == _l3lib.L3_ERR_SPLITS
+    assert finish(stride=2040) == _l3lib.L3_ERR_STRIDE
+    assert finish(res=FAKE + 8) == _l3lib.L3_ERR_ALIGNMENT
     assert lib.l3_add_rms_norm_partials(FAKE, FAKE, 0, FAKE, FAKE, FAKE, 64, 2048, 1e-5, None) == _l3lib.L3_ERR_SPLITS
     assert lib.l3_add_rms_norm_partials(FAKE, FAKE, 4, FAKE, FAKE, FAKE, 64, 2044, 1e-5, None) == _l3lib.L3_ERR_SHAPE
     cs = _l3lib.i64_array((256 * 512, 512))

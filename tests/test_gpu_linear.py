@@ -26,9 +26,11 @@ def assert_linear_close(y, ref, what):
 
 # (M, N, K): the 1B-architecture decode shapes (qkv, out projection, MLP down projection, lm head),
 # batch sizes up to 64, and shapes off every multiple the kernel tiles by
+# (rows above 16 are served by the split-K kernel and its finishing pass: N % 8 == 0, K % 128 == 0)
 SHAPES = [(1, 3072, 2048), (1, 2048, 2048), (1, 2048, 8192), (1, 128256, 2048), (3, 1024, 512), (16, 3072, 2048),
-          (17, 512, 256), (64, 3072, 2048), (64, 2048, 8192), (5, 20, 32), (2, 36, 64), (33, 100, 96),
-          (64, 16, 4096), (1, 16, 32), (8, 6144, 4096), (4, 2048, 8192), (4, 20, 128), (2, 3072, 2048), (3, 4, 384)]
+          (17, 512, 256), (64, 3072, 2048), (64, 2048, 8192), (5, 20, 32), (2, 36, 64), (33, 104, 384),
+          (64, 16, 4096), (1, 16, 32), (8, 6144, 4096), (4, 2048, 8192), (4, 20, 128), (2, 3072, 2048), (3, 4, 384),
+          (16, 100, 96), (40, 2048, 2048)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -62,6 +64,8 @@ def test_linear_decode_layouts_and_errors(gpu):
     assert torch.equal(cke.linear_decode(x[2:3], w), y[2:3])
     with pytest.raises(RuntimeError):
         cke.linear_decode(randn_bf16((65, K), 1).to(gpu), w)          # too many rows for this entry point
+    with pytest.raises(RuntimeError):                                 # 17..64 rows need N % 8 == 0 and K % 128 == 0
+        cke.linear_decode(randn_bf16((20, 96), 1).to(gpu), randn_bf16((64, 96), 2).to(gpu))
     with pytest.raises(RuntimeError):
         cke.linear_decode(randn_bf16((2, 48), 1).to(gpu), randn_bf16((8, 48), 2).to(gpu))   # K % 32 != 0
     with pytest.raises(RuntimeError):
@@ -70,7 +74,7 @@ def test_linear_decode_layouts_and_errors(gpu):
         cke.linear_decode(randn_bf16((2, K), 1), w)                   # CPU tensor
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 8192, 2048), (64, 8192, 2048), (7, 1024, 256), (16, 14336, 4096), (40, 52, 64)])
+@pytest.mark.parametrize("M,N,K", [(1, 8192, 2048), (12, 8192, 2048), (7, 1024, 256), (16, 14336, 4096), (9, 52, 64)])
 def test_linear_swiglu_decode(gpu, M, N, K):
     from custom_kernels import custom_kernels_extension as cke
 
@@ -166,7 +170,7 @@ def test_linear_fused_whole_mlp_and_limits(gpu):
 
 @pytest.mark.parametrize("B,NH,KVH,HD,K,norm", [(1, 32, 8, 64, 2048, True), (8, 32, 8, 64, 2048, True),
                                                 (16, 32, 8, 64, 2048, False), (3, 8, 2, 128, 512, True),
-                                                (64, 32, 8, 64, 2048, False), (2, 4, 4, 64, 96, False)])
+                                                (13, 32, 8, 64, 2048, False), (2, 4, 4, 64, 96, False)])
 def test_linear_qkv_rope_append_equals_the_separate_operators(gpu, B, NH, KVH, HD, K, norm):
     from custom_kernels import custom_kernels_extension as cke
     from custom_kernels import precompute_freqs_cis
@@ -228,6 +232,34 @@ def test_linear_splitk_against_oracle(gpu, M, N, K, ksplit):
     s = part.shape[0] - 1
     ref_last = linear_ref(t2f32(x)[:, s * per:], t2f32(w)[:, s * per:])
     assert np.abs(part[s].cpu().numpy() - ref_last).max() <= 1e-4 * max(1.0, np.abs(ref_last).max())
+
+
+@pytest.mark.parametrize("M,N,K,with_res", [(64, 2048, 8192, True), (64, 3072, 2048, False), (17, 256, 128, True),
+                                            (33, 2048, 2048, True)])
+def test_linear_splitk_finish_equals_the_unsplit_linear(gpu, M, N, K, with_res):
+    """Split-K + finish against the float64 oracle, and the residual form against a bf16 linear
+    followed by a bf16 addition (the two roundings of model.py:147-148)."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"linear_splitk_finish M={M} N={N} K={K} residual={with_res}", flush=True)
+    x = randn_bf16((M, 1, K), 41)
+    w = randn_bf16((N, K), 42, scale=0.05)
+    part = cke.linear_splitk(x.to(gpu), w.to(gpu))
+    y = cke.linear_splitk_finish(part)
+    torch.cuda.synchronize()
+    assert y.shape == (M, N)
+    assert_linear_close(y, linear_ref(t2f32(x), t2f32(w)).reshape(M, N), "split-K + finish")
+    assert torch.equal(y, _sum_in_split_order(part).to(torch.bfloat16))
+    assert torch.equal(cke.linear_decode(x.to(gpu), w.to(gpu)).view(M, N), y)      # what linear_decode does at these rows
+    if with_res:
+        res = randn_bf16((M, 1, N), 43).to(gpu)
+        yr = cke.linear_splitk_finish(part, res)
+        assert torch.equal(yr, (res.view(M, N) + y))
+        assert torch.equal(cke.linear_decode_fused(x.to(gpu), w.to(gpu), residual=res).view(M, N), yr)
+    with pytest.raises(RuntimeError):
+        cke.linear_splitk_finish(part.to(torch.bfloat16))
+    with pytest.raises(RuntimeError):
+        cke.linear_splitk_finish(part, randn_bf16((M, N + 8), 44).to(gpu))
 
 
 def test_linear_splitk_errors(gpu):

@@ -130,6 +130,8 @@ def test_decode_linear_random_shapes(gpu):
         M = int(rng.choice((1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 48, 64)))
         N = 4 * int(rng.integers(1, 1200))
         K = 32 * int(rng.integers(1, 200))
+        if M > 16:                                           # split-K + finish: N % 8 == 0, K % 128 == 0
+            N, K = 8 * ((N + 7) // 8), 128 * ((K + 127) // 128)
         print(f"linear case {i}: M={M} N={N} K={K}", flush=True)
         x = randn_bf16((M, 1, K), 8000 + i)
         w = randn_bf16((N, K), 9000 + i, scale=0.05)
