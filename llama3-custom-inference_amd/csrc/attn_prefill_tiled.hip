@@ -279,9 +279,10 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
 // leaves the matrix pipe idle during the softmax and the vector pipe idle during the products
 // (and the wavefronts of a workgroup, held in step by the per-tile barrier, do so together).
 // Here iteration `it` multiplies K of tile it, takes the softmax of tile it - 1 and adds tile
-// it - 2 to the output: three independent pieces of work in one basic block, which the
-// scheduler interleaves.  An LDS stage therefore holds K of one tile and V of the tile two
-// before it.  The rescale that a softmax finds is applied to the output accumulators at the
+// it - 2 to the output: three independent pieces of work in one basic block, placed by hand in
+// the steady state.  An LDS stage therefore holds K of one tile and V of the tile two before it;
+// the next stage is fetched while the current one is used, by loads that write LDS directly
+// (no registers, no copy).  The rescale that a softmax finds is applied to the output accumulators at the
 // start of the NEXT iteration (after the P of tile it - 2, which still refers to the previous
 // maximum, has been added); the two sets of score / probability registers swap roles every
 // iteration, hence the loop unrolled by two.
@@ -289,9 +290,21 @@ template <int HD, int CB, int NW>
 __global__ void __launch_bounds__(NW * kWaveSize)
 attn_prefill_pipe_kernel(const PrefillParams p) {
     using T = PrefillTile<HD, CB, NW>;
-    constexpr int NT = T::NT, TK = T::TK, LPR = T::LPR, U = T::U, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
-    constexpr int KPITCH = T::KPITCH, VPITCH = T::VPITCH, KBYTES = T::KBYTES, STAGE = T::STAGE;
-    __shared__ __align__(16) unsigned char s_tiles[2 * STAGE];
+    constexpr int TK = T::TK, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
+    // K/V tiles go from global memory straight into LDS (global_load_lds_dwordx4: a wavefront-wide
+    // load lands in 1 KiB of consecutive LDS), so rows cannot be padded; instead the 16-byte chunk c
+    // of token row r sits at chunk position c ^ key(r), which spreads the rows that an operand
+    // read touches together over all banks.
+    constexpr int CPR = HD / 8;                 // 16-byte chunks per token row
+    constexpr int ROWB = HD * 2;                // bytes per token row
+    constexpr int KBYTES = TK * ROWB;           // a K tile; a stage is a K tile followed by a V tile
+    constexpr int STAGE = 2 * KBYTES;
+    constexpr int IPW = CPR / NW;               // wavefront-wide loads per wavefront and tile
+    static_assert(CPR % NW == 0, "a tile must divide evenly over the wavefronts");
+    // Two separate arrays, so that the compiler can tell a read of one stage from the load in flight
+    // into the other and does not wait for that load before every LDS read.
+    __shared__ __align__(1024) unsigned char s_stage0[STAGE];
+    __shared__ __align__(1024) unsigned char s_stage1[STAGE];
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
@@ -336,31 +349,45 @@ attn_prefill_pipe_kernel(const PrefillParams p) {
         }
     }
 
-    const uint16_t* kbase = p.k + b * p.k_sb + kvh * p.k_sh + (tid % LPR) * 8;
-    const uint16_t* vbase = p.v + b * p.v_sb + kvh * p.v_sh + (tid % LPR) * 8;
-    const int ld_row = tid / LPR;
-    constexpr int ROWS_PER_LOAD = NT / LPR;
-    uint4 kr[U], vr[U];
-    // the stage of iteration `it`: K of tile it, V of tile it - 2 (rows outside the data are
-    // clamped to a valid row and never used)
-    auto issue = [&](int it) {
+    // global -> LDS: load j of a wavefront covers slots inst*64 .. +63 of the tile, slot = row * CPR + position
+    const uint16_t* kb = p.k + b * p.k_sb + kvh * p.k_sh;
+    const uint16_t* vb = p.v + b * p.v_sb + kvh * p.v_sh;
+    auto swz_key = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
+    // the stage of iteration `it`: K of tile it, V of tile it - 2 (rows outside the data are clamped
+    // to a valid row and never used)
+    auto dma = [&](int it, unsigned char* stage) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int row = u * ROWS_PER_LOAD + ld_row;
+        for (int j = 0; j < IPW; ++j) {
+            const int inst = wave * IPW + j;
+            const int slot = inst * kWaveSize + lane;
+            const int row = slot / CPR;
+            const int chunk = (slot % CPR) ^ swz_key(row);
             const int tok_k = min(it * TK + row, p.S - 1);
             const int tok_v = min(max((it - 2) * TK + row, 0), p.S - 1);
-            kr[u] = load16(kbase + int64_t(tok_k) * p.k_st);
-            vr[u] = load16(vbase + int64_t(tok_v) * p.v_st);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(kb + int64_t(tok_k) * p.k_st + chunk * 8),
+                L3_LDS_PTR(void, stage + inst * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(vb + int64_t(tok_v) * p.v_st + chunk * 8),
+                L3_LDS_PTR(void, stage + KBYTES + inst * 1024), 16, 0, 0);
         }
     };
-    auto stash = [&](unsigned char* stage) {
+    // operand addresses within a stage.  K: lane (fn, fg) reads chunk 4m + fg of row 16 tg + fn, whose
+    // key depends on fn alone.  V (transposing read): lane reads 8 bytes of row 32 ks + 4 fg + (fn >> 2)
+    // (+16) in the 32-byte column block nb, i.e. chunk 2 nb + ((lane & 3) >> 1); the key depends on the
+    // lane alone as well.  One address per m / nb, the rest is instruction offsets.
+    int ak[KC], av[NB];   // byte offsets within a stage
+    {
+        const int kkey = swz_key(fn);
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int row = u * ROWS_PER_LOAD + ld_row;
-            *reinterpret_cast<uint4*>(stage + row * KPITCH + (tid % LPR) * 16) = kr[u];
-            *reinterpret_cast<uint4*>(stage + KBYTES + row * VPITCH + (tid % LPR) * 16) = vr[u];
+        for (int m = 0; m < KC; ++m) ak[m] = fn * ROWB + (((m * 4 + fg) ^ kkey) << 4);
+        const int vrow = 4 * fg + (fn >> 2);
+        const int vkey = swz_key(vrow);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            av[nb] = KBYTES + vrow * ROWB + (((nb * 2 + ((lane & 3) >> 1)) ^ vkey) << 4) + (lane & 1) * 8;
         }
-    };
+    }
 
     f32x4_t O[CB][NB];
     float m_run[CB], l_part[CB];
@@ -385,12 +412,10 @@ attn_prefill_pipe_kernel(const PrefillParams p) {
 
     // One iteration on its LDS stage.  STEADY: all three phases are live and the softmax tile needs no
     // causal mask.
-    auto body = [&](auto steady_tag, int it, f32x4_t (&Sprod)[CB][NG], f32x4_t (&Scons)[CB][NG],
+    auto body = [&](auto steady_tag, auto parity_tag, int it, f32x4_t (&Sprod)[CB][NG], f32x4_t (&Scons)[CB][NG],
                     uint4 (&Pcons)[CB][KS], uint4 (&Pprod)[CB][KS]) {
         constexpr bool STEADY = decltype(steady_tag)::value;
-        const unsigned char* stage = s_tiles + (it & 1) * STAGE;
-        const unsigned char* rd_k = stage + fn * KPITCH + fg * 16;
-        const unsigned char* rd_v = stage + KBYTES + (4 * fg + (fn >> 2)) * VPITCH + (lane & 3) * 8;
+        const unsigned char* stage = decltype(parity_tag)::value ? s_stage1 : s_stage0;   // this iteration's stage
         const bool do_qk = STEADY || it < wt;
         const bool do_sm = STEADY || (it >= 1 && it <= wt);
         const bool do_pv = STEADY || (it >= 2 && it <= wt + 1);
@@ -471,16 +496,16 @@ attn_prefill_pipe_kernel(const PrefillParams p) {
                                                                 __builtin_bit_cast(bf16x8_t, Pcons[cb][ks]), O[cb][nb], 0, 0, 0);
         };
         auto read_k = [&](int g) {
-            return *reinterpret_cast<const uint4*>(rd_k + (g / KC) * 16 * KPITCH + (g % KC) * 64);
+            return *reinterpret_cast<const uint4*>(stage + ak[g % KC] + (g / KC) * 16 * ROWB);
         };
         // the k slots of a 32-token step pair (fg, i) with token 4*fg + i of the step's first 16-token
         // group for i < 4 and of its second group for i >= 4
         auto read_v = [&](int h) {
             const int ks = h / NB, nb = h % NB;
             const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                L3_LDS_PTR(s16x4_t, rd_v + (2 * ks) * 16 * VPITCH + nb * 32));
+                L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
             const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                L3_LDS_PTR(s16x4_t, rd_v + (2 * ks + 1) * 16 * VPITCH + nb * 32));
+                L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
             return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         };
 
@@ -549,22 +574,23 @@ attn_prefill_pipe_kernel(const PrefillParams p) {
         }
     };
 
-    auto run = [&](int it, f32x4_t (&Sprod)[CB][NG], f32x4_t (&Scons)[CB][NG], uint4 (&Pcons)[CB][KS],
-                   uint4 (&Pprod)[CB][KS]) {
+    auto run = [&](auto parity_tag, int it, f32x4_t (&Sprod)[CB][NG], f32x4_t (&Scons)[CB][NG],
+                   uint4 (&Pcons)[CB][KS], uint4 (&Pprod)[CB][KS]) {
+        constexpr int PAR = decltype(parity_tag)::value;
         const bool more = it + 1 < n_it;   // workgroup-uniform
-        if (more) issue(it + 1);
+        // the other stage was last read before the previous barrier: its refill can start now
+        if (more) dma(it + 1, PAR ? s_stage0 : s_stage1);
         if (it >= 2 && it < wt && it * TK <= wave_limit_min) {
-            body(std::true_type{}, it, Sprod, Scons, Pcons, Pprod);
+            body(std::true_type{}, parity_tag, it, Sprod, Scons, Pcons, Pprod);
         } else {
-            body(std::false_type{}, it, Sprod, Scons, Pcons, Pprod);
+            body(std::false_type{}, parity_tag, it, Sprod, Scons, Pcons, Pprod);
         }
-        // the other stage was last read before the previous barrier: refill it, then meet
-        if (more) stash(s_tiles + ((it + 1) & 1) * STAGE);
+        __builtin_amdgcn_s_waitcnt(0xF70);   // vmcnt(0): this wavefront's part of the next stage has landed
         __syncthreads();
     };
 
-    issue(0);
-    stash(s_tiles);
+    dma(0, s_stage0);
+    __builtin_amdgcn_s_waitcnt(0xF70);
     __syncthreads();
 
     f32x4_t SA[CB][NG], SB[CB][NG];
@@ -577,8 +603,8 @@ attn_prefill_pipe_kernel(const PrefillParams p) {
         for (int ks = 0; ks < KS; ++ks) PA[cb][ks] = PB[cb][ks] = make_uint4(0u, 0u, 0u, 0u);
     }
     for (int it = 0; it < n_it; it += 2) {
-        run(it, SA, SB, PA, PB);
-        if (it + 1 < n_it) run(it + 1, SB, SA, PB, PA);
+        run(std::integral_constant<int, 0>{}, it, SA, SB, PA, PB);
+        if (it + 1 < n_it) run(std::integral_constant<int, 1>{}, it + 1, SB, SA, PB, PA);
     }
 
 #pragma unroll
