@@ -4,6 +4,8 @@
 // product x * inv_rms * w is formed in float32 and rounded to bf16 once (the reference
 // rounds inv_rms and both products to bf16, custom_kernels.cu:362-366), and the row is
 // reduced with wave64 DPP steps instead of 32-lane shuffles plus a 32-entry shared stage.
+#include <algorithm>
+
 #include "l3_device.hpp"
 #include "l3_host.hpp"
 
@@ -83,6 +85,93 @@ rms_norm_rows_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
             o.w = pack_bf16x2(f[6] * inv * g[6], f[7] * inv * g[7]);
             store16(yr + vi * 8, o);
         }
+    }
+}
+
+// Thousands of rows (prefill): a wavefront walks over rows row, row + stride, ... and requests
+// the next row before it reduces the current one, so that the device reads and writes at the same
+// time instead of reading every row first and writing every row afterwards.  The norm weights stay
+// in registers.  C % 8 == 0 and C / 8 <= 64 * MAXV.  ADD as in the kernel above.
+template <int MAXV, bool ADD>
+__global__ void __launch_bounds__(kRmsThreads)
+rms_norm_stream_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ res,
+                       const uint16_t* __restrict__ w, uint16_t* __restrict__ sum_out, uint16_t* __restrict__ y,
+                       int64_t rows, int C, float eps) {
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int64_t stride = int64_t(gridDim.x) * (kRmsThreads / kWaveSize);
+    int64_t row = int64_t(blockIdx.x) * (kRmsThreads / kWaveSize) + threadIdx.x / kWaveSize;
+    if (row >= rows) return;
+    const int nvec = C / 8;
+    uint4 wv[MAXV], cur[MAXV], nxt[MAXV], rcur[ADD ? MAXV : 1], rnxt[ADD ? MAXV : 1];
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+        const int vi = lane + j * kWaveSize;
+        if (vi < nvec) {
+            cur[j] = load16(x + row * int64_t(C) + vi * 8);
+            if constexpr (ADD) rcur[j] = load16(res + row * int64_t(C) + vi * 8);
+            wv[j] = load16(w + vi * 8);
+        }
+    }
+    const float inv_c = 1.0f / float(C);
+    while (true) {
+        const int64_t nrow = row + stride;
+        const bool has_next = nrow < rows;   // wave-uniform
+        if (has_next) {
+#pragma unroll
+            for (int j = 0; j < MAXV; ++j) {
+                const int vi = lane + j * kWaveSize;
+                if (vi < nvec) {
+                    nxt[j] = load16(x + nrow * int64_t(C) + vi * 8);
+                    if constexpr (ADD) rnxt[j] = load16(res + nrow * int64_t(C) + vi * 8);
+                }
+            }
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAXV; ++j) {
+            const int vi = lane + j * kWaveSize;
+            if (vi < nvec) {
+                float f[8];
+                unpack8(cur[j], f);
+                if constexpr (ADD) {
+                    // s = bf16(x + res) goes out, and the norm is taken of the rounded s
+                    float r[8];
+                    unpack8(rcur[j], r);
+                    cur[j].x = pack_bf16x2(f[0] + r[0], f[1] + r[1]);
+                    cur[j].y = pack_bf16x2(f[2] + r[2], f[3] + r[3]);
+                    cur[j].z = pack_bf16x2(f[4] + r[4], f[5] + r[5]);
+                    cur[j].w = pack_bf16x2(f[6] + r[6], f[7] + r[7]);
+                    store16(sum_out + row * int64_t(C) + vi * 8, cur[j]);
+                    unpack8(cur[j], f);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+            }
+        }
+        ss = wave_sum(ss);
+        const float inv = rsqrtf(ss * inv_c + eps);
+#pragma unroll
+        for (int j = 0; j < MAXV; ++j) {
+            const int vi = lane + j * kWaveSize;
+            if (vi < nvec) {
+                float f[8], g[8];
+                unpack8(cur[j], f);
+                unpack8(wv[j], g);
+                uint4 o;
+                o.x = pack_bf16x2(f[0] * inv * g[0], f[1] * inv * g[1]);
+                o.y = pack_bf16x2(f[2] * inv * g[2], f[3] * inv * g[3]);
+                o.z = pack_bf16x2(f[4] * inv * g[4], f[5] * inv * g[5]);
+                o.w = pack_bf16x2(f[6] * inv * g[6], f[7] * inv * g[7]);
+                store16(y + row * int64_t(C) + vi * 8, o);
+            }
+        }
+        if (!has_next) break;
+#pragma unroll
+        for (int j = 0; j < MAXV; ++j) {
+            cur[j] = nxt[j];
+            if constexpr (ADD) rcur[j] = rnxt[j];
+        }
+        row = nrow;
     }
 }
 
@@ -191,7 +280,18 @@ int launch_rms_norm_impl(const uint16_t* x, const uint16_t* res, const uint16_t*
                          int64_t rows, int C, float eps, bool vec_ok, hipStream_t stream) {
     const int nvec = C / 8;
     const dim3 block(kRmsThreads);
-    if (vec_ok && rows >= 1024 && nvec <= 64 * 8) {
+    if (vec_ok && rows >= 2048 && nvec <= 64 * (ADD ? 4 : 8)) {
+        // thousands of rows: every wavefront takes several, reads overlapping writes
+        const int64_t waves = std::min<int64_t>(rows / 2, int64_t(current_device_cus()) * 8);
+        const dim3 grid(unsigned((waves + 3) / 4));
+        if (nvec <= 64 * 4) {
+            hipLaunchKernelGGL((rms_norm_stream_kernel<4, ADD>), grid, block, 0, stream, x, res, w, sum_out, y, rows, C,
+                               eps);
+        } else if constexpr (!ADD) {
+            hipLaunchKernelGGL((rms_norm_stream_kernel<8, false>), grid, block, 0, stream, x, res, w, sum_out, y, rows,
+                               C, eps);
+        }
+    } else if (vec_ok && rows >= 1024 && nvec <= 64 * 8) {
         // plenty of rows: a wavefront per row, no workgroup barrier
         const dim3 grid(unsigned((rows + 3) / 4));
         if (nvec <= 64 * 4) {

@@ -32,7 +32,7 @@ def test_rms_norm_config_shapes(gpu, C, shape):
 
 
 @pytest.mark.parametrize("C", [8, 64, 100, 136, 2056, 5120, 8192, 8200, 16384])
-@pytest.mark.parametrize("rows", [3, 1100])
+@pytest.mark.parametrize("rows", [3, 1100, 2500])
 def test_rms_norm_other_widths(gpu, C, rows):
     """Widths off the fast paths: not a multiple of 8 (2-byte path), wider than the
     register-resident limit, and tiny."""
@@ -192,7 +192,8 @@ def test_rot_embed_append_fuses_rope_and_cache_write(gpu, HD, NH, KVH):
     np.testing.assert_array_equal(t2bits(ck), t2bits(ck0))
 
 
-@pytest.mark.parametrize("shape", [(1, 1, 2048), (64, 1, 2048), (2, 700, 4096), (1, 3, 136), (1, 5, 100), (1, 2, 8200)])
+@pytest.mark.parametrize("shape", [(1, 1, 2048), (64, 1, 2048), (2, 700, 4096), (1, 3, 136), (1, 5, 100), (1, 2, 8200),
+                                   (4, 1024, 2048), (3, 1001, 1000), (2, 2048, 4096)])
 def test_add_rms_norm_equals_add_then_norm(gpu, shape):
     from custom_kernels import custom_kernels_extension as cke
 
