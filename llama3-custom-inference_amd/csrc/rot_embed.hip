@@ -39,6 +39,52 @@ rot_embed_vec_kernel(const uint16_t* __restrict__ x, const float* __restrict__ f
     store16(y + item * 8, o);
 }
 
+// The same work with the index arithmetic taken out of the lanes: blockIdx.y is the batch row,
+// blockIdx.x a block of `rpw` tokens, and a thread's place in the workgroup gives (token, head
+// group, 16-byte chunk) -- by shifts when the counts are powers of two (POW2).  A thread rotates
+// chunk c of HG consecutive heads of its token with one read of the table row (the flat kernel
+// above spends most of its instructions on 64-bit divisions).  Needs vpr * NH / HG <= 256 threads
+// per token and B <= 65535.
+template <int HG, bool POW2>
+__global__ void __launch_bounds__(kRopeThreads)
+rot_embed_rows_kernel(const uint16_t* __restrict__ x, const float* __restrict__ freq, uint16_t* __restrict__ y, int T,
+                      int NH, int HD, int64_t sb, int64_t st, int64_t sh, int tpr, int vpr, int rpw, int tpr_shift,
+                      int vpr_shift) {
+    const int tid = threadIdx.x;
+    int rl, hq, c;
+    if constexpr (POW2) {
+        rl = tid >> tpr_shift;
+        const int j = tid & (tpr - 1);
+        hq = j >> vpr_shift;
+        c = j & (vpr - 1);
+    } else {
+        rl = tid / tpr;
+        const int j = tid - rl * tpr;
+        hq = j / vpr;
+        c = j - hq * vpr;
+    }
+    const int t = int(blockIdx.x) * rpw + rl;
+    if (rl >= rpw || t >= T) return;
+    const int64_t b = blockIdx.y;
+    const float4* fp = reinterpret_cast<const float4*>(freq + int64_t(t) * HD + c * 8);
+    const uint16_t* xp = x + b * sb + t * st + int64_t(hq * HG) * sh + c * 8;
+    uint4 xv[HG];
+#pragma unroll
+    for (int i = 0; i < HG; ++i) xv[i] = load16(xp + i * sh);
+    const float4 f0 = fp[0];
+    const float4 f1 = fp[1];
+    uint16_t* yp = y + ((b * T + t) * NH + hq * HG) * HD + c * 8;
+#pragma unroll
+    for (int i = 0; i < HG; ++i) {
+        uint4 o;
+        o.x = rotate_pair(xv[i].x, f0.x, f0.y);
+        o.y = rotate_pair(xv[i].y, f0.z, f0.w);
+        o.z = rotate_pair(xv[i].z, f1.x, f1.y);
+        o.w = rotate_pair(xv[i].w, f1.z, f1.w);
+        store16(yp + i * HD, o);
+    }
+}
+
 // Fallback: one pair per thread with 4-byte accesses (any even HD, 4-byte aligned rows).
 __global__ void __launch_bounds__(kRopeThreads)
 rot_embed_pair_kernel(const uint16_t* __restrict__ x, const float* __restrict__ freq, uint16_t* __restrict__ y,
@@ -134,7 +180,28 @@ int launch_rot_embed_append_partials(const float* part, int ksplit, int64_t spli
 int launch_rot_embed(const uint16_t* x, const float* freq, uint16_t* y, int B, int T, int NH, int HD,
                      int64_t sb, int64_t st, int64_t sh, bool vec_ok, hipStream_t stream) {
     const int64_t rows = int64_t(B) * T * NH;
-    if (vec_ok) {
+    const int vpr = HD / 8;
+    const int hg = (NH % 4 == 0) ? 4 : (NH % 2 == 0) ? 2 : 1;
+    const int tpr = vec_ok ? vpr * (NH / hg) : 0;
+    if (vec_ok && tpr <= kRopeThreads && B <= 65535) {
+        const int rpw = kRopeThreads / tpr;
+        const bool pow2 = (tpr & (tpr - 1)) == 0 && (vpr & (vpr - 1)) == 0;
+        const int tpr_shift = pow2 ? __builtin_ctz(unsigned(tpr)) : 0;
+        const int vpr_shift = pow2 ? __builtin_ctz(unsigned(vpr)) : 0;
+        const dim3 grid(unsigned((T + rpw - 1) / rpw), unsigned(B));
+        const dim3 block(kRopeThreads);
+#define L3_ROPE_ROWS(HG, POW2)                                                                                       \
+    hipLaunchKernelGGL((rot_embed_rows_kernel<HG, POW2>), grid, block, 0, stream, x, freq, y, T, NH, HD, sb, st, sh, \
+                       tpr, vpr, rpw, tpr_shift, vpr_shift)
+        if (hg == 4) {
+            if (pow2) L3_ROPE_ROWS(4, true); else L3_ROPE_ROWS(4, false);
+        } else if (hg == 2) {
+            if (pow2) L3_ROPE_ROWS(2, true); else L3_ROPE_ROWS(2, false);
+        } else {
+            if (pow2) L3_ROPE_ROWS(1, true); else L3_ROPE_ROWS(1, false);
+        }
+#undef L3_ROPE_ROWS
+    } else if (vec_ok) {
         const int64_t items = rows * (HD / 8);
         const unsigned blocks = unsigned((items + kRopeThreads - 1) / kRopeThreads);
         hipLaunchKernelGGL(rot_embed_vec_kernel, dim3(blocks), dim3(kRopeThreads), 0, stream, x, freq, y, items, T,
