@@ -120,19 +120,20 @@ rot_embed_append_kernel(const uint16_t* __restrict__ qkv, const float* __restric
                         int64_t c_sb, int64_t c_st, int cache_len, int table_rows) {
     const int item = blockIdx.x * kRopeThreads + threadIdx.x;
     if (item >= total_items) return;
-    const int pos = *pos_dev;
-    if (pos < 0 || pos >= cache_len || pos >= table_rows) return;  // never write outside the cache
     const int vpr = HD / 8;
     const int slots = NH + 2 * KVH;
     const int c = item % vpr;
     const int slot = (item / vpr) % slots;
     const int b = item / (vpr * slots);
+    // the projection does not depend on the position: its loads go out before the position is waited for
     uint4 xv;
     if constexpr (PART) {
         xv = sum_splits_bf16x8(part + b * qkv_sb + slot * HD + c * 8, ksplit, split_stride);
     } else {
         xv = load16(qkv + b * qkv_sb + slot * HD + c * 8);
     }
+    const int pos = *pos_dev;
+    if (pos < 0 || pos >= cache_len || pos >= table_rows) return;  // never write outside the cache
     if (slot >= NH + KVH) {  // value head: plain copy into the cache
         store16(cache_v + b * c_sb + pos * c_st + (slot - NH - KVH) * HD + c * 8, xv);
         return;
