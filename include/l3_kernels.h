@@ -269,15 +269,17 @@ int l3_linear_qkv_rope_append(const void* x, const void* norm_weight, float norm
 /*
  * Split-K form of l3_linear_decode for 17 .. 64 activation rows (hipBLASLt's territory in the
  * reference: nn.Linear at batch 64, model.py:95,121,134).  Eight wavefronts of a workgroup share
- * the activations of one k range through LDS and take 128 weight rows; K is split `ksplit` ways
- * across workgroups, each covering at most 512 k, and split s writes its float32 partial products
+ * the activations of one k range through LDS and take 128 weight rows (64, with the k range halved
+ * among them, for small matrices); K is split `ksplit` ways across workgroups, each covering at
+ * most 512 (1024) k, and split s writes its float32 partial products
  * to part[s][m][n] (M x N floats per split, contiguous).  The splits are NOT added up here: the
  * elementwise operator that follows the linear in a decode step does that on its way
  * (l3_add_rms_norm_partials, l3_rot_embed_append_partials), in split order, without atomics;
  * l3_linear_splitk_finish does it where there is no such operator.
  * l3_linear_splitk_plan returns the split count for a device with num_cus compute units (<= 0: the
  * current device); l3_linear_splitk_workspace_bytes the size of `part`.  1 <= M <=
- * L3_LINEAR_SPLITK_MAX_ROWS, N % 8 == 0, K % 128 == 0, ceil((K / 128) / ksplit) <= 4; strides and
+ * L3_LINEAR_SPLITK_MAX_ROWS, N % 8 == 0, K % 128 == 0, ceil((K / 128) / ksplit) <= 4 (<= 8 for a matrix
+ * with fewer than 32 rows per compute unit, which gets 64-row workgroups); strides and
  * alignment as for l3_linear_decode.  Meant for matrices of a few thousand rows, where the split
  * count fills the device; for a matrix whose rows alone do (a vocabulary projection), every split
  * costs M x N floats of traffic and a library GEMM is the better tool.

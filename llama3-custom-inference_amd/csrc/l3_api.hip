@@ -511,12 +511,14 @@ int l3_linear_splitk(const void* x, const void* w, void* part, size_t part_bytes
     if (!x || !w || !part) return L3_ERR_NULL_POINTER;
     if (M <= 0 || M > L3_LINEAR_SPLITK_MAX_ROWS || N <= 0 || K <= 0 || N % 8 != 0 || K % 128 != 0) return L3_ERR_SHAPE;
     if (N > (1 << 24) || K > (1 << 24)) return L3_ERR_SHAPE;
-    if (ksplit <= 0 || ksplit > K / 128 || (K / 128 + ksplit - 1) / ksplit > 4) return L3_ERR_SPLITS;
+    if (ksplit <= 0 || ksplit > K / 128 ||
+        (K / 128 + ksplit - 1) / ksplit > linear_splitk_max_chunks(N, current_device_cus()))
+        return L3_ERR_SPLITS;
     if (x_stride < K || w_stride < K || x_stride % 8 || w_stride % 8) return L3_ERR_STRIDE;
     if (!aligned(x, 16) || !aligned(w, 16) || !aligned(part, 16)) return L3_ERR_ALIGNMENT;
     if (part_bytes < l3_linear_splitk_workspace_bytes(M, N, ksplit)) return L3_ERR_WORKSPACE;
     return launch_linear_splitk(static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w),
-                                static_cast<float*>(part), M, N, K, x_stride, w_stride, ksplit,
+                                static_cast<float*>(part), M, N, K, x_stride, w_stride, ksplit, current_device_cus(),
                                 static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 

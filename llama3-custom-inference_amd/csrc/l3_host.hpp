@@ -104,8 +104,9 @@ int launch_rot_embed_append_partials(const float* part, int ksplit, int64_t spli
                                      uint16_t* q_out, uint16_t* cache_k, uint16_t* cache_v, const int* pos_dev, int B,
                                      int NH, int KVH, int HD, int64_t c_sb, int64_t c_st, int cache_len,
                                      int table_rows, hipStream_t stream);
+int linear_splitk_max_chunks(int N, int num_cus);
 int launch_linear_splitk(const uint16_t* x, const uint16_t* w, float* part, int M, int N, int K, int64_t x_stride,
-                         int64_t w_stride, int ksplit, hipStream_t stream);
+                         int64_t w_stride, int ksplit, int num_cus, hipStream_t stream);
 int launch_linear_splitk_finish(const float* part, int ksplit, const uint16_t* res, uint16_t* y, int M, int N,
                                 int64_t y_stride, hipStream_t stream);
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream);

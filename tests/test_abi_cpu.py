@@ -242,8 +242,9 @@ def test_linear_splitk_plan_and_argument_checks():
         ks = lib.l3_linear_splitk_plan(N, K, 256)
         chunks = K // 128
         per = -(-chunks // ks)
-        assert 1 <= ks <= chunks and per <= 4
-        assert per == 4 or -(-N // 128) * ks >= 192
+        assert 1 <= ks <= chunks and per <= (8 if -(-N // 128) < 64 else 4)
+        rows_per_wg = 64 if -(-N // 128) < 64 else 128      # few rows: 64-row groups, k range halved inside
+        assert per == (8 if rows_per_wg == 64 else 4) or -(-N // rows_per_wg) * ks >= 192
     assert lib.l3_linear_splitk_plan(2048, 2000, 256) == _l3lib.L3_ERR_SHAPE
     assert lib.l3_linear_splitk_workspace_bytes(64, 2048, 16) == 16 * 64 * 2048 * 4
 
@@ -253,7 +254,8 @@ def test_linear_splitk_plan_and_argument_checks():
     assert call(part=None) == _l3lib.L3_ERR_NULL_POINTER
     assert call(M=65) == _l3lib.L3_ERR_SHAPE
     assert call(N=2044) == _l3lib.L3_ERR_SHAPE
-    assert call(ks=2) == _l3lib.L3_ERR_SPLITS          # 1024 k per workgroup
+    assert call(ks=1) == _l3lib.L3_ERR_SPLITS          # 2048 k per workgroup: more than it stages
+    assert call(N=16384, ks=2) == _l3lib.L3_ERR_SPLITS # 128-row groups stage at most 512 k
     assert call(ks=17) == _l3lib.L3_ERR_SPLITS
     assert call(nbytes=1024) == _l3lib.L3_ERR_WORKSPACE
     assert _l3lib.L3_LINEAR_MAX_ROWS == 16 and _l3lib.L3_LINEAR_SPLITK_MAX_ROWS == 64

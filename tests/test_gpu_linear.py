@@ -215,7 +215,8 @@ def _sum_in_split_order(part):
 
 @pytest.mark.parametrize("M,N,K,ksplit", [(64, 3072, 2048, 0), (64, 2048, 2048, 0), (64, 2048, 8192, 0), (17, 2048, 2048, 4),
                                           (40, 264, 384, 1), (33, 8, 128, 1), (64, 16384, 2048, 4), (64, 2048, 2048, 16),
-                                          (20, 1000, 1280, 3)])
+                                          (20, 1000, 1280, 3), (20, 1000, 1280, 2), (33, 512, 896, 1), (17, 256, 768, 1),
+                                          (64, 2048, 8192, 8), (24, 8192, 384, 1), (64, 3072, 2048, 2)])
 def test_linear_splitk_against_oracle(gpu, M, N, K, ksplit):
     from custom_kernels import custom_kernels_extension as cke
 
@@ -267,7 +268,7 @@ def test_linear_splitk_errors(gpu):
 
     w = randn_bf16((256, 2048), 1).to(gpu)
     with pytest.raises(RuntimeError):
-        cke.linear_splitk(randn_bf16((64, 2048), 2).to(gpu), w, 2)        # 1024 k per workgroup: more than it stages
+        cke.linear_splitk(randn_bf16((64, 2048), 2).to(gpu), w, 1)        # 2048 k per workgroup: more than it stages
     with pytest.raises(RuntimeError):
         cke.linear_splitk(randn_bf16((64, 2048), 2).to(gpu), w, 17)       # more splits than 128-k chunks
     with pytest.raises(RuntimeError):
