@@ -2,6 +2,8 @@
 // silu(a) * b (model.py:134 evaluates it with two torch kernels) and the greedy argmax over the
 // logits row (model.py:371).  In a graph-replayed decode step both are dispatch-bound; one
 // launch each instead of two resp. a 40 us single-workgroup library reduction.
+#include <algorithm>
+
 #include "l3_device.hpp"
 #include "l3_host.hpp"
 
@@ -13,22 +15,24 @@ constexpr int kMiscThreads = 256;
 
 // y = bf16( bf16(silu(a)) * b ) with silu_rounded of l3_device.hpp.
 
+// blockIdx.y walks over the rows (no index division in the lanes); rows of a and b may be strided
+// (the two halves of one fused gate|up projection), y is dense.
 __global__ void __launch_bounds__(kMiscThreads)
 silu_mul_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b, uint16_t* __restrict__ y,
-                int64_t nvec, int64_t vec_per_row, int64_t a_row_stride, int64_t b_row_stride) {
-    const int64_t i = int64_t(blockIdx.x) * kMiscThreads + threadIdx.x;
-    if (i >= nvec) return;
-    // rows of a and b may be strided (the two halves of one fused gate|up projection); y is dense
-    const int64_t row = i / vec_per_row, col = i % vec_per_row;
-    float fa[8], fb[8];
-    unpack8(load16(a + row * a_row_stride + col * 8), fa);
-    unpack8(load16(b + row * b_row_stride + col * 8), fb);
-    uint4 o;
-    o.x = pack_bf16x2(silu_rounded(fa[0]) * fb[0], silu_rounded(fa[1]) * fb[1]);
-    o.y = pack_bf16x2(silu_rounded(fa[2]) * fb[2], silu_rounded(fa[3]) * fb[3]);
-    o.z = pack_bf16x2(silu_rounded(fa[4]) * fb[4], silu_rounded(fa[5]) * fb[5]);
-    o.w = pack_bf16x2(silu_rounded(fa[6]) * fb[6], silu_rounded(fa[7]) * fb[7]);
-    store16(y + i * 8, o);
+                int64_t rows, int64_t vec_per_row, int64_t a_row_stride, int64_t b_row_stride) {
+    const int64_t col = int64_t(blockIdx.x) * kMiscThreads + threadIdx.x;
+    if (col >= vec_per_row) return;
+    for (int64_t row = blockIdx.y; row < rows; row += gridDim.y) {
+        float fa[8], fb[8];
+        unpack8(load16(a + row * a_row_stride + col * 8), fa);
+        unpack8(load16(b + row * b_row_stride + col * 8), fb);
+        uint4 o;
+        o.x = pack_bf16x2(silu_rounded(fa[0]) * fb[0], silu_rounded(fa[1]) * fb[1]);
+        o.y = pack_bf16x2(silu_rounded(fa[2]) * fb[2], silu_rounded(fa[3]) * fb[3]);
+        o.z = pack_bf16x2(silu_rounded(fa[4]) * fb[4], silu_rounded(fa[5]) * fb[5]);
+        o.w = pack_bf16x2(silu_rounded(fa[6]) * fb[6], silu_rounded(fa[7]) * fb[7]);
+        store16(y + (row * vec_per_row + col) * 8, o);
+    }
 }
 
 __global__ void __launch_bounds__(kMiscThreads)
@@ -175,9 +179,10 @@ int launch_greedy_step(const uint16_t* logits, int64_t row_stride, int rows, int
 
 int launch_silu_mul_rows(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t rows, int64_t cols,
                          int64_t a_row_stride, int64_t b_row_stride, hipStream_t stream) {
-    const int64_t nvec = rows * (cols / 8);
-    hipLaunchKernelGGL(silu_mul_kernel, dim3(unsigned((nvec + kMiscThreads - 1) / kMiscThreads)), dim3(kMiscThreads), 0,
-                       stream, a, b, y, nvec, cols / 8, a_row_stride, b_row_stride);
+    const int64_t vpr = cols / 8;
+    const dim3 grid(unsigned((vpr + kMiscThreads - 1) / kMiscThreads), unsigned(std::min<int64_t>(rows, 65535)));
+    hipLaunchKernelGGL(silu_mul_kernel, grid, dim3(kMiscThreads), 0, stream, a, b, y, rows, vpr, a_row_stride,
+                       b_row_stride);
     return int(hipGetLastError());
 }
 
@@ -185,7 +190,7 @@ int launch_silu_mul(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n
     if (vec_ok) {
         const int64_t nvec = n / 8;
         hipLaunchKernelGGL(silu_mul_kernel, dim3(unsigned((nvec + kMiscThreads - 1) / kMiscThreads)),
-                           dim3(kMiscThreads), 0, stream, a, b, y, nvec, nvec, int64_t(0), int64_t(0));
+                           dim3(kMiscThreads), 0, stream, a, b, y, int64_t(1), nvec, int64_t(0), int64_t(0));
     } else {
         hipLaunchKernelGGL(silu_mul_scalar_kernel, dim3(unsigned((n + kMiscThreads - 1) / kMiscThreads)),
                            dim3(kMiscThreads), 0, stream, a, b, y, n);

@@ -183,11 +183,10 @@ linear_splitk_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
 __global__ void __launch_bounds__(256)
 linear_splitk_finish_kernel(const float* __restrict__ part, int ksplit, int64_t split_stride,
                             const uint16_t* __restrict__ res, uint16_t* __restrict__ y, int M, int N, int64_t y_stride) {
-    const int nvec = N / 8;
-    const int64_t item = int64_t(blockIdx.x) * 256 + threadIdx.x;
-    if (item >= int64_t(M) * nvec) return;
-    const int m = int(item / nvec);
-    const int n = int(item % nvec) * 8;
+    const int vi = int(blockIdx.x) * 256 + threadIdx.x;   // blockIdx.y is the activation row
+    if (vi >= N / 8) return;
+    const int m = blockIdx.y;
+    const int n = vi * 8;
     uint4 o = sum_splits_bf16x8(part + int64_t(m) * N + n, ksplit, split_stride);
     if (res) {
         float a[8], b[8];
@@ -205,9 +204,8 @@ linear_splitk_finish_kernel(const float* __restrict__ part, int ksplit, int64_t 
 
 int launch_linear_splitk_finish(const float* part, int ksplit, const uint16_t* res, uint16_t* y, int M, int N,
                                 int64_t y_stride, hipStream_t stream) {
-    const int64_t items = int64_t(M) * (N / 8);
-    hipLaunchKernelGGL(linear_splitk_finish_kernel, dim3(unsigned((items + 255) / 256)), dim3(256), 0, stream, part,
-                       ksplit, int64_t(M) * N, res, y, M, N, y_stride);
+    hipLaunchKernelGGL(linear_splitk_finish_kernel, dim3(unsigned((N / 8 + 255) / 256), unsigned(M)), dim3(256), 0,
+                       stream, part, ksplit, int64_t(M) * N, res, y, M, N, y_stride);
     return int(hipGetLastError());
 }
 

@@ -166,7 +166,6 @@ rms_norm_stream_kernel(const uint16_t* __restrict__ x, const uint16_t* __restric
             }
         }
         if (!has_next) break;
-#pragma unroll
         for (int j = 0; j < MAXV; ++j) {
             cur[j] = nxt[j];
             if constexpr (ADD) rcur[j] = rnxt[j];
