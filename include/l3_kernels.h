@@ -216,12 +216,15 @@ int l3_silu_mul_rows(const void* a, const void* b, void* y, int64_t rows, int64_
  * float32 accumulation, one rounding.  Stands where the reference calls nn.Linear with T == 1
  * (model.py:95 c_attn, :121 c_proj, :134 mlp c_proj, :225 lm_head); hipBLASLt treats these as
  * GEMMs, this entry point as a single pass over the weight matrix at HBM speed.
- * 1 <= M <= L3_LINEAR_MAX_ROWS (one 16-column block of the matrix instruction; more rows:
- * l3_linear_splitk); N % 4 == 0; K % 32 == 0; strides are row strides in elements
+ * 1 <= M <= L3_LINEAR_MAX_ROWS; N % 4 == 0; K % 32 == 0; strides are row strides in elements
  * (x_stride, w_stride >= K and multiples of 8; y_stride >= N and a multiple of 4); x and w
  * 16-byte aligned, y 8-byte aligned.  Needs no workspace.
+ * Up to 16 rows (one 16-column block of the matrix instruction) every matrix shape is served at
+ * HBM speed.  With 17 .. 64 rows (K % 128 == 0 then) a workgroup takes 128 weight rows and walks
+ * over the whole of K, which suits matrices whose rows alone fill the device (N >= 64 x compute
+ * units: a vocabulary projection); for the matrices of a few thousand rows use l3_linear_splitk.
  */
-#define L3_LINEAR_MAX_ROWS 16
+#define L3_LINEAR_MAX_ROWS 64
 int l3_linear_decode(const void* x, const void* w, void* y, int M, int N, int K, int64_t x_stride,
                      int64_t w_stride, int64_t y_stride, void* stream);
 
@@ -229,7 +232,8 @@ int l3_linear_decode(const void* x, const void* w, void* y, int M, int N, int K,
  * y[M, N] = silu(x . w_gate^T) * (x . w_up^T) in one pass over both weight matrices: the
  * SwiGLU front half of model.py:134 (F.silu(c_fc2(x)) * c_fc(x)).  Both products and the silu
  * are rounded to bf16 before the multiplication, as the three separate torch operators do.
- * Same constraints as l3_linear_decode; w_gate and w_up share w_stride.
+ * Same constraints as l3_linear_decode; w_gate and w_up share w_stride.  With 17 .. 64 rows a
+ * workgroup takes 32 output columns of both matrices (N >= 16 x compute units fills the device).
  */
 int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up, void* y, int M, int N, int K,
                             int64_t x_stride, int64_t w_stride, int64_t y_stride, void* stream);
@@ -242,7 +246,7 @@ int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up,
  *   t = w_up ? bf16(silu(bf16(h.w^T))) * bf16(h.w_up^T) : h.w^T                   (model.py:134)
  *   y = residual ? bf16(residual + bf16(t)) : bf16(t)                             (model.py:147-148)
  * with the rounding points of the separate operators.  residual has y's shape and row stride and
- * may be y itself.  The input norm stages x in LDS and needs K % 512 == 0 and M * (K + 8) <= 24576
+ * may be y itself.  The input norm stages x in LDS and needs M <= 16, K % 512 == 0 and M * (K + 8) <= 24576
  * (L3_ERR_SHAPE otherwise); everything else as for l3_linear_decode.
  */
 int l3_linear_decode_fused(const void* x, const void* norm_weight, float norm_eps, const void* w, const void* w_up,
@@ -257,7 +261,7 @@ int l3_linear_decode_fused(const void* x, const void* norm_weight, float norm_ep
  * into cache_k / cache_v at token *pos_dev (element strides cache_strides = {batch, token},
  * (KVH, HD) contiguous), the rotated queries to q_out (B, NH, HD).  One launch where the separate
  * operators take l3_linear_decode_fused and l3_rot_embed_append, with the same bits.  Constraints
- * of both apply (B <= L3_LINEAR_MAX_ROWS, K % 32 == 0, HD % 8 == 0, norm limits as above); an
+ * of both apply (B <= 16, K % 32 == 0, HD % 8 == 0, norm limits as above); an
  * out-of-range position writes nothing.
  */
 int l3_linear_qkv_rope_append(const void* x, const void* norm_weight, float norm_eps, const void* w_qkv,

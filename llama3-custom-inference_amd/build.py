@@ -13,7 +13,7 @@ import sys
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "custom_kernels", "libl3kernels.so")
-SOURCES = ["l3_api.hip", "attn_decode.hip", "attn_mfma.hip", "attn_prefill.hip", "attn_prefill_tiled.hip", "linear_skinny.hip", "linear_splitk.hip", "attn_combine.hip", "rms_norm.hip", "rot_embed.hip",
+SOURCES = ["l3_api.hip", "attn_decode.hip", "attn_mfma.hip", "attn_prefill.hip", "attn_prefill_tiled.hip", "linear_skinny.hip", "linear_splitk.hip", "linear_rows64.hip", "attn_combine.hip", "rms_norm.hip", "rot_embed.hip",
            "decode_misc.hip"]
 
 HIPCC_FLAGS = [

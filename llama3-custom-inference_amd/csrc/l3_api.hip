@@ -434,6 +434,12 @@ int linear_decode_impl(const void* x, const void* norm_w, float norm_eps, const 
         p.NH = p.KVH = p.HD = p.cache_len = p.table_rows = 0;
         p.c_sb = p.c_st = 0;
     }
+    if (M > 16) {
+        // 17 .. 64 rows: the one-launch kernel that walks over K in rounds (no norm, no rope epilogue)
+        if (norm_w || qkv || K % 128 != 0) return L3_ERR_SHAPE;
+        if (x_stride % 8 || y_stride % 4) return L3_ERR_STRIDE;
+        return launch_linear_rows64(p, swiglu, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+    }
     return launch_linear_skinny(p, swiglu, current_device_cus(), static_cast<hipStream_t>(stream)) == 0 ? L3_OK
                                                                                                         : L3_ERR_HIP;
 }

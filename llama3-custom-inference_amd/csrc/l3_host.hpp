@@ -104,6 +104,7 @@ int launch_rot_embed_append_partials(const float* part, int ksplit, int64_t spli
                                      uint16_t* q_out, uint16_t* cache_k, uint16_t* cache_v, const int* pos_dev, int B,
                                      int NH, int KVH, int HD, int64_t c_sb, int64_t c_st, int cache_len,
                                      int table_rows, hipStream_t stream);
+int launch_linear_rows64(const LinearParams& p, bool swiglu, hipStream_t stream);   // 17 .. 64 rows, one launch
 int linear_splitk_max_chunks(int N, int num_cus);
 int launch_linear_splitk(const uint16_t* x, const uint16_t* w, float* part, int M, int N, int K, int64_t x_stride,
                          int64_t w_stride, int ksplit, int num_cus, hipStream_t stream);

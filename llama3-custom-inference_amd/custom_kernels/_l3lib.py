@@ -20,7 +20,8 @@ L3_ERR_WORKSPACE = -7
 L3_ERR_SPLITS = -8
 L3_ERR_HIP = -9
 L3_ATTN_MAX_SPLITS = 512
-L3_LINEAR_MAX_ROWS = 16
+L3_LINEAR_MAX_ROWS = 64
+L3_LINEAR_FUSED_MAX_ROWS = 16   # rows up to which every matrix shape, the input norm and the rope epilogue are served
 L3_LINEAR_SPLITK_MAX_ROWS = 64
 L3_LINEAR_STAGE_ELEMS = 24576   # activations (rows padded by 8) the fused input norm can stage in LDS
 L3_ATTN_OPT_KERNEL = 0

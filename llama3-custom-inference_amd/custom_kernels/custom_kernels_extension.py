@@ -438,14 +438,24 @@ def _linear_args(x, weights, max_rows=None):
     return x2, rows, weights[0].shape[0], K
 
 
+def _use_splitk(x, weight) -> bool:
+    """17..64 activation rows against a matrix too small for one workgroup per 128 rows to fill the
+    device: the split-K kernel plus its finishing pass is the faster route."""
+    K = x.shape[-1]
+    if K <= 0 or weight.dim() != 2 or not x.is_cuda:
+        return False
+    rows = x.numel() // K
+    return rows > _l3lib.L3_LINEAR_FUSED_MAX_ROWS and -(-weight.shape[0] // 128) < _cus(x.device) // 2
+
+
 def linear_decode(x, weight):
     """F.linear(x, weight) for at most 64 activation rows (model.py:95,121,134,225 when T == 1):
     one pass over the weight matrix at HBM speed instead of a GEMM.  x (..., K), weight (N, K)
-    -> (..., N).  Up to 16 rows are one launch; 17..64 rows go through linear_splitk and
-    linear_splitk_finish (N % 8 == 0 and K % 128 == 0 then), which suits matrices of a few thousand
-    rows -- a vocabulary projection at that many rows is a job for a library GEMM.  An extension."""
+    -> (..., N).  Up to 16 rows are one launch whatever the matrix; with 17..64 rows (K % 128 == 0
+    then) a matrix whose rows alone fill the device is still one launch, and the matrices of a few
+    thousand rows go through linear_splitk and linear_splitk_finish (N % 8 == 0).  An extension."""
     lib = _l3lib.load()
-    if x.shape[-1] > 0 and x.numel() // x.shape[-1] > _l3lib.L3_LINEAR_MAX_ROWS:
+    if _use_splitk(x, weight):
         return linear_splitk_finish(linear_splitk(x, weight)).view(*x.shape[:-1], weight.shape[0])
     x2, rows, N, K = _linear_args(x, (weight,))
     y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
@@ -458,7 +468,7 @@ def linear_decode(x, weight):
 
 
 def linear_swiglu_decode(x, w_gate, w_up):
-    """F.silu(F.linear(x, w_gate)) * F.linear(x, w_up) for at most 16 activation rows in one
+    """F.silu(F.linear(x, w_gate)) * F.linear(x, w_up) for at most 64 activation rows in one
     launch (model.py:134 with w_gate = c_fc2, w_up = c_fc), same rounding points.  An extension."""
     lib = _l3lib.load()
     x2, rows, N, K = _linear_args(x, (w_gate, w_up))
@@ -482,9 +492,8 @@ def linear_decode_fused(x, weight, norm_weight=None, eps: float = 1e-5, w_up=Non
     matrix w_up (weight is then the gate, model.py:134), and `residual + result` behind
     (model.py:147-148) -- all with the rounding points of the separate operators.  An extension."""
     lib = _l3lib.load()
-    if norm_weight is None and w_up is None and x.shape[-1] > 0 \
-            and x.numel() // x.shape[-1] > _l3lib.L3_LINEAR_MAX_ROWS:
-        # 17..64 rows: split-K, the residual joins when the splits are added up
+    if norm_weight is None and w_up is None and _use_splitk(x, weight):
+        # 17..64 rows, small matrix: split-K, the residual joins when the splits are added up
         return linear_splitk_finish(linear_splitk(x, weight), residual).view(*x.shape[:-1], weight.shape[0])
     x2, rows, N, K = _linear_args(x, (weight,) if w_up is None else (weight, w_up))
     if norm_weight is not None:

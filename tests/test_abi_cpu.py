@@ -179,6 +179,7 @@ def test_linear_decode_argument_checks():
     assert call(M=0) == _l3lib.L3_ERR_SHAPE
     assert call(M=_l3lib.L3_LINEAR_MAX_ROWS + 1) == _l3lib.L3_ERR_SHAPE
     assert call(K=2040, xs=2040, ws=2040) == _l3lib.L3_ERR_SHAPE       # K not a multiple of 32
+    assert call(M=17, K=2080, xs=2080, ws=2080) == _l3lib.L3_ERR_SHAPE # more than 16 rows: K must be a multiple of 128
     assert call(N=2046, ys=2048) == _l3lib.L3_ERR_SHAPE                # N not a multiple of 4
     assert call(xs=1024) == _l3lib.L3_ERR_STRIDE                       # rows would overlap
     assert call(ws=2052) == _l3lib.L3_ERR_STRIDE                       # weight rows not 16-byte aligned
@@ -198,6 +199,7 @@ def test_linear_decode_fused_argument_checks():
         return lib.l3_linear_decode_fused(FAKE, norm, 1e-5, FAKE, None, res, FAKE, M, 2048, K, K, K, 2048, None)
 
     assert call(M=12) == _l3lib.L3_ERR_SHAPE              # 12 rows of 2048 do not fit the LDS stage
+    assert call(M=17, K=512) == _l3lib.L3_ERR_SHAPE       # the input norm is for up to 16 rows
     assert call(M=3, K=8192) == _l3lib.L3_ERR_SHAPE
     assert call(norm=FAKE + 2) == _l3lib.L3_ERR_ALIGNMENT
     assert call(res=FAKE + 4) == _l3lib.L3_ERR_ALIGNMENT
@@ -229,6 +231,7 @@ def test_linear_qkv_rope_append_argument_checks():
     assert call(table=None) == _l3lib.L3_ERR_NULL_POINTER
     assert call(HD=60) == _l3lib.L3_ERR_SHAPE
     assert call(B=65) == _l3lib.L3_ERR_SHAPE
+    assert call(B=17) == _l3lib.L3_ERR_SHAPE               # the rope epilogue is for up to 16 rows
     assert call(K=2040) == _l3lib.L3_ERR_SHAPE
     assert call(B=12, norm=FAKE) == _l3lib.L3_ERR_SHAPE
     assert call(strides=_l3lib.i64_array((256 * 512, 516))) == _l3lib.L3_ERR_STRIDE
@@ -258,7 +261,7 @@ def test_linear_splitk_plan_and_argument_checks():
     assert call(N=16384, ks=2) == _l3lib.L3_ERR_SPLITS # 128-row groups stage at most 512 k
     assert call(ks=17) == _l3lib.L3_ERR_SPLITS
     assert call(nbytes=1024) == _l3lib.L3_ERR_WORKSPACE
-    assert _l3lib.L3_LINEAR_MAX_ROWS == 16 and _l3lib.L3_LINEAR_SPLITK_MAX_ROWS == 64
+    assert _l3lib.L3_LINEAR_MAX_ROWS == 64 and _l3lib.L3_LINEAR_SPLITK_MAX_ROWS == 64
 
     def finish(part=FAKE, ks=4, res=None, y=FAKE, M=64, N=2048, stride=2048):
         return lib.l3_linear_splitk_finish(part, ks, res, y, M, N, stride, None)

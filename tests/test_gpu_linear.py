@@ -30,7 +30,7 @@ def assert_linear_close(y, ref, what):
 SHAPES = [(1, 3072, 2048), (1, 2048, 2048), (1, 2048, 8192), (1, 128256, 2048), (3, 1024, 512), (16, 3072, 2048),
           (17, 512, 256), (64, 3072, 2048), (64, 2048, 8192), (5, 20, 32), (2, 36, 64), (33, 104, 384),
           (64, 16, 4096), (1, 16, 32), (8, 6144, 4096), (4, 2048, 8192), (4, 20, 128), (2, 3072, 2048), (3, 4, 384),
-          (16, 100, 96), (40, 2048, 2048)]
+          (16, 100, 96), (40, 2048, 2048), (64, 32768, 2048), (17, 20000, 1152), (33, 16388, 384)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -74,7 +74,9 @@ def test_linear_decode_layouts_and_errors(gpu):
         cke.linear_decode(randn_bf16((2, K), 1), w)                   # CPU tensor
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 8192, 2048), (12, 8192, 2048), (7, 1024, 256), (16, 14336, 4096), (9, 52, 64)])
+@pytest.mark.parametrize("M,N,K", [(1, 8192, 2048), (12, 8192, 2048), (7, 1024, 256), (16, 14336, 4096), (9, 52, 64),
+                                   (64, 8192, 2048), (17, 8192, 2048), (40, 52, 640), (33, 1000, 1408), (64, 14336, 4096),
+                                   (20, 96, 128)])
 def test_linear_swiglu_decode(gpu, M, N, K):
     from custom_kernels import custom_kernels_extension as cke
 
@@ -88,8 +90,17 @@ def test_linear_swiglu_decode(gpu, M, N, K):
     assert y.shape == (M, N)
     # the fused kernel accumulates in the same order as the plain one: the three-operator sequence
     # gives the same bits
-    seq = cke.silu_mul(cke.linear_decode(xd, wgd), cke.linear_decode(xd, wud))
-    assert torch.equal(y, seq)
+    if M > 16 and N % 8:
+        seq = y          # the split-K route of the plain linear needs N % 8 == 0: oracle only
+    else:
+        seq = cke.silu_mul(cke.linear_decode(xd, wgd), cke.linear_decode(xd, wud))
+    if M <= 16:
+        assert torch.equal(y, seq)
+    else:
+        # above 16 rows the plain linear may add its k ranges up in another order (split-K): a gate or
+        # up value can round the other way now and then
+        dseq = bf16_ulp_distance(t2bits(y), t2bits(seq))
+        assert (dseq > 0).mean() < 0.02 and (dseq > 2).mean() < 2e-3
     # against exact arithmetic with the same rounding points: a gate or up value that rounds the other
     # way moves the product by about one ulp of that factor
     ref = swiglu_linear_ref(t2f32(x), t2f32(wg), t2f32(wu))
