@@ -58,7 +58,8 @@ class AttnCase:
     """One attention shape with `slots` independent copies of its inputs, pre-allocated outputs
     and workspace, launched straight through the C ABI (no per-call allocation)."""
 
-    def __init__(self, torch, lib, l3, dev, B, QH, KVH, S, HD, slots, src_k=None, src_v=None, src_q=None):
+    def __init__(self, torch, lib, l3, dev, B, QH, KVH, S, HD, slots, src_k=None, src_v=None, src_q=None,
+                 cache_len=0):
         self.torch, self.lib = torch, lib
         self.B, self.QH, self.KVH, self.S, self.HD = B, QH, KVH, S, HD
         self.bytes = attn_bytes(B, QH, KVH, S, HD)
@@ -70,8 +71,17 @@ class AttnCase:
         self.cpu = (q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
         # token-major storage, transposed views: the model's cache layout (benchmark_kernel.py:165-173)
         self.q = [q.to(dev).transpose(1, 2) for _ in range(slots)]
-        self.k = [k.to(dev).transpose(1, 2) for _ in range(slots)]
-        self.v = [v.to(dev).transpose(1, 2) for _ in range(slots)]
+        if cache_len > S:
+            # the model's layout (model.py:107-111): a (B, L, KVH, HD) cache of which the first S tokens are attended
+            def cache_view(t):
+                full = torch.zeros((B, cache_len, KVH, HD), dtype=torch.bfloat16, device=dev)
+                full[:, :S] = t.to(dev)
+                return full[:, :S].transpose(1, 2)
+            self.k = [cache_view(k) for _ in range(slots)]
+            self.v = [cache_view(v) for _ in range(slots)]
+        else:
+            self.k = [k.to(dev).transpose(1, 2) for _ in range(slots)]
+            self.v = [v.to(dev).transpose(1, 2) for _ in range(slots)]
         self.out = [torch.empty_like(t) for t in self.q]
         # 0 = the library plans for the current device (split count and kernel form)
         self.req_splits = FORCE_SPLITS
@@ -180,8 +190,10 @@ def run_attention(args, torch, lib, l3, dev, name):
     # enough copies that a pass over all of them moves > 1 GiB between two uses of the same bytes
     slots = max(4, int(math.ceil((1 << 30) / pass_bytes)))
     slots = min(slots, 64)
+    if args.cache_len:
+        label += f" [K/V are views of (B, {args.cache_len}, KVH, HD) caches]"
     cases = [AttnCase(torch, lib, l3, dev, B, QH, KVH, S, HD, slots, src_k=k[:, :S].contiguous(),
-                      src_v=v[:, :S].contiguous(), src_q=q) for S in lengths]
+                      src_v=v[:, :S].contiguous(), src_q=q, cache_len=args.cache_len) for S in lengths]
 
     def one_pass(slot):
         sp = torch.cuda.current_stream().cuda_stream
@@ -540,6 +552,8 @@ def main():
                     help="split-KV kernel to measure (default: the library's choice)")
     ap.add_argument("--splits", type=int, default=0, help="force the split count (0 = the library's choice)")
     ap.add_argument("--lengths", default="", help="comma-separated KV lengths replacing the workload's own (experiments)")
+    ap.add_argument("--cache-len", type=int, default=0,
+                    help="attention workloads: K/V as views of caches this many tokens long (the model's batch stride)")
     args = ap.parse_args()
 
     global FORCE_SPLITS
