@@ -440,7 +440,8 @@ def run_prefill(args, torch, lib, l3, dev):
 def run_linear(args, torch, lib, l3, dev):
     """The nn.Linear calls of one decode step of the 1B architecture (model.py:95,121,134,225) at
     batch 1 (l3_linear_decode / l3_linear_swiglu_decode) and 64 (l3_linear_splitk + finish for the
-    three matrices of a few thousand rows): a stream over the weight matrix, priced against HBM.  Each shape owns enough weight copies that the Infinity Cache
+    three matrices of a few thousand rows, l3_linear_swiglu_decode for the gate|up pair): a stream
+    over the weight matrix, priced against HBM.  Each shape owns enough weight copies that the Infinity Cache
     cannot hold them; stock F.linear (hipBLASLt) on the same tensors is timed beside it."""
     import torch.nn.functional as F
     from custom_kernels import custom_kernels_extension as cke
@@ -465,9 +466,8 @@ def run_linear(args, torch, lib, l3, dev):
                 # up to 16 rows: l3_linear_decode; 64 rows: l3_linear_splitk + l3_linear_splitk_finish
                 run_l3 = lambda: [cke.linear_decode(x, a) for a in ws]  # noqa: E731
                 run_t = lambda: [F.linear(x, a) for a in ws]  # noqa: E731
-            # At 64 rows the SwiGLU pair and the vocabulary projection stay with the library GEMM (as in the
-            # end-to-end harness): their rows alone fill the device, so splitting K only adds traffic.
-            library = M > 16 and (swiglu or N > 32768)
+            # At 64 rows the vocabulary projection stays with the library GEMM (as in the end-to-end harness).
+            library = M > 16 and not swiglu and N > 32768
             if library:
                 run_l3 = run_t
             run_l3()
@@ -485,8 +485,8 @@ def run_linear(args, torch, lib, l3, dev):
                            "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
                            "bytes": nbytes, "torch_us": round(tms * 1e3, 2),
                            "path": "F.linear (library GEMM)" if library else
-                                   ("l3_linear_splitk + l3_linear_splitk_finish" if M > 16 else
-                                    ("l3_linear_swiglu_decode" if swiglu else "l3_linear_decode"))})
+                                   ("l3_linear_swiglu_decode" if swiglu else
+                                    ("l3_linear_splitk + l3_linear_splitk_finish" if M > 16 else "l3_linear_decode"))})
             per_token = 1 if name == "lm_head" else 16
             total_us += ms * 1e3 * per_token
             torch_us += tms * 1e3 * per_token
