@@ -41,6 +41,11 @@ FORCE_SPLITS = 0        # --splits
 MEASURED_TRAFFIC = {
     # profiles/attn_splitkv_mfma_c2_sweep_hbm_traffic.md: 38.21 MB fetched + 2.47 MB written per launch
     ("c2", "attn_splitkv_mfma_kernel"): 40680000,
+    # profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md (largest shape of each workload)
+    ("c3a", "attn_splitkv_mfma_kernel"): 136660000,   # 135.37 MB fetched + 1.29 MB written
+    ("c3b", "attn_splitkv_mfma_kernel"): 136550000,   # 134.39 MB fetched + 2.16 MB written (partials)
+    ("rms", "rms_norm_stream_kernel"): 67270000,      # 4096 x 4096: 33.72 MB fetched + 33.55 MB written
+    ("rope", "rot_embed_rows_kernel"): 68670000,      # 4096 x 32 x 128: 35.12 MB fetched + 33.55 MB written
 }
 
 
@@ -365,7 +370,11 @@ def run_rows(args, torch, lib, l3, dev, name):
         "steps": args.steps, "ms_per_step": round(ms, 5), "dtype": "bf16",
         "config": {"workload": label, "accumulate": "f32", "launch": "hip graph", "seed": SEED},
         "roofline": {"bound": "hbm", "achieved": rec["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": rec["frac"], "traffic": None, "algorithmic_bytes_per_launch": nbytes},
+                     "frac": rec["frac"],
+                     "traffic": MEASURED_TRAFFIC.get((name, "rms_norm_stream_kernel" if name == "rms"
+                                                      else "rot_embed_rows_kernel")),
+                     "kernel": "rms_norm_stream_kernel" if name == "rms" else "rot_embed_rows_kernel",
+                     "algorithmic_bytes_per_launch": nbytes},
         "cpu_baseline": cpu, "per_shape": detail,
     }
 
