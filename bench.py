@@ -600,7 +600,16 @@ def main():
     else:
         import llama_arch
 
-        res = llama_arch.bench_e2e(args, torch, dev)
+        cpu_ops = None
+        if not args.no_cpu_baseline:
+            from oracle import cpu_baseline
+
+            class cpu_ops:
+                rms_norm = staticmethod(cpu_baseline.rms_norm_cpu)
+                rot_embed = staticmethod(cpu_baseline.rot_embed_cpu)
+                flash_attention_decode = staticmethod(cpu_baseline.attention_cpu)
+
+        res = llama_arch.bench_e2e(args, torch, dev, cpu_ops)
 
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
             "steps": res.pop("steps"), "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),

@@ -469,10 +469,12 @@ def e2e_summary(torch_mod, dev, batches=(1, 64), input_len=128, gen_len=128, rep
     return out
 
 
-def bench_e2e(args, torch_mod, dev):
+def bench_e2e(args, torch_mod, dev, cpu_ops=None):
     """bench.py --workload e2e: the end-to-end configuration (16 layers, hidden 2048, 32/8 heads, head_dim 64,
     FFN 8192, vocab 128256 tied, N(0, 0.02) weights, 128 random prompt ids + 128 greedy tokens) at
-    batch 1 and 64, every RMSNorm / rotary / decode-attention call going through the HIP operators."""
+    batch 1 and 64, every RMSNorm / rotary / decode-attention call going through the HIP operators.
+    `cpu_ops` (an object with rms_norm, rot_embed and flash_attention_decode working on CPU tensors) is the
+    caller's operator table for the timed CPU baseline; without one no baseline is reported."""
     import os
 
     from custom_kernels import custom_kernels_extension as cke
@@ -514,16 +516,9 @@ def bench_e2e(args, torch_mod, dev):
         torch_mod.cuda.empty_cache()
 
     cpu = None
-    if not args.no_cpu_baseline:
-        from oracle import cpu_baseline
-
-        class _CpuOps:
-            rms_norm = staticmethod(cpu_baseline.rms_norm_cpu)
-            rot_embed = staticmethod(cpu_baseline.rot_embed_cpu)
-            flash_attention_decode = staticmethod(cpu_baseline.attention_cpu)
-
+    if cpu_ops is not None:
         cfg = LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=1)
-        cpu_model = LlamaDecoder(cfg, _CpuOps, "cpu")
+        cpu_model = LlamaDecoder(cfg, cpu_ops, "cpu")
         short = 16
         tps, dt, _ = timed_generate(cpu_model, 1, input_len, short)
         cpu = {"value": round(tps, 2), "unit": "tokens/s", "cores": torch_mod.get_num_threads(), "kind": "port",
