@@ -190,5 +190,17 @@ def strerror(code: int) -> str:
     return load().l3_strerror(int(code)).decode()
 
 
+_i64_arrays = {}
+
+
 def i64_array(values):
-    return (ctypes.c_int64 * len(values))(*[int(v) for v in values])
+    """A C array of int64 holding `values` (a sequence of ints).  Stride tuples repeat from call to
+    call, so the arrays are kept; callers only ever pass them as read-only arguments."""
+    if not isinstance(values, tuple):
+        values = tuple(values)
+    arr = _i64_arrays.get(values)
+    if arr is None:
+        arr = (ctypes.c_int64 * len(values))(*[int(v) for v in values])
+        if len(_i64_arrays) < 4096:
+            _i64_arrays[values] = arr
+    return arr

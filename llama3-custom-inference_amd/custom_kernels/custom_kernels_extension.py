@@ -12,6 +12,7 @@ Kernels are enqueued on torch's current stream of the input's device and the cal
 not synchronise.  There is no fallback path: a missing library or a non-GPU tensor raises.
 """
 
+import contextlib
 import math
 
 import torch
@@ -41,8 +42,26 @@ def _require_gpu_bf16(name: str, t: torch.Tensor):
         raise RuntimeError(f"expected scalar type BFloat16 for {name} but found {t.dtype}")
 
 
+# The raw handle of torch's current stream without building a Stream object (2 us per call saved);
+# the public accessor is the fallback where this build of torch does not have the direct one.
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_NO_GUARD = contextlib.nullcontext()
+
+
 def _stream_ptr(device) -> int:
+    if _raw_current_stream is not None:
+        idx = device.index
+        return _raw_current_stream(idx if idx is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
+
+
+def _on_device(device):
+    """Context in which `device` is the current one: nothing to do (and nothing to pay) when it
+    already is, which is every call of a single-GPU process."""
+    idx = device.index
+    if idx is None or idx == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(idx)
 
 
 def _cus(device) -> int:
@@ -99,7 +118,7 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0):
     if B == 0 or S == 0:
         raise RuntimeError("flash_attention_decode needs at least one sequence and one cached token")
 
-    with torch.cuda.device(query.device):
+    with _on_device(query.device):
         # num_splits == 0 lets the library plan for the current device (split count and kernel form)
         ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, num_splits)
         stream_ptr = _stream_ptr(query.device)
@@ -159,7 +178,7 @@ def flash_attention_prefill(query, keys, values):
     out = torch.empty((B, T, QH, HD), dtype=query.dtype, device=query.device).transpose(1, 2)
     if out.numel() == 0:
         return out
-    with torch.cuda.device(query.device):
+    with _on_device(query.device):
         rc = lib.l3_attn_prefill(
             query.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr(), B, QH, KVH, T, S, HD,
             _l3lib.i64_array((query.stride(0), query.stride(1), query.stride(2))),
@@ -180,7 +199,7 @@ def flash_attention_split(query, keys, values, num_splits: int = 0):
     concatenated along dim 2 and finished by flash_attention_combine."""
     lib = _l3lib.load()
     B, QH, KVH, S, HD = _check_qkv(query, keys, values)
-    with torch.cuda.device(query.device):
+    with _on_device(query.device):
         n_req = num_splits if num_splits > 0 else lib.l3_attn_choose_splits(B, KVH, S, HD, 0)
         if n_req < 0:
             _fail(n_req)
@@ -213,7 +232,7 @@ def flash_attention_combine(part_o, part_ml, dtype=torch.bfloat16):
     po = part_o if part_o.is_contiguous() else part_o.contiguous()
     pm = part_ml if part_ml.is_contiguous() else part_ml.contiguous()
     out = torch.empty((B, 1, QH, HD), dtype=dtype, device=part_o.device).transpose(1, 2)
-    with torch.cuda.device(part_o.device):
+    with _on_device(part_o.device):
         rc = lib.l3_attn_combine(po.data_ptr(), pm.data_ptr(), out.data_ptr(), B, QH, HD, n,
                                  _l3lib.i64_array((out.stride(0), out.stride(1))), _stream_ptr(part_o.device))
     if rc != 0:
@@ -234,7 +253,7 @@ def flash_attention_decode_devlen(query, keys, values, kv_len, num_splits: int =
         raise RuntimeError("kv_len must be a one-element int32 GPU tensor")
     if out is None:
         out = torch.empty_like(query)
-    with torch.cuda.device(query.device):
+    with _on_device(query.device):
         ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, L, HD, num_splits)
         stream_ptr = _stream_ptr(query.device)
         ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None
@@ -279,7 +298,7 @@ def rot_embed_append(qkv, freq_table, cache_k, cache_v, pos, n_head: int, out=No
         raise RuntimeError("pos must be a one-element int32 GPU tensor")
     if out is None:
         out = torch.empty((B, 1, n_head, HD), dtype=qkv.dtype, device=qkv.device)
-    with torch.cuda.device(qkv.device):
+    with _on_device(qkv.device):
         rc = lib.l3_rot_embed_append(qkv.data_ptr(), freq_table.data_ptr(), out.data_ptr(), cache_k.data_ptr(),
                                      cache_v.data_ptr(), pos.data_ptr(), B, n_head, KVH, HD, qkv.stride(0),
                                      _l3lib.i64_array((cache_k.stride(0), cache_k.stride(1))), L,
@@ -317,7 +336,7 @@ def linear_qkv_rope_append(x, w_qkv, freq_table, cache_k, cache_v, pos, n_head: 
             raise RuntimeError(f"linear_qkv_rope_append: norm_weight {tuple(norm_weight.shape)} / {rows} rows "
                                f"do not fit the fused input norm (K={K})")
     out = torch.empty((rows, 1, n_head, HD), dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.l3_linear_qkv_rope_append(x2.data_ptr(), None if norm_weight is None else norm_weight.data_ptr(),
                                            float(eps), w_qkv.data_ptr(), freq_table.data_ptr(), out.data_ptr(),
                                            cache_k.data_ptr(), cache_v.data_ptr(), pos.data_ptr(), rows, n_head, KVH,
@@ -341,11 +360,11 @@ def rms_norm(input, weight, eps):
         raise RuntimeError(f"weight has {weight.numel()} elements, expected {C}")
     x = input if input.is_contiguous() else input.contiguous()
     w = weight if weight.is_contiguous() else weight.contiguous()
-    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    out = torch.empty_like(x)
     rows = x.size(0) * x.size(1)
     if rows == 0:
         return out
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.l3_rms_norm(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, C, float(eps),
                              _stream_ptr(x.device))
     if rc != 0:
@@ -375,7 +394,7 @@ def add_rms_norm(input, residual, weight, eps):
     rows = x.size(0) * x.size(1)
     if rows == 0:
         return s, y
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.l3_add_rms_norm(x.data_ptr(), r.data_ptr(), w.data_ptr(), s.data_ptr(), y.data_ptr(), rows, C,
                                  float(eps), _stream_ptr(x.device))
     if rc != 0:
@@ -402,7 +421,7 @@ def silu_mul(a, b):
                 and a2.stride(0) % 8 == 0 and b2.stride(0) % 8 == 0 and a2.data_ptr() == a.data_ptr() \
                 and b2.data_ptr() == b.data_ptr():
             y = torch.empty(a.shape, dtype=a.dtype, device=a.device)
-            with torch.cuda.device(a.device):
+            with _on_device(a.device):
                 rc = lib.l3_silu_mul_rows(a2.data_ptr(), b2.data_ptr(), y.data_ptr(), rows, C, max(a2.stride(0), C),
                                           max(b2.stride(0), C), _stream_ptr(a.device))
             if rc != 0:
@@ -413,7 +432,7 @@ def silu_mul(a, b):
     y = torch.empty(ac.shape, dtype=ac.dtype, device=ac.device)
     if y.numel() == 0:
         return y
-    with torch.cuda.device(ac.device):
+    with _on_device(ac.device):
         rc = lib.l3_silu_mul(ac.data_ptr(), bc.data_ptr(), y.data_ptr(), y.numel(), _stream_ptr(ac.device))
     if rc != 0:
         _fail(rc, f"n={y.numel()}")
@@ -459,7 +478,7 @@ def linear_decode(x, weight):
         return linear_splitk_finish(linear_splitk(x, weight)).view(*x.shape[:-1], weight.shape[0])
     x2, rows, N, K = _linear_args(x, (weight,))
     y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.l3_linear_decode(x2.data_ptr(), weight.data_ptr(), y.data_ptr(), rows, N, K, x2.stride(0),
                                   weight.stride(0), N, _stream_ptr(x.device))
     if rc != 0:
@@ -473,7 +492,7 @@ def linear_swiglu_decode(x, w_gate, w_up):
     lib = _l3lib.load()
     x2, rows, N, K = _linear_args(x, (w_gate, w_up))
     y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.l3_linear_swiglu_decode(x2.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(), y.data_ptr(), rows, N, K,
                                          x2.stride(0), w_gate.stride(0), N, _stream_ptr(x.device))
     if rc != 0:
@@ -512,7 +531,7 @@ def linear_decode_fused(x, weight, norm_weight=None, eps: float = 1e-5, w_up=Non
         if not r2.is_contiguous():
             r2 = r2.contiguous()
     y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.l3_linear_decode_fused(x2.data_ptr(), None if norm_weight is None else norm_weight.data_ptr(),
                                         float(eps), weight.data_ptr(), None if w_up is None else w_up.data_ptr(),
                                         None if r2 is None else r2.data_ptr(), y.data_ptr(), rows, N, K,
@@ -530,7 +549,7 @@ def linear_splitk(x, weight, ksplit: int = 0):
     longer fit one matrix-instruction column block (model.py:95,121,134).  An extension."""
     lib = _l3lib.load()
     x2, rows, N, K = _linear_args(x, (weight,), _l3lib.L3_LINEAR_SPLITK_MAX_ROWS)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         if ksplit <= 0:
             ksplit = lib.l3_linear_splitk_plan(N, K, _cus(x.device))
             if ksplit < 0:
@@ -560,7 +579,7 @@ def linear_splitk_finish(part, residual=None):
         if not r2.is_contiguous():
             r2 = r2.contiguous()
     y = torch.empty((rows, N), dtype=torch.bfloat16, device=part.device)
-    with torch.cuda.device(part.device):
+    with _on_device(part.device):
         rc = lib.l3_linear_splitk_finish(part.data_ptr(), ksplit, None if r2 is None else r2.data_ptr(), y.data_ptr(),
                                          rows, N, N, _stream_ptr(part.device))
     if rc != 0:
@@ -585,7 +604,7 @@ def add_rms_norm_partials(input, part, weight, eps):
     x = input if input.is_contiguous() else input.contiguous()
     s = torch.empty(x.shape, dtype=x.dtype, device=x.device)
     y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.l3_add_rms_norm_partials(x.data_ptr(), part.data_ptr(), part.shape[0], weight.data_ptr(),
                                           s.data_ptr(), y.data_ptr(), rows, C, float(eps), _stream_ptr(x.device))
     if rc != 0:
@@ -615,7 +634,7 @@ def rot_embed_append_partials(part, freq_table, cache_k, cache_v, pos, n_head: i
     if not pos.is_cuda or pos.dtype != torch.int32 or pos.numel() != 1:
         raise RuntimeError("pos must be a one-element int32 GPU tensor")
     out = torch.empty((B, 1, n_head, HD), dtype=cache_k.dtype, device=part.device)
-    with torch.cuda.device(part.device):
+    with _on_device(part.device):
         rc = lib.l3_rot_embed_append_partials(part.data_ptr(), ksplit, freq_table.data_ptr(), out.data_ptr(),
                                               cache_k.data_ptr(), cache_v.data_ptr(), pos.data_ptr(), B, n_head, KVH,
                                               HD, _l3lib.i64_array((cache_k.stride(0), cache_k.stride(1))), L,
@@ -637,7 +656,7 @@ def argmax(logits):
     out = torch.empty(rows, dtype=torch.int64, device=logits.device)
     if rows == 0:
         return out
-    with torch.cuda.device(logits.device):
+    with _on_device(logits.device):
         ws_bytes = lib.l3_argmax_workspace_bytes(rows, V)
         stream_ptr = _stream_ptr(logits.device)
         ws = _workspace(logits.device, stream_ptr, ws_bytes)
@@ -669,7 +688,7 @@ def greedy_step(logits, tokens, text_mask, tok, pos, kv_len, eos, stop_tokens):
           and stop_tokens.dtype == torch.int64 and stop_tokens.is_contiguous())
     if not ok or any(t.device != logits.device for t in (tokens, text_mask, tok, pos, kv_len, eos, stop_tokens)):
         raise RuntimeError("greedy_step: state tensors have the wrong dtype, shape, layout or device")
-    with torch.cuda.device(logits.device):
+    with _on_device(logits.device):
         ws_bytes = lib.l3_argmax_workspace_bytes(rows, V)
         stream_ptr = _stream_ptr(logits.device)
         ws = _workspace(logits.device, stream_ptr, ws_bytes)
@@ -696,10 +715,10 @@ def rot_embed(input, freq):
     if input.stride(3) != 1:
         raise RuntimeError("the head dimension of input must be contiguous")
     f = freq if freq.is_contiguous() else freq.contiguous()
-    out = torch.empty((B, T, NH, HD), dtype=input.dtype, device=input.device)
+    out = input.new_empty((B, T, NH, HD))
     if out.numel() == 0:
         return out
-    with torch.cuda.device(input.device):
+    with _on_device(input.device):
         rc = lib.l3_rot_embed(input.data_ptr(), f.data_ptr(), out.data_ptr(), B, T, NH, HD,
                               _l3lib.i64_array((input.stride(0), input.stride(1), input.stride(2))),
                               _stream_ptr(input.device))
