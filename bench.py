@@ -403,8 +403,10 @@ def run_prefill(args, torch, lib, l3, dev):
             prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, form)
             cke.flash_attention_prefill(q, k, v)
             gph = capture_graph(torch, lambda: [cke.flash_attention_prefill(q, k, v) for _ in range(reps)])
-            for _ in range(3):      # untimed: the first replays after an idle spell run at lower clocks
+            t_warm = time.perf_counter()    # untimed: after an idle spell the first milliseconds run at lower clocks
+            while time.perf_counter() - t_warm < 0.03:
                 gph.replay()
+                torch.cuda.synchronize()
             forms[fname] = event_time_ms(torch, gph.replay, 5) / reps
             del gph
             lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, prev)

@@ -55,8 +55,10 @@ struct PrefillTile {
     static_assert(CHUNKS % NT == 0, "tile must divide evenly over the workgroup");
 };
 
+// Two wavefronts per SIMD whatever the workgroup size: a 4-wave workgroup could otherwise be given
+// 512 registers per wavefront, and then only one workgroup would fit a compute unit.
 template <int HD, int CB, int NW>
-__global__ void __launch_bounds__(NW * kWaveSize)
+__global__ void __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attn_prefill_tiled_kernel(const PrefillParams p) {
     using T = PrefillTile<HD, CB, NW>;
     constexpr int NT = T::NT, TK = T::TK, LPR = T::LPR, U = T::U, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
@@ -287,7 +289,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
 // maximum, has been added); the two sets of score / probability registers swap roles every
 // iteration, hence the loop unrolled by two.
 template <int HD, int CB, int NW>
-__global__ void __launch_bounds__(NW * kWaveSize)
+__global__ void __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attn_prefill_pipe_kernel(const PrefillParams p) {
     using T = PrefillTile<HD, CB, NW>;
     constexpr int TK = T::TK, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
@@ -644,11 +646,11 @@ int launch_tiled(const PrefillParams& p, bool pipelined, hipStream_t stream) {
 
 }  // namespace
 
-int prefill_tiled_positions_per_wg(int R) { return kPrefillTiledWaves * kPrefillTiledColBlocks * (16 / R); }
+int prefill_tiled_positions_per_wg(int HD, int R) { return prefill_tiled_waves(HD) * kPrefillTiledColBlocks * (16 / R); }
 
 int launch_attn_prefill_tiled(const PrefillParams& p, int HD, bool pipelined, hipStream_t stream) {
-    if (HD == 64) return launch_tiled<64, kPrefillTiledColBlocks, kPrefillTiledWaves>(p, pipelined, stream);
-    return launch_tiled<128, kPrefillTiledColBlocks, kPrefillTiledWaves>(p, pipelined, stream);
+    if (HD == 64) return launch_tiled<64, kPrefillTiledColBlocks, prefill_tiled_waves(64)>(p, pipelined, stream);
+    return launch_tiled<128, kPrefillTiledColBlocks, prefill_tiled_waves(128)>(p, pipelined, stream);
 }
 
 }  // namespace l3

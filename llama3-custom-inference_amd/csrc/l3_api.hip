@@ -305,7 +305,7 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     // better spread over many independent wavefronts.
     int form = g_prefill_form.load(std::memory_order_relaxed);
     if (form == L3_ATTN_PREFILL_AUTO) {
-        const int wg_pos = prefill_tiled_positions_per_wg(QH / KVH);
+        const int wg_pos = prefill_tiled_positions_per_wg(HD, QH / KVH);
         const int64_t tiled_wgs = int64_t(B) * KVH * ((T + wg_pos - 1) / wg_pos);
         form = (T >= 4 * wg_pos && tiled_wgs >= current_device_cus() / 2) ? L3_ATTN_PREFILL_PIPELINED
                                                                           : L3_ATTN_PREFILL_WAVE;
