@@ -104,6 +104,27 @@ def test_rot_embed_config_shapes(gpu, HD, shape):
         np.testing.assert_array_equal(t2bits(out), t2bits(out_c))
 
 
+@pytest.mark.parametrize("B,T,NH,HD", [(3, 1501, 32, 128),    # 2 tokens per workgroup, odd T: a half-filled last block
+                                        (2, 3100, 20, 128),    # 80 threads per token: 3 tokens per workgroup, idle lanes
+                                        (5, 7000, 8, 64),      # 16 tokens per workgroup
+                                        (2, 5200, 6, 128),     # head pairs, 48 threads per token
+                                        (1, 9001, 7, 64)])     # single heads, 56 threads per token
+def test_rot_embed_many_tokens(gpu, B, T, NH, HD):
+    """Thousands of tokens per batch row with head counts that give 2, 3, 4, 5 and 16 tokens per
+    workgroup, idle lanes, and token counts that do not fill the last workgroup."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"rot_embed B={B} T={T} NH={NH} HD={HD}", flush=True)
+    tab = precompute_freqs_cis_ref(HD, T, theta=500000.0, use_scaled=True, scale_factor=32.0)
+    wide = randn_bf16((B, T, NH * HD + 2 * HD), 77)      # a view into wider rows, as q is into qkv
+    x = wide[..., :NH * HD].view(B, T, NH, HD)
+    xg = wide.to(gpu)[..., :NH * HD].view(B, T, NH, HD)
+    out = cke.rot_embed(xg, torch.from_numpy(np.ascontiguousarray(tab)).to(gpu))
+    torch.cuda.synchronize()
+    assert out.is_contiguous()
+    assert_within_ulps(out, rot_embed_ref(t2f32(x), tab), 1, what=f"rope {tuple(x.shape)}")
+
+
 def test_rot_embed_identity_at_position_zero_and_norms(gpu):
     from custom_kernels import custom_kernels_extension as cke
 
