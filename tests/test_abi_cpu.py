@@ -4,6 +4,8 @@ declares, rejects bad arguments before any launch, and plans splits sanely."""
 import ctypes
 import os
 import re
+import shutil
+import subprocess
 
 import pytest
 
@@ -28,6 +30,38 @@ def test_every_declared_symbol_is_exported_and_bound():
     for n in names:
         assert getattr(lib, n) is not None
     assert lib.l3_version() >= 100
+
+
+C_CALLER = r"""
+#include <stdio.h>
+#include "l3_kernels.h"
+
+int main(void) {
+    /* host-logic entry points only: nothing here touches a GPU */
+    if (l3_version() < 100) return 1;
+    if (l3_attn_choose_splits(1, 8, 32768, 128, 256) < 2) return 2;
+    if (l3_attn_choose_splits(1, 8, 32768, 96, 256) != L3_ERR_HEAD_SIZE) return 3;
+    if (l3_attn_decode_workspace_bytes(1, 32, 8, 32768, 128, 4) != (size_t)(4 * 32 * 128 * 4 + 4 * 32 * 8)) return 4;
+    if (l3_rms_norm(0, 0, 0, 1, 2048, 1e-5f, 0) != L3_ERR_NULL_POINTER) return 5;
+    printf("%s\n", l3_strerror(L3_ERR_HEAD_RATIO));
+    return 0;
+}
+"""
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="needs a C compiler")
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    """What a maintainer binding the library from C (or cgo, JNI ...) relies on: the header compiles as
+    C99 with nothing but the standard headers, and a C program linked against the library reaches the
+    entry points by their undecorated names."""
+    lib_path = _l3lib.library_path()
+    src = tmp_path / "caller.c"
+    src.write_text(C_CALLER)
+    exe = tmp_path / "caller"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.dirname(HEADER), str(src),
+                    "-o", str(exe), lib_path, "-Wl,-rpath," + os.path.dirname(lib_path)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert "Unsupported QKV head ratio" in out
 
 
 def test_error_codes_match_header():
