@@ -301,14 +301,19 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     p.v_sb = v_strides[0]; p.v_sh = v_strides[1]; p.v_st = v_strides[2];
     p.o_sb = out_strides[0]; p.o_sh = out_strides[1]; p.o_st = out_strides[2];
     p.scale_log2e = scale * 1.4426950408889634f;
-    // Long prompts share K/V tiles across a workgroup; short ones (few columns per kv head) are
-    // better spread over many independent wavefronts.
+    // Long prompts share K/V tiles across a workgroup.  Short ones are better spread over many
+    // independent wavefronts (16 columns each) -- as long as the device can hold them all at once:
+    // measured (head ratios 1, 3, 4 and 8), the tiled form wins from 192 tokens (head size 64) or
+    // 384 tokens (128) on, and earlier when the wavefront-private form would need more than eight
+    // wavefronts per compute unit and the prompt fills at least one workgroup of the tiled form.
     int form = g_prefill_form.load(std::memory_order_relaxed);
     if (form == L3_ATTN_PREFILL_AUTO) {
-        const int wg_pos = prefill_tiled_positions_per_wg(HD, QH / KVH);
-        const int64_t tiled_wgs = int64_t(B) * KVH * ((T + wg_pos - 1) / wg_pos);
-        form = (T >= 4 * wg_pos && tiled_wgs >= current_device_cus() / 2) ? L3_ATTN_PREFILL_PIPELINED
-                                                                          : L3_ATTN_PREFILL_WAVE;
+        const int R = QH / KVH;
+        const int wg_pos = prefill_tiled_positions_per_wg(HD, R);
+        const int64_t private_waves = int64_t(B) * KVH * ((int64_t(T) * R + 15) / 16);
+        const int long_prompt = HD == 64 ? 192 : 384;
+        const bool tiled = T >= long_prompt || (T >= wg_pos && private_waves > 8 * int64_t(current_device_cus()));
+        form = tiled ? L3_ATTN_PREFILL_PIPELINED : L3_ATTN_PREFILL_WAVE;
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int rc = (form == L3_ATTN_PREFILL_WAVE) ? launch_attn_prefill(p, HD, st)
