@@ -138,6 +138,16 @@ def test_split_planning():
         assert lib.l3_attn_choose_splits(256, 8, 256, HD, 256) == 1
         # the device size matters
         assert lib.l3_attn_choose_splits(1, 8, 32768, HD, 64) < lib.l3_attn_choose_splits(1, 8, 32768, HD, 256)
+    # many sequences (8 kv heads: one workgroup per sequence and split group, 256 units):
+    plan = lambda B, S, HD: lib.l3_attn_choose_splits(B, 8, S, HD, 256)  # noqa: E731
+    assert plan(3, 32768, 128) == 79            # at most 85 (3 * 85 = 255 workgroups for 256 units), whole tiles: 79 x 416 tokens
+    assert plan(16, 4096, 64) == 16             # few sequences: one workgroup per unit
+    assert plan(48, 4096, 128) == 4             # from 32 sequences on, three quarters of the units
+    assert plan(64, 4096, 128) == 3
+    assert plan(96, 2048, 64) == 2
+    assert plan(96, 512, 64) == 1               # short streams at a quarter of the units or more: no combine
+    assert plan(128, 128, 64) == 1 and plan(192, 1024, 128) == 1
+    assert plan(100, 4096, 128) == 2            # a long stream is worth the second group
     assert lib.l3_attn_choose_splits(1, 8, 256, 96, 256) == _l3lib.L3_ERR_HEAD_SIZE
     assert lib.l3_attn_choose_splits(0, 8, 256, 64, 256) == _l3lib.L3_ERR_SHAPE
     assert cke.attention_num_splits(16, 8, 4096, 64) == lib.l3_attn_choose_splits(16, 8, 4096, 64, 256)
