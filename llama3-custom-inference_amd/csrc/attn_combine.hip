@@ -117,9 +117,93 @@ attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__
     }
 }
 
+// Many (batch, query head) pairs with a few splits each (large batches): one WAVEFRONT per pair, four
+// pairs per workgroup, no LDS and no barrier -- the eight-wavefront form above would launch thousands
+// of workgroups that each merge two or three rows.  Same arithmetic, in the same order, as one
+// wavefront of that kernel.
+template <int HD>
+__global__ void __launch_bounds__(4 * kWaveSize)
+attn_combine_rows_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
+                         uint16_t* __restrict__ out, int QH, int n_rows, int64_t total_pairs, int64_t o_sb,
+                         int64_t o_sh, const int* __restrict__ seqlen_dev, int tokens_per_split) {
+    constexpr int TPR = HD / 4;             // lanes covering a partial row with float4 loads
+    constexpr int RPL = kWaveSize / TPR;    // rows per wavefront-wide load
+    constexpr int NLD = kCombineRows / RPL; // row loads per pass
+
+    const int lane = threadIdx.x & (kWaveSize - 1);
+    const int wave = threadIdx.x / kWaveSize;
+    const int64_t bq = int64_t(blockIdx.x) * 4 + wave;
+    if (bq >= total_pairs) return;   // whole wavefront; the kernel has no barrier
+    int n = n_rows;
+    if (seqlen_dev) n = min(n_rows, max(1, (*seqlen_dev + tokens_per_split - 1) / tokens_per_split));
+    const float2* ml = part_ml + bq * n_rows;
+    const float4* po = reinterpret_cast<const float4*>(part_o + bq * n_rows * HD);
+    const int dq = lane % TPR;
+    const int sub = lane / TPR;
+
+    float m_w = kMaskedScore, l_w = 0.f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int r0 = 0; r0 < n; r0 += kCombineRows) {
+        float2 st = make_float2(kMaskedScore, 0.f);
+        if (lane < kCombineRows && r0 + lane < n) st = ml[r0 + lane];
+        float4 x[NLD];
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (r0 + u * RPL < n) {   // wavefront-uniform: loads past the last split are not issued
+                const int r = min(r0 + u * RPL + sub, n - 1);   // rows past the end get weight 0 below
+                x[u] = po[int64_t(r) * TPR + dq];
+            }
+        }
+        const float m_new = fmaxf(m_w, wave_max(st.x));
+        const float alpha = fast_exp2(m_w - m_new);
+        const float wgt = fast_exp2(st.x - m_new);
+        l_w = fmaf(l_w, alpha, wave_sum(st.y * wgt));
+        acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
+        m_w = m_new;
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            const float w = __shfl(wgt, u * RPL + sub, kWaveSize);
+            acc.x = fmaf(w, x[u].x, acc.x);
+            acc.y = fmaf(w, x[u].y, acc.y);
+            acc.z = fmaf(w, x[u].z, acc.z);
+            acc.w = fmaf(w, x[u].w, acc.w);
+        }
+    }
+#pragma unroll
+    for (int off = TPR; off < kWaveSize; off <<= 1) {
+        acc.x += __shfl_xor(acc.x, off, kWaveSize);
+        acc.y += __shfl_xor(acc.y, off, kWaveSize);
+        acc.z += __shfl_xor(acc.z, off, kWaveSize);
+        acc.w += __shfl_xor(acc.w, off, kWaveSize);
+    }
+    if (lane < TPR) {
+        const float inv = 1.0f / l_w;
+        uint2 packed;
+        packed.x = pack_bf16x2(acc.x * inv, acc.y * inv);
+        packed.y = pack_bf16x2(acc.z * inv, acc.w * inv);
+        const int64_t b = bq / QH;
+        const int qh = int(bq % QH);
+        *reinterpret_cast<uint2*>(out + b * o_sb + int64_t(qh) * o_sh + lane * 4) = packed;
+    }
+}
+
 }  // namespace
 
 int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream) {
+    const int64_t pairs = int64_t(p.B) * p.QH;
+    if (pairs >= 1024 && p.num_splits <= kCombineRows) {   // many pairs, few splits each: a wavefront per pair
+        const dim3 rgrid{unsigned((pairs + 3) / 4)};
+        const dim3 rblock{4 * kWaveSize};
+        if (HD == 64) {
+            hipLaunchKernelGGL((attn_combine_rows_kernel<64>), rgrid, rblock, 0, stream, p.part_o, p.part_ml, p.out,
+                               p.QH, p.num_splits, pairs, p.o_sb, p.o_sh, p.seqlen_dev, p.tokens_per_split);
+        } else {
+            hipLaunchKernelGGL((attn_combine_rows_kernel<128>), rgrid, rblock, 0, stream, p.part_o, p.part_ml, p.out,
+                               p.QH, p.num_splits, pairs, p.o_sb, p.o_sh, p.seqlen_dev, p.tokens_per_split);
+        }
+        return int(hipGetLastError());
+    }
     const bool few = int64_t(p.B) * p.QH <= 64 && p.num_splits > kCombineRows;   // few heads, many rows each
     const dim3 grid(unsigned(p.B) * unsigned(p.QH), few ? 4u : 1u);
     const dim3 block(kCombineWaves * kWaveSize);

@@ -45,6 +45,28 @@ def test_head_ratios(gpu, HD, QH, KVH, splits):
     _run(gpu, 2, QH, KVH, 333, HD, seed=QH + KVH, splits=splits)
 
 
+@pytest.mark.parametrize("B,QH,KVH,S,HD,splits", [(40, 32, 8, 300, 64, 2), (40, 32, 8, 300, 128, 3),
+                                                   (130, 8, 8, 97, 64, 2), (33, 32, 4, 1000, 128, 31),
+                                                   (515, 2, 2, 70, 64, 2), (36, 32, 8, 2100, 128, 32),
+                                                   (100, 32, 8, 1024, 128, 0)])
+def test_many_sequences_with_few_splits(gpu, attn_kernel, B, QH, KVH, S, HD, splits):
+    """A thousand or more (batch, query head) pairs with 2 ... 32 splits each: the combine runs with a
+    wavefront per pair (515 x 2 pairs do not fill its last workgroup); the last case takes the plan's
+    own choice for 100 long sequences (two splits with the MFMA kernel)."""
+    if splits == 0:
+        from custom_kernels import custom_kernels_extension as cke
+        assert cke.attention_num_splits(B, KVH, S, HD, 256) == (2 if attn_kernel == "mfma" else 1)
+        q, k, v = make_qkv(B, QH, KVH, S, HD, seed=9)
+        qg, kg, vg = make_qkv(B, QH, KVH, S, HD, seed=9, device=gpu)
+        out = cke.flash_attention_decode(qg, kg, vg)
+        torch.cuda.synchronize()
+        rows = [0, 1, 50, B - 1]                      # the oracle on a few sequences only
+        ref = attention_decode_ref(t2f32(q[rows]), t2f32(k[rows]), t2f32(v[rows]))
+        assert_attn_close(out[rows], ref, what="100 long sequences")
+        return
+    _run(gpu, B, QH, KVH, S, HD, seed=B + splits, splits=splits)
+
+
 @pytest.mark.parametrize("HD", [64, 128])
 @pytest.mark.parametrize("splits", [1, 2, 5, 16, 512])
 def test_result_independent_of_split_count(gpu, HD, splits):
@@ -234,7 +256,7 @@ def test_pieces_of_a_sequence_combine_to_the_whole(gpu, HD):
 
 
 # ---- KV length read from device memory (one recorded launch serves a growing cache)
-@pytest.mark.parametrize("HD,B,L", [(64, 1, 256), (64, 3, 300), (128, 2, 1024), (64, 64, 256)])
+@pytest.mark.parametrize("HD,B,L", [(64, 1, 256), (64, 3, 300), (128, 2, 1024), (64, 64, 256), (128, 40, 200)])
 def test_device_side_kv_length(gpu, HD, B, L):
     from custom_kernels import custom_kernels_extension as cke
 
