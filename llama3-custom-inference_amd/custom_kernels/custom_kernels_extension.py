@@ -459,12 +459,16 @@ def _linear_args(x, weights, max_rows=None):
 
 def _use_splitk(x, weight) -> bool:
     """17..64 activation rows against a matrix too small for one workgroup per 128 rows to fill the
-    device: the split-K kernel plus its finishing pass is the faster route."""
+    device: the split-K kernel plus its finishing pass is the faster route (measured at 17, 32 and 64
+    rows, K 2048..8192: up to 16384 matrix rows on 256 compute units; from 32768 on the single launch wins)."""
     K = x.shape[-1]
     if K <= 0 or weight.dim() != 2 or not x.is_cuda:
         return False
     rows = x.numel() // K
-    return rows > _l3lib.L3_LINEAR_FUSED_MAX_ROWS and -(-weight.shape[0] // 128) < _cus(x.device) // 2
+    N = weight.shape[0]
+    if N % 8:          # the finishing pass writes eight columns per lane; the single launch needs only N % 4 == 0
+        return False
+    return rows > _l3lib.L3_LINEAR_FUSED_MAX_ROWS and -(-N // 128) < _cus(x.device)
 
 
 def linear_decode(x, weight):
