@@ -15,9 +15,10 @@ namespace {
 
 constexpr int kRmsThreads = 256;
 
-// One row per group of LANES threads (64: a wavefront per row, four rows per workgroup;
-// 256: the whole workgroup on one row).  A thread keeps up to MAXV 16-byte vectors of its
-// row in registers; requires C % 8 == 0 and C / 8 <= LANES * MAXV.
+// One row per group of LANES threads (the launcher uses 256: the whole workgroup on one row,
+// for fewer than 1024 rows and for rows too wide for the streaming kernel further down).  A
+// thread keeps up to MAXV 16-byte vectors of its row in registers; requires C % 8 == 0 and
+// C / 8 <= LANES * MAXV.
 //
 // ADD = true fuses the residual addition that precedes every RMSNorm but the first in a
 // transformer block (model.py:147-148: x = x + attn(...); ...ln_2(x)): s = bf16(x + res) is
@@ -279,25 +280,15 @@ int launch_rms_norm_impl(const uint16_t* x, const uint16_t* res, const uint16_t*
                          int64_t rows, int C, float eps, bool vec_ok, hipStream_t stream) {
     const int nvec = C / 8;
     const dim3 block(kRmsThreads);
-    if (vec_ok && rows >= 2048 && nvec <= 64 * (ADD ? 4 : 8)) {
-        // thousands of rows: every wavefront takes several, reads overlapping writes
+    if (vec_ok && rows >= 1024 && nvec <= 64 * 8) {
+        // a thousand rows or more: every wavefront takes several, reads overlapping writes
         const int64_t waves = std::min<int64_t>(rows / 2, int64_t(current_device_cus()) * 8);
         const dim3 grid(unsigned((waves + 3) / 4));
         if (nvec <= 64 * 4) {
             hipLaunchKernelGGL((rms_norm_stream_kernel<4, ADD>), grid, block, 0, stream, x, res, w, sum_out, y, rows, C,
                                eps);
-        } else if constexpr (!ADD) {
-            hipLaunchKernelGGL((rms_norm_stream_kernel<8, false>), grid, block, 0, stream, x, res, w, sum_out, y, rows,
-                               C, eps);
-        }
-    } else if (vec_ok && rows >= 1024 && nvec <= 64 * 8) {
-        // plenty of rows: a wavefront per row, no workgroup barrier
-        const dim3 grid(unsigned((rows + 3) / 4));
-        if (nvec <= 64 * 4) {
-            hipLaunchKernelGGL((rms_norm_rows_kernel<64, 4, ADD>), grid, block, 0, stream, x, res, w, sum_out, y, rows,
-                               C, eps);
         } else {
-            hipLaunchKernelGGL((rms_norm_rows_kernel<64, 8, ADD>), grid, block, 0, stream, x, res, w, sum_out, y, rows,
+            hipLaunchKernelGGL((rms_norm_stream_kernel<8, ADD>), grid, block, 0, stream, x, res, w, sum_out, y, rows,
                                C, eps);
         }
     } else if (vec_ok && nvec <= 256 * 4) {
