@@ -94,21 +94,22 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
         }
         // Streaming form; a workgroup covers heads_per_wg kv heads x (8 / heads_per_wg) splits, so the
         // split count comes in groups.  Few (batch, head group) pairs: one 8-wave workgroup per compute
-        // unit, never more (a workgroup or two beyond one per unit run as a second round).  From an
-        // eighth of the units on, three quarters of the units already saturate HBM and every further
-        // split only adds partials for the combine; and a single group (no combine at all) is kept
-        // while a workgroup's stream stays short.
+        // unit, never more (a workgroup or two beyond one per unit run as a second round).  From a
+        // thirty-second of the units on, three quarters of the units already saturate HBM and every
+        // further split only adds partials for the combine; and where a group is a single split (eight
+        // kv heads per workgroup) it is kept alone, with no combine at all, while a workgroup's stream
+        // stays short.
         const int hpw = attn_mfma_heads_per_wg(KVH);
         const int spg = kMfmaWaves / hpw;
         const int64_t wgs_per_split_group = int64_t(B) * (KVH / hpw);
         int64_t groups;
-        if (wgs_per_split_group * 8 >= num_cus) {
+        if (wgs_per_split_group * 32 >= num_cus) {
             groups = (int64_t(num_cus) * 3 / 4) / wgs_per_split_group;
             if (groups < 1) groups = 1;
             // K + V bytes a workgroup streams when there is a single group
             const int64_t stream_bytes = int64_t(kMfmaWaves) * ((S + spg - 1) / spg) * HD * 4;
             const bool short_stream = stream_bytes <= (int64_t(3) << 20);
-            if (short_stream && wgs_per_split_group * 4 >= num_cus) {
+            if (short_stream && spg == 1 && wgs_per_split_group * 4 >= num_cus) {
                 groups = 1;   // a quarter of the units busy, but no partials and no second launch
             } else if (groups == 1 && !short_stream && int64_t(num_cus) / wgs_per_split_group >= 2) {
                 groups = 2;

@@ -141,8 +141,9 @@ def test_split_planning():
     # many sequences (8 kv heads: one workgroup per sequence and split group, 256 units):
     plan = lambda B, S, HD: lib.l3_attn_choose_splits(B, 8, S, HD, 256)  # noqa: E731
     assert plan(3, 32768, 128) == 79            # at most 85 (3 * 85 = 255 workgroups for 256 units), whole tiles: 79 x 416 tokens
-    assert plan(16, 4096, 64) == 16             # few sequences: one workgroup per unit
-    assert plan(48, 4096, 128) == 4             # from 32 sequences on, three quarters of the units
+    assert plan(4, 4096, 64) == 64              # few sequences: one workgroup per unit
+    assert plan(16, 4096, 64) == 11             # from 8 sequences on, three quarters of the units: 12 groups, whole tiles
+    assert plan(48, 4096, 128) == 4
     assert plan(64, 4096, 128) == 3
     assert plan(96, 2048, 64) == 2
     assert plan(96, 512, 64) == 1               # short streams at a quarter of the units or more: no combine
