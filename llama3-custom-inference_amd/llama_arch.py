@@ -139,10 +139,14 @@ class LlamaDecoder:
             y = self.ops.flash_attention_decode(q, k, v)
         return y.transpose(1, 2).contiguous().view(B, T, c.n_embd)
 
+    FUSED_MAX_ROWS = 6   # rows up to which the fused single-launch linears carry the decode step
+
     def _splitk(self, rows: int) -> bool:
-        """17..64 activation rows: the split-K linears (activations shared through LDS, splits added
-        up by the operator that follows) stand for F.linear on the three smaller matrices."""
-        return self.decode_linear_rows > 0 and 16 < rows <= 64 and hasattr(self.ops, "linear_splitk")
+        """7..64 activation rows: the split-K linears (activations shared through LDS, splits added
+        up by the operator that follows) stand for F.linear on the three smaller matrices.  Measured
+        end to end, this route overtakes the fused single-launch linears at 7 rows (level at 6, +5 % at
+        8, +12..18 % from 11 on): every workgroup of those re-reads the activations of its k range."""
+        return self.decode_linear_rows > 0 and self.FUSED_MAX_ROWS < rows <= 64 and hasattr(self.ops, "linear_splitk")
 
     def _gate_up(self, L):
         """c_fc2 and c_fc stacked into one (2 * hidden, C) matrix: one GEMM instead of two."""
@@ -151,7 +155,7 @@ class LlamaDecoder:
         return L["c_fc_cat"]
 
     def _decode_layers_splitk(self, x, append_and_attend):
-        """The layers of one decode step (T == 1) at 17..64 rows; returns the final hidden state.
+        """The layers of one decode step (T == 1) at 7..64 rows; returns the final hidden state.
         append_and_attend(L, qkv partial products) -> attention output (B, 1, C)."""
         c, ops = self.config, self.ops
         H = c.hidden_dim
@@ -169,7 +173,7 @@ class LlamaDecoder:
         """Rows up to which the decode step uses linear_decode_fused (norms and residual additions
         folded into the linears); 0 when the operator module has no such operator."""
         f = getattr(self.ops, "linear_decode_fused_max_rows", None)
-        return min(self.decode_linear_rows, f(self.config.n_embd)) if f else 0
+        return min(self.decode_linear_rows, f(self.config.n_embd), self.FUSED_MAX_ROWS) if f else 0
 
     def _prefill_attention(self, q, k, v):
         """Causal GQA attention for T > 1.  The reference hands this case to torch
