@@ -1,5 +1,5 @@
 """GPU parity on shapes drawn from a seeded generator: decode attention (plan chosen by the
-library, or a forced split count), causal prefill, RMSNorm, rotary embedding and the decode
+library, or a forced split count; few and many sequences), causal prefill, RMSNorm, rotary embedding and the decode
 linears, each against the float64 oracle.  The draws are deterministic (same cases every run);
 every case prints its parameters before it launches anything."""
 
@@ -43,6 +43,30 @@ def test_decode_attention_random_shapes(gpu, case):
     out = cke.flash_attention_decode(qg, kg, vg, splits)
     torch.cuda.synchronize()
     assert_attn_close(out, attention_decode_ref(t2f32(q), t2f32(k), t2f32(v)), what=f"decode case {i}")
+
+
+def _draw_large_batch_cases(n, seed):
+    """Dozens to hundreds of sequences with every kv-head count the kernel groups differently (1, 2, 3, 4, 8,
+    16 heads per batch row): the split plan's branches for many (batch, head group) pairs, the combine
+    with a wavefront per pair, and the cooperative form with many workgroups."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n):
+        HD = int(rng.choice((64, 128)))
+        R = int(rng.choice(RATIOS))
+        KVH = int(rng.choice((1, 2, 3, 4, 8, 16)))
+        B = int(rng.integers(30, 270))
+        S = int(rng.choice((int(rng.integers(1, 130)), int(rng.integers(130, 1100)))))
+        S = max(1, min(S, int(2e8 // (B * R * KVH * HD))))     # keeps the float64 oracle in seconds
+        extra = int(rng.choice((0, 5, 64)))
+        splits = int(rng.choice((0, 0, 0, 2, 3)))
+        cases.append((100 + i, B, R * KVH, KVH, S, HD, S + extra, splits))
+    return cases
+
+
+@pytest.mark.parametrize("case", _draw_large_batch_cases(16, 2025), ids=lambda c: f"b{c[0]}")
+def test_decode_attention_large_batches(gpu, case):
+    test_decode_attention_random_shapes(gpu, case)
 
 
 def _draw_prefill_cases(n, seed):
