@@ -387,8 +387,8 @@ def run_prefill(args, torch, lib, l3, dev):
     from custom_kernels import custom_kernels_extension as cke
 
     MFMA_PEAK_TFLOPS = 2500.0
-    shapes = [(1, 32, 8, 128, 64), (2, 32, 8, 2048, 64), (1, 32, 8, 2048, 128), (1, 32, 8, 4096, 128),
-              (1, 32, 8, 8192, 128)]
+    shapes = [(1, 32, 8, 128, 64), (2, 32, 8, 2048, 64), (1, 32, 8, 8192, 64), (1, 32, 8, 2048, 128),
+              (1, 32, 8, 4096, 128), (1, 32, 8, 8192, 128)]
     detail, head = [], None
     for (B, QH, KVH, T, HD) in shapes:
         g = torch.Generator().manual_seed(SEED)
