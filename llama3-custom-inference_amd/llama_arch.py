@@ -140,6 +140,7 @@ class LlamaDecoder:
         return y.transpose(1, 2).contiguous().view(B, T, c.n_embd)
 
     FUSED_MAX_ROWS = 6   # rows up to which the fused single-launch linears carry the decode step
+    SWIGLU_MAX_ROWS = 14  # rows up to which the split-K route takes the single-launch gate|up + SwiGLU linear (+3 % at 7..10 rows, level at 16)
 
     def _splitk(self, rows: int) -> bool:
         """7..64 activation rows: the split-K linears (activations shared through LDS, splits added
@@ -159,12 +160,16 @@ class LlamaDecoder:
         append_and_attend(L, qkv partial products) -> attention output (B, 1, C)."""
         c, ops = self.config, self.ops
         H = c.hidden_dim
+        rows = x.numel() // x.shape[-1]
         h = ops.rms_norm(x, self.layers[0]["ln_1"], c.norm_eps)
         for i, L in enumerate(self.layers):
             y = append_and_attend(L, ops.linear_splitk(h, L["c_attn"]))
             x, h = ops.add_rms_norm_partials(x, ops.linear_splitk(y, L["c_proj"]), L["ln_2"], c.norm_eps)
-            gu = F.linear(h, self._gate_up(L))
-            t = ops.silu_mul(gu[..., :H], gu[..., H:])
+            if rows <= self.SWIGLU_MAX_ROWS:
+                t = ops.linear_swiglu_decode(h, L["c_fc2"], L["c_fc"])     # one launch for the pair and the product
+            else:
+                gu = F.linear(h, self._gate_up(L))
+                t = ops.silu_mul(gu[..., :H], gu[..., H:])
             next_norm = self.layers[i + 1]["ln_1"] if i + 1 < len(self.layers) else self.ln_f
             x, h = ops.add_rms_norm_partials(x, ops.linear_splitk(t, L["mlp_proj"]), next_norm, c.norm_eps)
         return h
