@@ -139,14 +139,16 @@ class LlamaDecoder:
             y = self.ops.flash_attention_decode(q, k, v)
         return y.transpose(1, 2).contiguous().view(B, T, c.n_embd)
 
-    FUSED_MAX_ROWS = 6   # rows up to which the fused single-launch linears carry the decode step
+    FUSED_MAX_ROWS = 4   # rows up to which the fused single-launch linears carry the whole decode step
+    QKV_FUSED_MAX_ROWS = 16   # rows up to which the split-K route takes the single-launch qkv + rope + append linear (+2..6 %)
     SWIGLU_MAX_ROWS = 14  # rows up to which the split-K route takes the single-launch gate|up + SwiGLU linear (+3 % at 7..10 rows, level at 16)
 
     def _splitk(self, rows: int) -> bool:
-        """7..64 activation rows: the split-K linears (activations shared through LDS, splits added
-        up by the operator that follows) stand for F.linear on the three smaller matrices.  Measured
-        end to end, this route overtakes the fused single-launch linears at 7 rows (level at 6, +5 % at
-        8, +12..18 % from 11 on): every workgroup of those re-reads the activations of its k range."""
+        """5..64 activation rows: the split-K linears (activations shared through LDS, splits added
+        up by the operator that follows) stand for F.linear on the output and down projections, and
+        from 17 rows on for the qkv projection too.  Measured end to end, this route overtakes the
+        fused single-launch linears at 5 rows (+6 % at 5, +8 % at 6, more beyond): every workgroup of
+        those re-reads the activations of its k range, which the 8192-wide down projection feels first."""
         return self.decode_linear_rows > 0 and self.FUSED_MAX_ROWS < rows <= 64 and hasattr(self.ops, "linear_splitk")
 
     def _gate_up(self, L):
@@ -155,15 +157,18 @@ class LlamaDecoder:
             L["c_fc_cat"] = torch.cat([L["c_fc2"], L["c_fc"]], dim=0)
         return L["c_fc_cat"]
 
-    def _decode_layers_splitk(self, x, append_and_attend):
-        """The layers of one decode step (T == 1) at 7..64 rows; returns the final hidden state.
-        append_and_attend(L, qkv partial products) -> attention output (B, 1, C)."""
+    def _decode_layers_splitk(self, x, append_and_attend, project_and_attend=None):
+        """The layers of one decode step (T == 1) at 5..64 rows; returns the final hidden state.
+        append_and_attend(L, qkv partial products) -> attention output (B, 1, C);
+        project_and_attend(L, normalised input) -> the same from the single-launch qkv projection
+        (rotary embedding and cache append inside), taken while the rows are few enough for it."""
         c, ops = self.config, self.ops
         H = c.hidden_dim
         rows = x.numel() // x.shape[-1]
+        qkv_fused = project_and_attend is not None and rows <= self.QKV_FUSED_MAX_ROWS
         h = ops.rms_norm(x, self.layers[0]["ln_1"], c.norm_eps)
         for i, L in enumerate(self.layers):
-            y = append_and_attend(L, ops.linear_splitk(h, L["c_attn"]))
+            y = project_and_attend(L, h) if qkv_fused else append_and_attend(L, ops.linear_splitk(h, L["c_attn"]))
             x, h = ops.add_rms_norm_partials(x, ops.linear_splitk(y, L["c_proj"]), L["ln_2"], c.norm_eps)
             if rows <= self.SWIGLU_MAX_ROWS:
                 t = ops.linear_swiglu_decode(h, L["c_fc2"], L["c_fc"])     # one launch for the pair and the product
@@ -216,7 +221,14 @@ class LlamaDecoder:
                                                     L["cache_v"][:B, :start_pos + 1].transpose(1, 2))
                 return y.transpose(1, 2).reshape(B, 1, c.n_embd)
 
-            h = self._decode_layers_splitk(x, append_and_attend)
+            def project_and_attend(L, hn):
+                q = self.ops.linear_qkv_rope_append(hn, L["c_attn"], self.freqs_cis, L["cache_k"], L["cache_v"], pos,
+                                                    c.n_head)
+                y = self.ops.flash_attention_decode(q.transpose(1, 2), L["cache_k"][:B, :start_pos + 1].transpose(1, 2),
+                                                    L["cache_v"][:B, :start_pos + 1].transpose(1, 2))
+                return y.transpose(1, 2).reshape(B, 1, c.n_embd)
+
+            h = self._decode_layers_splitk(x, append_and_attend, project_and_attend)
             return F.linear(h, self.wte).float()
         for L in self.layers:
             x = x + self._attention(L, self.ops.rms_norm(x, L["ln_1"], c.norm_eps), freqs_cis, start_pos)
@@ -370,7 +382,14 @@ class GraphedDecodeLoop:
                                                       L["cache_v"][:B].transpose(1, 2), self.kv_len)
                 return y.transpose(1, 2).reshape(B, 1, c.n_embd)
 
-            logits = F.linear(m._decode_layers_splitk(x, append_and_attend)[:, -1], m.wte)
+            def project_and_attend(L, hn):
+                q = ops.linear_qkv_rope_append(hn, L["c_attn"], m.freqs_cis, L["cache_k"], L["cache_v"], self.pos,
+                                               c.n_head)
+                y = ops.flash_attention_decode_devlen(q.transpose(1, 2), L["cache_k"][:B].transpose(1, 2),
+                                                      L["cache_v"][:B].transpose(1, 2), self.kv_len)
+                return y.transpose(1, 2).reshape(B, 1, c.n_embd)
+
+            logits = F.linear(m._decode_layers_splitk(x, append_and_attend, project_and_attend)[:, -1], m.wte)
         else:
             h = ops.rms_norm(x, m.layers[0]["ln_1"], c.norm_eps)
             for i, L in enumerate(m.layers):
