@@ -55,6 +55,11 @@ linear_rows64_kernel(const LinearParams p) {
 
     const int total_chunks = p.K / KC;
     const int rounds = (total_chunks + RC - 1) / RC;
+    // Workgroups walk over K in the same cyclic order but start at different rounds: weight rows are
+    // a power of two apart in memory, and with every workgroup of the device on the same 1 KiB column
+    // strip at the same time only a fraction of the memory channels would be busy.  (With a ragged
+    // last round everyone starts at round 0, so that the ragged round stays the last.)
+    const int first_round = (total_chunks % RC == 0) ? int(blockIdx.x) % rounds : 0;
 
     // staging roles: 64 rows x 16 pieces of 16 bytes per chunk = 1024 pieces over 512 threads
     const int st_row = tid / 16, st_col = tid % 16;           // rows st_row and st_row + 32
@@ -74,7 +79,7 @@ linear_rows64_kernel(const LinearParams p) {
     // simply waits for everything).
     auto request = [&](auto full_tag, int r, uint4 (&rw)[WC][SPC]) {
         constexpr bool FULL = decltype(full_tag)::value;
-        const int c0 = r * RC;
+        const int c0 = ((r + first_round) % rounds) * RC;
         const int n = FULL ? RC : total_chunks - c0;
 #pragma unroll
         for (int j = 0; j < RC; ++j) {
