@@ -76,8 +76,9 @@ int l3_attn_set_option(int option, int value);
  * Split count the attention kernel would pick for this problem on a device with
  * `num_cus` compute units (<= 0: ask the current HIP device, 256 if there is none).
  * Pure integer host logic.  Replaces the fixed rule n_step = ceil(S / 64) of
- * custom_kernels.cu:243,251; the count is chosen so that the wavefronts fill the device
- * while every split keeps at least one full tile of tokens.
+ * custom_kernels.cu:243,251; the count is chosen so that the workgroups fill the device (one
+ * per compute unit, three quarters of them when there are many sequences, a single split
+ * where that saves the combine) while every split keeps at least one full tile of tokens.
  * Returns a value in [1, L3_ATTN_MAX_SPLITS], or a negative error code.
  */
 int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus);
