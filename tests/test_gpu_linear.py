@@ -76,7 +76,8 @@ def test_linear_decode_layouts_and_errors(gpu):
 
 @pytest.mark.parametrize("M,N,K", [(1, 8192, 2048), (12, 8192, 2048), (7, 1024, 256), (16, 14336, 4096), (9, 52, 64),
                                    (64, 8192, 2048), (17, 8192, 2048), (40, 52, 640), (33, 1000, 1408), (64, 14336, 4096),
-                                   (20, 96, 128)])
+                                   (20, 96, 128), (4, 1684, 1024), (2, 1684, 2048), (13, 3420, 4096), (4, 4680, 3072),
+                                   (15, 3804, 4096)])
 def test_linear_swiglu_decode(gpu, M, N, K):
     from custom_kernels import custom_kernels_extension as cke
 
@@ -88,19 +89,17 @@ def test_linear_swiglu_decode(gpu, M, N, K):
     y = cke.linear_swiglu_decode(xd, wgd, wud)
     torch.cuda.synchronize()
     assert y.shape == (M, N)
-    # the fused kernel accumulates in the same order as the plain one: the three-operator sequence
-    # gives the same bits
+    # The three-operator sequence has the same rounding points.  The sums over K are not added up in
+    # the same order, though (the fused form deals its wavefronts over two matrices, and up to 4 rows
+    # the plain linear splits the k range of a small matrix further; above 16 rows it may go split-K):
+    # a gate or up value whose float32 sum straddles a bf16 rounding boundary rounds the other way
+    # now and then, and the product follows.
     if M > 16 and N % 8:
         seq = y          # the split-K route of the plain linear needs N % 8 == 0: oracle only
     else:
         seq = cke.silu_mul(cke.linear_decode(xd, wgd), cke.linear_decode(xd, wud))
-    if M <= 16:
-        assert torch.equal(y, seq)
-    else:
-        # above 16 rows the plain linear may add its k ranges up in another order (split-K): a gate or
-        # up value can round the other way now and then
-        dseq = bf16_ulp_distance(t2bits(y), t2bits(seq))
-        assert (dseq > 0).mean() < 0.02 and (dseq > 2).mean() < 2e-3
+    dseq = bf16_ulp_distance(t2bits(y), t2bits(seq))
+    assert (dseq > 0).mean() < 0.02 and (dseq > 2).mean() < 2e-3
     # against exact arithmetic with the same rounding points: a gate or up value that rounds the other
     # way moves the product by about one ulp of that factor
     ref = swiglu_linear_ref(t2f32(x), t2f32(wg), t2f32(wu))
