@@ -307,7 +307,8 @@ int l3_linear_splitk_finish(const void* part, int ksplit, const void* residual, 
 /*
  * l3_add_rms_norm whose residual operand is a split-K linear's partial products (`part`,
  * ksplit x rows x C floats): r = bf16(sum of the splits), sum_out = bf16(x + r),
- * y = rms_norm(sum_out) -- the bits of the unsplit sequence given the same r.  C % 8 == 0,
+ * y = rms_norm(sum_out): sum_out has the bits of the unsplit sequence given the same r; y agrees
+ * with l3_rms_norm of it to one bf16 ulp (the squares are added in another order).  C % 8 == 0,
  * C <= 8192; all pointers 16-byte aligned.
  */
 int l3_add_rms_norm_partials(const void* x, const void* part, int ksplit, const void* w, void* sum_out, void* y,
