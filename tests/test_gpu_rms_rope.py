@@ -158,6 +158,23 @@ def test_rot_embed_cancellation_stays_within_one_ulp(gpu):
     assert_within_ulps(out, rot_embed_ref(t2f32(xb), tab), 1, what="cancelling pairs")
 
 
+@pytest.mark.parametrize("B,T,NH,HD", [(2, 37, 80, 128), (1, 300, 132, 64), (3, 5, 96, 128)])
+def test_rot_embed_many_heads(gpu, B, T, NH, HD):
+    """More heads than a workgroup's threads can share per token (16-byte chunks x head groups > 256):
+    the flat one-item-per-lane kernel."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    print(f"rot_embed B={B} T={T} NH={NH} HD={HD}", flush=True)
+    tab = precompute_freqs_cis_ref(HD, 100 + T, theta=500000.0, use_scaled=True, scale_factor=32.0)[100:]
+    wide = randn_bf16((B, T, NH * HD + 64), 91)
+    x = wide[..., :NH * HD].view(B, T, NH, HD)
+    xg = wide.to(gpu)[..., :NH * HD].view(B, T, NH, HD)
+    out = cke.rot_embed(xg, torch.from_numpy(np.ascontiguousarray(tab)).to(gpu))
+    torch.cuda.synchronize()
+    assert out.is_contiguous()
+    assert_within_ulps(out, rot_embed_ref(t2f32(x), tab), 1, what=f"rope {tuple(x.shape)}")
+
+
 def test_rot_embed_pair_path_and_errors(gpu):
     from custom_kernels import custom_kernels_extension as cke
 
