@@ -111,7 +111,7 @@ def test_linear_swiglu_decode(gpu, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 3072, 2048), (8, 3072, 2048), (11, 512, 2048), (1, 2048, 8192), (2, 128, 8192),
-                                   (16, 100, 512), (3, 128256, 2048), (5, 64, 1536), (5, 4096, 4096)])
+                                   (16, 100, 512), (3, 128256, 2048), (5, 64, 1536), (5, 4096, 4096), (5, 2048, 4096)])
 def test_linear_fused_input_norm(gpu, M, N, K):
     from custom_kernels import custom_kernels_extension as cke
     from oracle import rms_norm_ref, round_to_bf16
