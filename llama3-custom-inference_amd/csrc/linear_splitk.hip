@@ -182,7 +182,7 @@ linear_splitk_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
 // operator to fold the sum into.  Eight outputs per lane.
 __global__ void __launch_bounds__(256)
 linear_splitk_finish_kernel(const float* __restrict__ part, int ksplit, int64_t split_stride,
-                            const uint16_t* __restrict__ res, uint16_t* __restrict__ y, int M, int N, int64_t y_stride) {
+                            const uint16_t* __restrict__ res, uint16_t* __restrict__ y, int N, int64_t y_stride) {
     const int vi = int(blockIdx.x) * 256 + threadIdx.x;   // blockIdx.y is the activation row
     if (vi >= N / 8) return;
     const int m = blockIdx.y;
@@ -205,7 +205,7 @@ linear_splitk_finish_kernel(const float* __restrict__ part, int ksplit, int64_t 
 int launch_linear_splitk_finish(const float* part, int ksplit, const uint16_t* res, uint16_t* y, int M, int N,
                                 int64_t y_stride, hipStream_t stream) {
     hipLaunchKernelGGL(linear_splitk_finish_kernel, dim3(unsigned((N / 8 + 255) / 256), unsigned(M)), dim3(256), 0,
-                       stream, part, ksplit, int64_t(M) * N, res, y, M, N, y_stride);
+                       stream, part, ksplit, int64_t(M) * N, res, y, N, y_stride);
     return int(hipGetLastError());
 }
 
