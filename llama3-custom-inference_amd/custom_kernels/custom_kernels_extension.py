@@ -446,15 +446,28 @@ def _linear_args(x, weights, max_rows=None):
     max_rows = _l3lib.L3_LINEAR_MAX_ROWS if max_rows is None else max_rows
     if x.dim() < 1 or rows < 1 or rows > max_rows:
         raise RuntimeError(f"linear_decode: 1..{max_rows} activation rows expected, got {tuple(x.shape)}")
+    w0 = weights[0]
     for w in weights:
         _require_gpu_bf16("weight", w)
-        if w.dim() != 2 or w.shape[1] != K or w.stride(1) != 1 or tuple(w.shape) != tuple(weights[0].shape) \
-                or w.stride(0) != weights[0].stride(0):
+        if w.dim() != 2 or w.shape[1] != K or w.stride(1) != 1 or \
+                (w is not w0 and (w.shape[0] != w0.shape[0] or w.stride(0) != w0.stride(0))):
             raise RuntimeError(f"linear_decode: weight {tuple(w.shape)} does not fit x {tuple(x.shape)}")
-    x2 = x.reshape(rows, K)
-    if x2.stride(1) != 1:
-        x2 = x2.contiguous()
-    return x2, rows, weights[0].shape[0], K
+    if x.dim() == 2 and x.stride(1) == 1:
+        x2 = x                          # rows as they are (any row stride)
+    elif x.is_contiguous():
+        x2 = x.view(rows, K)
+    else:
+        x2 = x.reshape(rows, K)
+        if x2.stride(1) != 1:
+            x2 = x2.contiguous()
+    return x2, rows, w0.shape[0], K
+
+
+def _rows_out(x, rows: int, N: int):
+    """A contiguous output of x's leading shape with N columns, (rows, N) to the kernel."""
+    if x.dim() == 2:
+        return x.new_empty((rows, N))
+    return x.new_empty(x.shape[:-1] + (N,))
 
 
 def _use_splitk(x, weight) -> bool:
@@ -481,13 +494,13 @@ def linear_decode(x, weight):
     if _use_splitk(x, weight):
         return linear_splitk_finish(linear_splitk(x, weight)).view(*x.shape[:-1], weight.shape[0])
     x2, rows, N, K = _linear_args(x, (weight,))
-    y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
+    y = _rows_out(x, rows, N)
     with _on_device(x.device):
         rc = lib.l3_linear_decode(x2.data_ptr(), weight.data_ptr(), y.data_ptr(), rows, N, K, x2.stride(0),
                                   weight.stride(0), N, _stream_ptr(x.device))
     if rc != 0:
         _fail(rc, f"M={rows} N={N} K={K}")
-    return y.view(*x.shape[:-1], N)
+    return y
 
 
 def linear_swiglu_decode(x, w_gate, w_up):
@@ -495,13 +508,13 @@ def linear_swiglu_decode(x, w_gate, w_up):
     launch (model.py:134 with w_gate = c_fc2, w_up = c_fc), same rounding points.  An extension."""
     lib = _l3lib.load()
     x2, rows, N, K = _linear_args(x, (w_gate, w_up))
-    y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
+    y = _rows_out(x, rows, N)
     with _on_device(x.device):
         rc = lib.l3_linear_swiglu_decode(x2.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(), y.data_ptr(), rows, N, K,
                                          x2.stride(0), w_gate.stride(0), N, _stream_ptr(x.device))
     if rc != 0:
         _fail(rc, f"M={rows} N={N} K={K}")
-    return y.view(*x.shape[:-1], N)
+    return y
 
 
 def linear_decode_fused_max_rows(K: int) -> int:
@@ -531,10 +544,8 @@ def linear_decode_fused(x, weight, norm_weight=None, eps: float = 1e-5, w_up=Non
         _require_gpu_bf16("residual", residual)
         if residual.numel() != rows * N or residual.shape[-1] != N:
             raise RuntimeError(f"linear_decode_fused: residual {tuple(residual.shape)} does not fit ({rows}, {N})")
-        r2 = residual.reshape(rows, N)
-        if not r2.is_contiguous():
-            r2 = r2.contiguous()
-    y = torch.empty((rows, N), dtype=x.dtype, device=x.device)
+        r2 = residual if residual.is_contiguous() else residual.reshape(rows, N).contiguous()
+    y = _rows_out(x, rows, N)
     with _on_device(x.device):
         rc = lib.l3_linear_decode_fused(x2.data_ptr(), None if norm_weight is None else norm_weight.data_ptr(),
                                         float(eps), weight.data_ptr(), None if w_up is None else w_up.data_ptr(),
@@ -542,7 +553,7 @@ def linear_decode_fused(x, weight, norm_weight=None, eps: float = 1e-5, w_up=Non
                                         x2.stride(0), weight.stride(0), N, _stream_ptr(x.device))
     if rc != 0:
         _fail(rc, f"M={rows} N={N} K={K}")
-    return y.view(*x.shape[:-1], N)
+    return y
 
 
 def linear_splitk(x, weight, ksplit: int = 0):
