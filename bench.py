@@ -34,6 +34,7 @@ for _p in (ROOT, PKG):
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 SEED = 42               # the reference's default seed (benchmark_kernel.py:126)
 FORCE_SPLITS = 0        # --splits
+ATTN_FLAGS = 0          # --attn-kernel fma sets L3_ATTN_FLAG_KERNEL_FMA
 
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
@@ -49,9 +50,9 @@ MEASURED_TRAFFIC = {
 }
 
 
-def attn_kernel_name(lib):
+def attn_kernel_name(lib=None):
     from custom_kernels import _l3lib as l3
-    return "mfma" if lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL, -1) == l3.L3_ATTN_KERNEL_MFMA else "fma"
+    return "fma" if ATTN_FLAGS & l3.L3_ATTN_FLAG_KERNEL_FMA else "mfma"
 
 
 def attn_bytes(B, QH, KVH, S, HD):
@@ -90,8 +91,8 @@ class AttnCase:
         self.out = [torch.empty_like(t) for t in self.q]
         # 0 = the library plans for the current device (split count and kernel form)
         self.req_splits = FORCE_SPLITS
-        self.num_splits = FORCE_SPLITS or lib.l3_attn_choose_splits(B, KVH, S, HD, 0)
-        self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.req_splits)
+        self.num_splits = FORCE_SPLITS or lib.l3_attn_choose_splits(B, KVH, S, HD, 0, ATTN_FLAGS)
+        self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.req_splits, ATTN_FLAGS)
         self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
         self.part_o = self.part_ml = None
         self._args = []
@@ -102,7 +103,7 @@ class AttnCase:
                 B, QH, KVH, S, HD,
                 l3.i64_array((qt.stride(0), qt.stride(1))), l3.i64_array((kt.stride(0), kt.stride(1), kt.stride(2))),
                 l3.i64_array((vt.stride(0), vt.stride(1), vt.stride(2))), l3.i64_array((ot.stride(0), ot.stride(1))),
-                1.0 / math.sqrt(HD), self.req_splits))
+                1.0 / math.sqrt(HD), self.req_splits, ATTN_FLAGS))
 
     def launch(self, slot, stream_ptr):
         rc = self.lib.l3_attn_decode(*self._args[slot % self.slots], stream_ptr)
@@ -118,7 +119,7 @@ class AttnCase:
             self.part_ml = self.torch.empty((self.B, self.QH, n, 2), dtype=self.torch.float32, device=self.ws.device)
         rc = self.lib.l3_attn_split(a[0], a[1], a[2], self.part_o.data_ptr(), self.part_ml.data_ptr(),
                                     self.B, self.QH, self.KVH, self.S, self.HD, a[11], a[12], a[13], a[15],
-                                    self.req_splits, stream_ptr)
+                                    self.req_splits, ATTN_FLAGS, stream_ptr)
         if rc < 0:
             raise RuntimeError(f"l3_attn_split failed: {rc}")
 
@@ -398,18 +399,16 @@ def run_prefill(args, torch, lib, l3, dev):
         flops = 4.0 * B * QH * HD * (T * (T + 1) / 2)
         reps = 8
         forms = {}
-        for fname, form in (("auto", l3.L3_ATTN_PREFILL_AUTO), ("wave", l3.L3_ATTN_PREFILL_WAVE),
-                            ("tiled", l3.L3_ATTN_PREFILL_TILED), ("pipelined", l3.L3_ATTN_PREFILL_PIPELINED)):
-            prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, form)
-            cke.flash_attention_prefill(q, k, v)
-            gph = capture_graph(torch, lambda: [cke.flash_attention_prefill(q, k, v) for _ in range(reps)])
+        for fname in ("auto", "wave", "tiled", "pipelined"):
+            with cke.attention_flags(prefill=fname):
+                cke.flash_attention_prefill(q, k, v)
+                gph = capture_graph(torch, lambda: [cke.flash_attention_prefill(q, k, v) for _ in range(reps)])
             t_warm = time.perf_counter()    # untimed: after an idle spell the first milliseconds run at lower clocks
             while time.perf_counter() - t_warm < 0.03:
                 gph.replay()
                 torch.cuda.synchronize()
             forms[fname] = event_time_ms(torch, gph.replay, 5) / reps
             del gph
-            lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, prev)
         ms = forms["auto"]
         try:
             F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
@@ -584,9 +583,9 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.attn_kernel != "default":
-        lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL,
-                               l3.L3_ATTN_KERNEL_MFMA if args.attn_kernel == "mfma" else l3.L3_ATTN_KERNEL_FMA)
+    global ATTN_FLAGS
+    if args.attn_kernel == "fma":
+        ATTN_FLAGS = l3.L3_ATTN_FLAG_KERNEL_FMA
     attn_opts = {"split_kv_kernel": attn_kernel_name(lib)}
 
     if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):

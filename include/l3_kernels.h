@@ -37,7 +37,8 @@ enum {
     L3_ERR_ALIGNMENT = -6,      /* a base pointer is not aligned for the vector loads */
     L3_ERR_WORKSPACE = -7,      /* workspace NULL or smaller than l3_attn_decode_workspace_bytes */
     L3_ERR_SPLITS = -8,         /* num_splits negative or above L3_ATTN_MAX_SPLITS */
-    L3_ERR_HIP = -9             /* the HIP runtime reported an error at launch */
+    L3_ERR_HIP = -9,            /* the HIP runtime reported an error at launch */
+    L3_ERR_FLAGS = -10          /* bits set in `flags` that this version does not define */
 };
 
 #define L3_ATTN_MAX_SPLITS 512
@@ -49,28 +50,25 @@ int l3_version(void);
 const char* l3_strerror(int code);
 
 /*
- * Process-wide choice of the split-KV kernel l3_attn_decode launches: MFMA tiles fed through
- * LDS (the default, chosen by measurement) or FMA dot products on the vector ALUs.  Both
- * compute the same thing; the switch exists so that the comparison can be repeated (the
- * reference has one kernel and no counterpart of this call).  `option` must be
- * L3_ATTN_OPT_KERNEL; returns the previous value; a `value` other than the two kernels only
- * queries.  The initial value is MFMA unless the environment variable L3_ATTN_IMPL is "fma".
- * Split planning depends on the kernel, so choose before sizing workspaces.
- *
- * L3_ATTN_OPT_PREFILL chooses the form of l3_attn_prefill in the same way: AUTO (by prompt
- * length: WAVE for short prompts, PIPELINED for long ones), WAVE (every wavefront streams K/V on
- * its own), TILED (a workgroup shares K/V tiles; a tile's three phases run in turn) or PIPELINED
- * (the same tiling with the phases of three consecutive tiles interleaved).
+ * Per-call options of the attention entry points: the `flags` argument, 0 = the library's own
+ * choices.  The library keeps no option between calls (no setter, no environment variable), so
+ * calls from different threads cannot change each other's plan or workspace size; pass the same
+ * flags to l3_attn_choose_splits / l3_attn_decode_workspace_bytes as to the call they size.
+ *   L3_ATTN_FLAG_KERNEL_FMA  decode: the split-KV kernel built on FMA dot products on the vector
+ *                            ALUs instead of the default MFMA tiles fed through LDS.  Both compute
+ *                            the same thing; the flag exists so that the comparison can be repeated
+ *                            (the reference has one kernel and no counterpart of this choice).
+ *   L3_ATTN_FLAG_PREFILL_*   prefill: force one form of l3_attn_prefill instead of the choice by
+ *                            prompt length -- WAVE (every wavefront streams K/V on its own), TILED
+ *                            (a workgroup shares K/V tiles; a tile's three phases run in turn) or
+ *                            PIPELINED (the same tiling with the phases of three tiles interleaved).
+ * Any other bit gives L3_ERR_FLAGS.
  */
-#define L3_ATTN_OPT_KERNEL 0
-#define L3_ATTN_KERNEL_FMA 0
-#define L3_ATTN_KERNEL_MFMA 1
-#define L3_ATTN_OPT_PREFILL 1
-#define L3_ATTN_PREFILL_AUTO 0
-#define L3_ATTN_PREFILL_WAVE 1
-#define L3_ATTN_PREFILL_TILED 2
-#define L3_ATTN_PREFILL_PIPELINED 3
-int l3_attn_set_option(int option, int value);
+#define L3_ATTN_FLAG_KERNEL_FMA 0x1
+#define L3_ATTN_FLAG_PREFILL_WAVE 0x10
+#define L3_ATTN_FLAG_PREFILL_TILED 0x20
+#define L3_ATTN_FLAG_PREFILL_PIPELINED 0x30
+#define L3_ATTN_FLAG_PREFILL_MASK 0x30
 
 /*
  * Split count the attention kernel would pick for this problem on a device with
@@ -81,7 +79,7 @@ int l3_attn_set_option(int option, int value);
  * where that saves the combine) while every split keeps at least one full tile of tokens.
  * Returns a value in [1, L3_ATTN_MAX_SPLITS], or a negative error code.
  */
-int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus);
+int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus, int flags);
 
 /*
  * Bytes of workspace l3_attn_decode needs for `num_splits` (0 = the automatic choice for
@@ -89,7 +87,7 @@ int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus);
  * output directly).  Replaces the three per-call temporaries of custom_kernels.cu:269-271
  * (tmp_result, score_maxes, softmax_sums); partial outputs are kept in float32 here.
  */
-size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int num_splits);
+size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int num_splits, int flags);
 
 /*
  * out[b, h, :] = softmax(scale * q[b, h, :] . k[b, h / (QH/KVH), :, :]^T) @ v[b, h / (QH/KVH), :, :]
@@ -114,11 +112,11 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out,
                    int B, int QH, int KVH, int S, int HD,
                    const int64_t q_strides[2], const int64_t k_strides[3],
                    const int64_t v_strides[3], const int64_t out_strides[2],
-                   float scale, int num_splits, void* stream);
+                   float scale, int num_splits, int flags, void* stream);
 
 /*
  * l3_attn_decode with the KV length read from device memory at run time (*kv_len_dev, clamped to
- * max_S), so that one recorded launch -- a HIP graph node -- serves every step of a decode loop
+ * [1, max_S]: a length below 1 attends to token 0 alone), so that one recorded launch -- a HIP graph node -- serves every step of a decode loop
  * whose cache grows by a token per step.  `k`/`v` are views of the whole cache row range
  * [0, max_S) with the usual {batch, head, token} strides; the split plan and the workspace are
  * sized for max_S.  No counterpart in the reference, whose KV length is the tensor shape
@@ -129,7 +127,7 @@ int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out
                           int B, int QH, int KVH, int max_S, int HD,
                           const int64_t q_strides[2], const int64_t k_strides[3],
                           const int64_t v_strides[3], const int64_t out_strides[2],
-                          float scale, int num_splits, const int32_t* kv_len_dev, void* stream);
+                          float scale, int num_splits, int flags, const int32_t* kv_len_dev, void* stream);
 
 /*
  * Causal GQA attention for T > 1 query tokens per sequence (prompt prefill):
@@ -144,7 +142,7 @@ int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out
  */
 int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int B, int QH, int KVH, int T, int S,
                     int HD, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
-                    const int64_t out_strides[3], float scale, void* stream);
+                    const int64_t out_strides[3], float scale, int flags, void* stream);
 
 /*
  * The two stages of l3_attn_decode on their own, for callers that hold one sequence's KV
@@ -168,7 +166,7 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
 int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, float* part_ml,
                   int B, int QH, int KVH, int S, int HD,
                   const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
-                  float scale, int num_splits, void* stream);
+                  float scale, int num_splits, int flags, void* stream);
 int l3_attn_combine(const float* part_o, const float* part_ml, void* out, int B, int QH, int HD, int n,
                     const int64_t out_strides[2], void* stream);
 
@@ -217,15 +215,12 @@ int l3_silu_mul_rows(const void* a, const void* b, void* y, int64_t rows, int64_
  * float32 accumulation, one rounding.  Stands where the reference calls nn.Linear with T == 1
  * (model.py:95 c_attn, :121 c_proj, :134 mlp c_proj, :225 lm_head); hipBLASLt treats these as
  * GEMMs, this entry point as a single pass over the weight matrix at HBM speed.
- * 1 <= M <= L3_LINEAR_MAX_ROWS; N % 4 == 0; K % 32 == 0; strides are row strides in elements
- * (x_stride, w_stride >= K and multiples of 8; y_stride >= N and a multiple of 4); x and w
- * 16-byte aligned, y 8-byte aligned.  Needs no workspace.
- * Up to 16 rows (one 16-column block of the matrix instruction) every matrix shape is served at
- * HBM speed.  With 17 .. 64 rows (K % 128 == 0 then) a workgroup takes 128 weight rows and walks
- * over the whole of K, which suits matrices whose rows alone fill the device (N >= 64 x compute
- * units: a vocabulary projection); for the matrices of a few thousand rows use l3_linear_splitk.
+ * 1 <= M <= L3_LINEAR_MAX_ROWS (one 16-column block of the matrix instruction); N % 4 == 0; K % 32 == 0;
+ * strides are row strides in elements (x_stride, w_stride >= K and multiples of 8; y_stride >= N and a
+ * multiple of 4); x and w 16-byte aligned, y 8-byte aligned.  Needs no workspace.  For 17 .. 64 rows use
+ * l3_linear_splitk (matrices of a few thousand rows) or a library GEMM (larger ones).
  */
-#define L3_LINEAR_MAX_ROWS 64
+#define L3_LINEAR_MAX_ROWS 16
 int l3_linear_decode(const void* x, const void* w, void* y, int M, int N, int K, int64_t x_stride,
                      int64_t w_stride, int64_t y_stride, void* stream);
 
@@ -233,8 +228,7 @@ int l3_linear_decode(const void* x, const void* w, void* y, int M, int N, int K,
  * y[M, N] = silu(x . w_gate^T) * (x . w_up^T) in one pass over both weight matrices: the
  * SwiGLU front half of model.py:134 (F.silu(c_fc2(x)) * c_fc(x)).  Both products and the silu
  * are rounded to bf16 before the multiplication, as the three separate torch operators do.
- * Same constraints as l3_linear_decode; w_gate and w_up share w_stride.  With 17 .. 64 rows a
- * workgroup takes 32 output columns of both matrices (N >= 16 x compute units fills the device).
+ * Same constraints as l3_linear_decode; w_gate and w_up share w_stride.
  */
 int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up, void* y, int M, int N, int K,
                             int64_t x_stride, int64_t w_stride, int64_t y_stride, void* stream);
@@ -247,7 +241,7 @@ int l3_linear_swiglu_decode(const void* x, const void* w_gate, const void* w_up,
  *   t = w_up ? bf16(silu(bf16(h.w^T))) * bf16(h.w_up^T) : h.w^T                   (model.py:134)
  *   y = residual ? bf16(residual + bf16(t)) : bf16(t)                             (model.py:147-148)
  * with the rounding points of the separate operators.  residual has y's shape and row stride and
- * may be y itself.  The input norm stages x in LDS and needs M <= 16, K % 512 == 0 and M * (K + 8) <= 24576
+ * may be y itself.  The input norm stages x in LDS and needs K % 512 == 0 and M * (K + 8) <= 24576
  * (L3_ERR_SHAPE otherwise); everything else as for l3_linear_decode.
  */
 int l3_linear_decode_fused(const void* x, const void* norm_weight, float norm_eps, const void* w, const void* w_up,
@@ -324,7 +318,7 @@ int l3_rot_embed_append_partials(const void* part, int ksplit, const float* freq
 
 /*
  * out[r] = index of the first maximum of the bf16 row logits[r*row_stride : r*row_stride + V]
- * (int64, like torch.argmax; a row of NaNs gives 0): the greedy pick of model.py:371.  Two small
+ * (int64; a NaN counts as the maximum and the first one wins, as in torch.argmax): the greedy pick of model.py:371.  Two small
  * launches (per-chunk maxima into the caller's workspace of l3_argmax_workspace_bytes(rows, V)
  * bytes, then one merge per row).  rows <= 65535.  No counterpart among the reference's kernels.
  */
@@ -380,6 +374,18 @@ int l3_rot_embed(const void* x, const float* freq, void* y, int B, int T, int NH
 int l3_rot_embed_append(const void* qkv, const float* freq_table, void* q_out, void* cache_k, void* cache_v,
                         const int32_t* pos_dev, int B, int NH, int KVH, int HD, int64_t qkv_batch_stride,
                         const int64_t cache_strides[2], int cache_len, int table_rows, void* stream);
+
+/*
+ * Measurement yardstick, not an operator: reads `bytes` (a multiple of 16, 16-byte aligned) of
+ * device memory once with 16-byte loads from `workgroups` 512-thread workgroups (<= 0: four per
+ * compute unit), all workgroups together sweeping the buffer front to back.  The loads are kept
+ * alive by xor-ing what they return; the xor goes to `sink` (4 bytes, device memory) only when it
+ * equals a constant that no realistic input produces, so the kernel writes nothing.  Timed by the
+ * benchmark over buffers larger than the memory-side cache, it gives the read bandwidth this
+ * device delivers to a pure stream: the ceiling every HBM-bound kernel here is read against.
+ * No counterpart in the reference.
+ */
+int l3_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups, void* stream);
 
 #ifdef __cplusplus
 }

@@ -53,7 +53,7 @@ attn_splitkv_fma_kernel(const AttnParams p) {
     const int b = bid % p.B;
     const int split = bid / p.B;
     const int t_begin = split * p.tokens_per_split;
-    const int S = p.seqlen_dev ? min(*p.seqlen_dev, p.S) : p.S;  // wave-uniform
+    const int S = p.seqlen_dev ? max(1, min(*p.seqlen_dev, p.S)) : p.S;  // wave-uniform; a length below 1 counts as 1
     if (t_begin >= S) return;  // whole workgroup: split beyond a device-side KV length, the combine skips it
     const int t_end = min(S, t_begin + p.tokens_per_split);
 

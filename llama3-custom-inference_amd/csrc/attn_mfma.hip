@@ -69,7 +69,7 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
         if (split >= p.num_splits) return;  // whole wavefront; no barrier follows
     }
     const int t_begin = split * p.tokens_per_split;
-    const int S = p.seqlen_dev ? min(*p.seqlen_dev, p.S) : p.S;  // wave-uniform
+    const int S = p.seqlen_dev ? max(1, min(*p.seqlen_dev, p.S)) : p.S;  // wave-uniform; a length below 1 counts as 1
     if (t_begin >= S) return;  // split beyond a device-side KV length (whole workgroup when COOP): the combine skips it
     const int t_end = min(S, t_begin + p.tokens_per_split);
     const float c = p.scale_log2e;

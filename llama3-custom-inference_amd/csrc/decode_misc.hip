@@ -44,9 +44,11 @@ silu_mul_scalar_kernel(const uint16_t* __restrict__ a, const uint16_t* __restric
 }
 
 // (value, index) pairs ordered by value, then by smaller index: the first maximum wins, as
-// torch.argmax documents.  NaN never wins against a number (comparisons with NaN are false).
+// torch.argmax documents.  A NaN ranks above every number (the first NaN wins), which is how
+// torch.argmax treats it: a numerical blow-up shows up in the token stream the same way on both paths.
 __device__ __forceinline__ void argmax_merge(float& v, int& idx, float ov, int oidx) {
-    if (ov > v || (ov == v && oidx < idx)) {
+    const bool o_nan = ov != ov, v_nan = v != v;
+    if (o_nan ? (!v_nan || oidx < idx) : (!v_nan && (ov > v || (ov == v && oidx < idx)))) {
         v = ov;
         idx = oidx;
     }
@@ -96,7 +98,7 @@ argmax_final_kernel(const float* __restrict__ part_val, const int* __restrict__ 
     for (int off = 1; off < kWaveSize; off <<= 1) {
         argmax_merge(v, idx, __shfl_xor(v, off, kWaveSize), __shfl_xor(idx, off, kWaveSize));
     }
-    if (threadIdx.x == 0) out[row] = (idx == 0x7fffffff) ? 0 : idx;  // all-NaN row: index 0
+    if (threadIdx.x == 0) out[row] = (idx == 0x7fffffff) ? 0 : idx;  // V == 0 cannot happen (checked by the caller)
 }
 
 // Second argmax stage fused with the bookkeeping generate() does per greedy token

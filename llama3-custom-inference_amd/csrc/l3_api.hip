@@ -60,18 +60,10 @@ int current_device_cus() {
 }
 
 namespace {
-std::atomic<int> g_attn_kernel{-1};  // -1: not chosen yet
-std::atomic<int> g_prefill_form{L3_ATTN_PREFILL_AUTO};
+// The split-KV kernel a call's flags ask for (the library keeps no such choice between calls).
+int attn_impl_of(int flags) { return (flags & L3_ATTN_FLAG_KERNEL_FMA) ? kAttnImplFma : kAttnImplMfma; }
+bool attn_flags_ok(int flags) { return (flags & ~(L3_ATTN_FLAG_KERNEL_FMA | L3_ATTN_FLAG_PREFILL_MASK)) == 0; }
 }  // namespace
-
-int attn_kernel_option() {
-    int v = g_attn_kernel.load(std::memory_order_relaxed);
-    if (v >= 0) return v;
-    const char* e = getenv("L3_ATTN_IMPL");
-    v = (e && strcmp(e, "fma") == 0) ? kAttnImplFma : kAttnImplMfma;
-    g_attn_kernel.store(v, std::memory_order_relaxed);
-    return v;
-}
 
 AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl) {
     const int tile = attn_tile_tokens(HD, impl);
@@ -152,36 +144,24 @@ const char* l3_strerror(int code) {
         case L3_ERR_WORKSPACE: return "workspace missing or too small";
         case L3_ERR_SPLITS: return "num_splits out of range";
         case L3_ERR_HIP: return "HIP runtime error at kernel launch";
+        case L3_ERR_FLAGS: return "unknown bits in flags";
         default: return "unknown error code";
     }
 }
 
-int l3_attn_set_option(int option, int value) {
-    if (option == L3_ATTN_OPT_PREFILL) {
-        const int prev_form = g_prefill_form.load(std::memory_order_relaxed);
-        if (value == L3_ATTN_PREFILL_AUTO || value == L3_ATTN_PREFILL_WAVE || value == L3_ATTN_PREFILL_TILED ||
-            value == L3_ATTN_PREFILL_PIPELINED)
-            g_prefill_form.store(value, std::memory_order_relaxed);
-        return prev_form;
-    }
-    if (option != L3_ATTN_OPT_KERNEL) return L3_ERR_SHAPE;
-    const int prev = attn_kernel_option();
-    if (value == L3_ATTN_KERNEL_FMA || value == L3_ATTN_KERNEL_MFMA) g_attn_kernel.store(value, std::memory_order_relaxed);
-    return prev;
-}
-
-int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus) {
+int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus, int flags) {
     if (HD != 64 && HD != 128) return L3_ERR_HEAD_SIZE;
     if (B <= 0 || KVH <= 0 || S <= 0) return L3_ERR_SHAPE;
+    if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
     if (num_cus <= 0) num_cus = current_device_cus();
-    return attn_make_plan(B, KVH, S, HD, 0, num_cus, attn_kernel_option()).num_splits;
+    return attn_make_plan(B, KVH, S, HD, 0, num_cus, attn_impl_of(flags)).num_splits;
 }
 
-size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int num_splits) {
+size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int num_splits, int flags) {
     if (check_attn_shape(B, QH, KVH, S, HD) != L3_OK) return 0;
-    if (num_splits < 0 || num_splits > L3_ATTN_MAX_SPLITS) return 0;
+    if (num_splits < 0 || num_splits > L3_ATTN_MAX_SPLITS || !attn_flags_ok(flags)) return 0;
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
-    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, attn_kernel_option());
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, attn_impl_of(flags));
     return attn_workspace_bytes(B, QH, HD, plan.num_splits);
 }
 
@@ -245,12 +225,13 @@ namespace {
 int attn_decode_impl(const void* q, const void* k, const void* v, void* out, void* workspace,
                      size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
                      const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
-                     const int64_t out_strides[2], float scale, int num_splits, const int* seqlen_dev,
+                     const int64_t out_strides[2], float scale, int num_splits, int flags, const int* seqlen_dev,
                      void* stream) {
     if (int rc = check_attn_args(q, k, v, out, B, QH, KVH, S, HD, q_strides, k_strides, v_strides, out_strides,
                                  num_splits, true); rc != L3_OK)
         return rc;
-    const int impl = attn_kernel_option();
+    if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
+    const int impl = attn_impl_of(flags);
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
     const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
     const size_t need = attn_workspace_bytes(B, QH, HD, plan.num_splits);
@@ -277,28 +258,29 @@ int attn_decode_impl(const void* q, const void* k, const void* v, void* out, voi
 int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void* workspace,
                    size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
                    const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
-                   const int64_t out_strides[2], float scale, int num_splits, void* stream) {
+                   const int64_t out_strides[2], float scale, int num_splits, int flags, void* stream) {
     return attn_decode_impl(q, k, v, out, workspace, workspace_bytes, B, QH, KVH, S, HD, q_strides, k_strides,
-                            v_strides, out_strides, scale, num_splits, nullptr, stream);
+                            v_strides, out_strides, scale, num_splits, flags, nullptr, stream);
 }
 
 int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out, void* workspace,
                           size_t workspace_bytes, int B, int QH, int KVH, int max_S, int HD,
                           const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
-                          const int64_t out_strides[2], float scale, int num_splits, const int32_t* kv_len_dev,
-                          void* stream) {
+                          const int64_t out_strides[2], float scale, int num_splits, int flags,
+                          const int32_t* kv_len_dev, void* stream) {
     if (!kv_len_dev) return L3_ERR_NULL_POINTER;
     if (!aligned(kv_len_dev, 4)) return L3_ERR_ALIGNMENT;
     return attn_decode_impl(q, k, v, out, workspace, workspace_bytes, B, QH, KVH, max_S, HD, q_strides, k_strides,
-                            v_strides, out_strides, scale, num_splits, kv_len_dev, stream);
+                            v_strides, out_strides, scale, num_splits, flags, kv_len_dev, stream);
 }
 
 int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int B, int QH, int KVH, int T, int S,
                     int HD, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
-                    const int64_t out_strides[3], float scale, void* stream) {
+                    const int64_t out_strides[3], float scale, int flags, void* stream) {
     if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !out_strides)
         return L3_ERR_NULL_POINTER;
     if (int rc = check_attn_shape(B, QH, KVH, S, HD); rc != L3_OK) return rc;
+    if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
     if (T <= 0 || T > S) return L3_ERR_SHAPE;
     if (int64_t(B) * KVH * ((int64_t(T) + 1) / 2 + kMfmaWaves) >= (int64_t(1) << 31)) return L3_ERR_SHAPE;  // grid
     const int q_dims[3] = {B, QH, T};
@@ -326,31 +308,33 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     // measured (head ratios 1, 3, 4 and 8), the tiled form wins from 192 tokens (head size 64) or
     // 384 tokens (128) on, and earlier when the wavefront-private form would need more than eight
     // wavefronts per compute unit and the prompt fills at least one workgroup of the tiled form.
-    int form = g_prefill_form.load(std::memory_order_relaxed);
-    if (form == L3_ATTN_PREFILL_AUTO) {
+    int form = flags & L3_ATTN_FLAG_PREFILL_MASK;
+    if (form == 0) {
         const int R = QH / KVH;
         const int wg_pos = prefill_tiled_positions_per_wg(HD, R);
         const int64_t private_waves = int64_t(B) * KVH * ((int64_t(T) * R + 15) / 16);
         const int long_prompt = HD == 64 ? 192 : 384;
         const bool tiled = T >= long_prompt || (T >= wg_pos && private_waves > 8 * int64_t(current_device_cus()));
-        form = tiled ? L3_ATTN_PREFILL_PIPELINED : L3_ATTN_PREFILL_WAVE;
+        form = tiled ? L3_ATTN_FLAG_PREFILL_PIPELINED : L3_ATTN_FLAG_PREFILL_WAVE;
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int rc = (form == L3_ATTN_PREFILL_WAVE) ? launch_attn_prefill(p, HD, st)
-                                                  : launch_attn_prefill_tiled(p, HD, form == L3_ATTN_PREFILL_PIPELINED, st);
+    const int rc = (form == L3_ATTN_FLAG_PREFILL_WAVE)
+                       ? launch_attn_prefill(p, HD, st)
+                       : launch_attn_prefill_tiled(p, HD, form == L3_ATTN_FLAG_PREFILL_PIPELINED, st);
     return rc == 0 ? L3_OK : L3_ERR_HIP;
 }
 
 int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, float* part_ml,
                   int B, int QH, int KVH, int S, int HD,
                   const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
-                  float scale, int num_splits, void* stream) {
+                  float scale, int num_splits, int flags, void* stream) {
     if (!part_o || !part_ml) return L3_ERR_NULL_POINTER;
     if (int rc = check_attn_args(q, k, v, nullptr, B, QH, KVH, S, HD, q_strides, k_strides, v_strides, nullptr,
                                  num_splits, false); rc != L3_OK)
         return rc;
     if (!aligned(part_o, 16) || !aligned(part_ml, 8)) return L3_ERR_ALIGNMENT;
-    const int impl = attn_kernel_option();
+    if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
+    const int impl = attn_impl_of(flags);
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
     const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
     AttnParams p;
@@ -458,12 +442,6 @@ int linear_decode_impl(const void* x, const void* norm_w, float norm_eps, const 
         p.rope_table = nullptr; p.rope_pos = nullptr; p.q_out = p.cache_k = p.cache_v = nullptr;
         p.NH = p.KVH = p.HD = p.cache_len = p.table_rows = 0;
         p.c_sb = p.c_st = 0;
-    }
-    if (M > 16) {
-        // 17 .. 64 rows: the one-launch kernel that walks over K in rounds (no norm, no rope epilogue)
-        if (norm_w || qkv || K % 128 != 0) return L3_ERR_SHAPE;
-        if (x_stride % 8 || y_stride % 4) return L3_ERR_STRIDE;
-        return launch_linear_rows64(p, swiglu, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
     }
     return launch_linear_skinny(p, swiglu, current_device_cus(), static_cast<hipStream_t>(stream)) == 0 ? L3_OK
                                                                                                         : L3_ERR_HIP;
@@ -675,6 +653,16 @@ int l3_rot_embed_append(const void* qkv, const float* freq_table, void* q_out, v
                                    static_cast<uint16_t*>(cache_k), static_cast<uint16_t*>(cache_v), pos_dev, B, NH,
                                    KVH, HD, qkv_batch_stride, cache_strides[0], cache_strides[1], cache_len,
                                    table_rows, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+}
+
+int l3_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups, void* stream) {
+    if (!src || !sink) return L3_ERR_NULL_POINTER;
+    if (bytes == 0 || bytes % 16 != 0) return L3_ERR_SHAPE;
+    if (!aligned(src, 16) || !aligned(sink, 4)) return L3_ERR_ALIGNMENT;
+    if (workgroups <= 0) workgroups = 4 * current_device_cus();
+    if (workgroups > (1 << 20)) return L3_ERR_SHAPE;
+    return launch_hbm_read_stream(src, bytes, sink, workgroups, static_cast<hipStream_t>(stream)) == 0 ? L3_OK
+                                                                                                       : L3_ERR_HIP;
 }
 
 }  // extern "C"

@@ -32,9 +32,6 @@ constexpr int attn_tile_tokens(int HD, int impl) {
 // Adjacent kv heads that share a workgroup of the MFMA kernel (largest power of two <= 8 dividing KVH).
 int attn_mfma_heads_per_wg(int KVH);
 
-// Which kernel l3_attn_decode uses (see l3_attn_set_option in the C ABI).
-int attn_kernel_option();
-
 // Pure integer logic (no HIP): the plan for `requested` splits (0 = automatic).
 AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl);
 
@@ -104,7 +101,6 @@ int launch_rot_embed_append_partials(const float* part, int ksplit, int64_t spli
                                      uint16_t* q_out, uint16_t* cache_k, uint16_t* cache_v, const int* pos_dev, int B,
                                      int NH, int KVH, int HD, int64_t c_sb, int64_t c_st, int cache_len,
                                      int table_rows, hipStream_t stream);
-int launch_linear_rows64(const LinearParams& p, bool swiglu, hipStream_t stream);   // 17 .. 64 rows, one launch
 int linear_splitk_max_chunks(int N, int num_cus);
 int launch_linear_splitk(const uint16_t* x, const uint16_t* w, float* part, int M, int N, int K, int64_t x_stride,
                          int64_t w_stride, int ksplit, int num_cus, hipStream_t stream);
@@ -122,6 +118,7 @@ int launch_attn_prefill_tiled(const PrefillParams& p, int HD, bool pipelined, hi
 int launch_attn_splitkv_fma(const AttnParams& p, int HD, int R, hipStream_t stream);
 int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipStream_t stream);
 int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream);
+int launch_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups, hipStream_t stream);
 int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
                     bool vec_ok, hipStream_t stream);
 int launch_add_rms_norm(const uint16_t* x, const uint16_t* res, const uint16_t* w, uint16_t* sum_out, uint16_t* y,

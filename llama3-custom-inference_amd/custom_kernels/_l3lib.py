@@ -19,41 +19,38 @@ L3_ERR_ALIGNMENT = -6
 L3_ERR_WORKSPACE = -7
 L3_ERR_SPLITS = -8
 L3_ERR_HIP = -9
+L3_ERR_FLAGS = -10
 L3_ATTN_MAX_SPLITS = 512
-L3_LINEAR_MAX_ROWS = 64
-L3_LINEAR_FUSED_MAX_ROWS = 16   # rows up to which every matrix shape, the input norm and the rope epilogue are served
+L3_LINEAR_MAX_ROWS = 16         # one launch, any matrix shape, optional input norm / SwiGLU / residual / rope epilogue
 L3_LINEAR_SPLITK_MAX_ROWS = 64
 L3_LINEAR_STAGE_ELEMS = 24576   # activations (rows padded by 8) the fused input norm can stage in LDS
-L3_ATTN_OPT_KERNEL = 0
-L3_ATTN_KERNEL_FMA = 0
-L3_ATTN_KERNEL_MFMA = 1
-L3_ATTN_OPT_PREFILL = 1
-L3_ATTN_PREFILL_AUTO = 0
-L3_ATTN_PREFILL_WAVE = 1
-L3_ATTN_PREFILL_TILED = 2
-L3_ATTN_PREFILL_PIPELINED = 3
+L3_ATTN_FLAG_KERNEL_FMA = 0x1
+L3_ATTN_FLAG_PREFILL_WAVE = 0x10
+L3_ATTN_FLAG_PREFILL_TILED = 0x20
+L3_ATTN_FLAG_PREFILL_PIPELINED = 0x30
+L3_ATTN_FLAG_PREFILL_MASK = 0x30
 
 # name -> (restype, argtypes); mirrors include/l3_kernels.h line by line
 _c_i64p = ctypes.POINTER(ctypes.c_int64)
 SIGNATURES = {
     "l3_version": (ctypes.c_int, []),
     "l3_strerror": (ctypes.c_char_p, [ctypes.c_int]),
-    "l3_attn_set_option": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
-    "l3_attn_choose_splits": (ctypes.c_int, [ctypes.c_int] * 5),
-    "l3_attn_decode_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 6),
+    "l3_attn_choose_splits": (ctypes.c_int, [ctypes.c_int] * 6),
+    "l3_attn_decode_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 7),
     "l3_attn_decode": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v out
          ctypes.c_void_p, ctypes.c_size_t,                                    # workspace, bytes
          ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,  # B QH KVH S HD
          _c_i64p, _c_i64p, _c_i64p, _c_i64p,                                  # strides
-         ctypes.c_float, ctypes.c_int, ctypes.c_void_p],                      # scale splits stream
+         ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],        # scale splits flags stream
     ),
     "l3_attn_decode_devlen": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
          ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-         _c_i64p, _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p],
+         _c_i64p, _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+         ctypes.c_void_p],
     ),
     "l3_rot_embed_append": (
         ctypes.c_int,
@@ -65,13 +62,13 @@ SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,  # B QH KVH T S HD
-         _c_i64p, _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_void_p],
+         _c_i64p, _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_int, ctypes.c_void_p],
     ),
     "l3_attn_split": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v part_o part_ml
          ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,                   # B QH KVH S HD
-         _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_int, ctypes.c_void_p],
+         _c_i64p, _c_i64p, _c_i64p, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],
     ),
     "l3_attn_combine": (
         ctypes.c_int,
@@ -156,6 +153,9 @@ SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
          ctypes.c_int, _c_i64p, ctypes.c_void_p],
+    ),
+    "l3_hbm_read_stream": (
+        ctypes.c_int, [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p],
     ),
 }
 

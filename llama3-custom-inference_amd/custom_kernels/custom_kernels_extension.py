@@ -13,13 +13,14 @@ not synchronise.  There is no fallback path: a missing library or a non-GPU tens
 """
 
 import contextlib
+import contextvars
 import math
 
 import torch
 
 from . import _l3lib
 
-__all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits",
+__all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits", "attention_flags",
            "flash_attention_split", "flash_attention_combine", "flash_attention_decode_devlen",
            "rot_embed_append", "add_rms_norm", "silu_mul", "argmax", "flash_attention_prefill"]
 
@@ -89,21 +90,58 @@ def _workspace(device, stream_ptr: int, nbytes: int):
     return ws
 
 
-def attention_num_splits(B: int, KVH: int, S: int, HD: int, num_cus: int = 256) -> int:
+# Flags the attention operators pass to the library when the caller gives none: a context-local
+# value (per thread / per asyncio task), never a process-wide switch.  The library itself keeps no
+# option between calls.
+_attn_flags = contextvars.ContextVar("l3_attn_flags", default=0)
+
+_FLAG_NAMES = {"mfma": 0, "fma": _l3lib.L3_ATTN_FLAG_KERNEL_FMA, "auto": 0, "wave": _l3lib.L3_ATTN_FLAG_PREFILL_WAVE,
+               "tiled": _l3lib.L3_ATTN_FLAG_PREFILL_TILED, "pipelined": _l3lib.L3_ATTN_FLAG_PREFILL_PIPELINED}
+
+
+@contextlib.contextmanager
+def attention_flags(kernel: str = "mfma", prefill: str = "auto"):
+    """Within the block, attention calls of this thread that pass no ``flags`` use the named
+    split-KV kernel ("mfma" / "fma") and prefill form ("auto" / "wave" / "tiled" / "pipelined").
+    For measurements and tests; the defaults are the library's own choices."""
+    token = _attn_flags.set(_FLAG_NAMES[kernel] | _FLAG_NAMES[prefill])
+    try:
+        yield
+    finally:
+        _attn_flags.reset(token)
+
+
+def _flags(flags):
+    return _attn_flags.get() if flags is None else int(flags)
+
+
+def attention_num_splits(B: int, KVH: int, S: int, HD: int, num_cus: int = 256, flags=None) -> int:
     """Split count the kernel picks for this problem (pure host logic, runs without a GPU)."""
-    n = _l3lib.load().l3_attn_choose_splits(B, KVH, S, HD, num_cus)
+    n = _l3lib.load().l3_attn_choose_splits(B, KVH, S, HD, num_cus, _flags(flags))
     if n < 0:
         _fail(n)
     return n
 
 
-def flash_attention_decode(query, keys, values, num_splits: int = 0):
+def _check_out(out, like, what: str):
+    """A caller-supplied output is written through its raw pointer with `like`'s shape: it must be
+    a bf16 tensor of that shape on the same device whose rows the kernels can address."""
+    if not isinstance(out, torch.Tensor) or out.dtype != torch.bfloat16 or out.device != like.device \
+            or tuple(out.shape) != tuple(like.shape):
+        raise RuntimeError(f"{what}: out must be a bf16 tensor of shape {tuple(like.shape)} on {like.device}")
+    if out.stride(-1) != 1 or any(st % 8 for st, n in zip(out.stride()[:-1], out.shape[:-1]) if n > 1):
+        raise RuntimeError(f"{what}: out needs a contiguous last dimension and 16-byte aligned rows")
+
+
+def flash_attention_decode(query, keys, values, num_splits: int = 0, flags=None):
     """query (B, QH, 1, HD); keys/values (B, KVH, S, HD) views of the KV cache (model.py:107-118).
 
-    ``num_splits`` (0 = automatic) is an extension for tests and sweeps; the reference
-    signature is the three tensors.
+    ``num_splits`` (0 = automatic) and ``flags`` (L3_ATTN_FLAG_* bits, None = attention_flags()'s
+    context, normally 0) are extensions for tests and sweeps; the reference signature is the three
+    tensors.
     """
     lib = _l3lib.load()
+    flags = _flags(flags)
     B, QH, KVH, S, HD = _check_qkv(query, keys, values)
     if keys.device != query.device or values.device != query.device:
         raise RuntimeError("query, keys and values must be on the same device")
@@ -120,7 +158,7 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0):
 
     with _on_device(query.device):
         # num_splits == 0 lets the library plan for the current device (split count and kernel form)
-        ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, num_splits)
+        ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, num_splits, flags)
         stream_ptr = _stream_ptr(query.device)
         ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None
         rc = lib.l3_attn_decode(
@@ -131,7 +169,7 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0):
             _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
             _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
             _l3lib.i64_array((out.stride(0), out.stride(1))),
-            1.0 / math.sqrt(HD), num_splits, stream_ptr)
+            1.0 / math.sqrt(HD), num_splits, flags, stream_ptr)
     if rc != 0:
         _fail(rc, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
     return out
@@ -153,7 +191,7 @@ def _check_qkv(query, keys, values):
     return B, QH, KVH, S, HD
 
 
-def flash_attention_prefill(query, keys, values):
+def flash_attention_prefill(query, keys, values, flags=None):
     """Causal GQA attention for T > 1 query tokens: query (B, QH, T, HD), keys / values
     (B, KVH, S, HD) cache views with S >= T; query i attends to tokens 0 .. S - T + i.  Returns a
     (B, QH, T, HD) view of a contiguous (B, T, QH, HD) tensor, so the model's
@@ -185,22 +223,23 @@ def flash_attention_prefill(query, keys, values):
             _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
             _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
             _l3lib.i64_array((out.stride(0), out.stride(1), out.stride(2))),
-            1.0 / math.sqrt(HD), _stream_ptr(query.device))
+            1.0 / math.sqrt(HD), _flags(flags), _stream_ptr(query.device))
     if rc != 0:
         _fail(rc, f"B={B} QH={QH} KVH={KVH} T={T} S={S} HD={HD}")
     return out
 
 
-def flash_attention_split(query, keys, values, num_splits: int = 0):
+def flash_attention_split(query, keys, values, num_splits: int = 0, flags=None):
     """First stage of flash_attention_decode on its own (an extension; the reference runs its two
     kernels only together, custom_kernels.cu:274-275).  Returns float32 partials
     ``(part_o (B, QH, n, HD), part_ml (B, QH, n, 2))``: unnormalised outputs and (max, sum) per
     split, scores in log2 units.  Partials of several token ranges of one sequence can be
     concatenated along dim 2 and finished by flash_attention_combine."""
     lib = _l3lib.load()
+    flags = _flags(flags)
     B, QH, KVH, S, HD = _check_qkv(query, keys, values)
     with _on_device(query.device):
-        n_req = num_splits if num_splits > 0 else lib.l3_attn_choose_splits(B, KVH, S, HD, 0)
+        n_req = num_splits if num_splits > 0 else lib.l3_attn_choose_splits(B, KVH, S, HD, 0, flags)
         if n_req < 0:
             _fail(n_req)
         part_o = torch.empty((B, QH, n_req, HD), dtype=torch.float32, device=query.device)
@@ -211,7 +250,7 @@ def flash_attention_split(query, keys, values, num_splits: int = 0):
             _l3lib.i64_array((query.stride(0), query.stride(1))),
             _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
             _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
-            1.0 / math.sqrt(HD), num_splits, _stream_ptr(query.device))
+            1.0 / math.sqrt(HD), num_splits, flags, _stream_ptr(query.device))
     if n < 0:
         _fail(n, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
     if n != n_req:  # the kernel laid its rows out for n splits: re-view the front of the buffers
@@ -240,7 +279,7 @@ def flash_attention_combine(part_o, part_ml, dtype=torch.bfloat16):
     return out
 
 
-def flash_attention_decode_devlen(query, keys, values, kv_len, num_splits: int = 0, out=None):
+def flash_attention_decode_devlen(query, keys, values, kv_len, num_splits: int = 0, out=None, flags=None):
     """flash_attention_decode whose KV length is the int32 GPU scalar ``kv_len`` instead of the
     tensor shape: ``keys`` / ``values`` are (B, KVH, L, HD) views of the whole cache and only the
     first ``kv_len`` tokens are attended.  The launch does not depend on the length, so it can be
@@ -248,13 +287,18 @@ def flash_attention_decode_devlen(query, keys, values, kv_len, num_splits: int =
     takes the length from keys.size(2), custom_kernels.cu:246).  ``out`` may be supplied to keep
     the call allocation-free under capture."""
     lib = _l3lib.load()
+    flags = _flags(flags)
     B, QH, KVH, L, HD = _check_qkv(query, keys, values)
-    if not kv_len.is_cuda or kv_len.dtype != torch.int32 or kv_len.numel() != 1:
-        raise RuntimeError("kv_len must be a one-element int32 GPU tensor")
+    if keys.device != query.device or values.device != query.device:
+        raise RuntimeError("query, keys and values must be on the same device")
+    if not kv_len.is_cuda or kv_len.dtype != torch.int32 or kv_len.numel() != 1 or kv_len.device != query.device:
+        raise RuntimeError("kv_len must be a one-element int32 tensor on the query's GPU")
     if out is None:
         out = torch.empty_like(query)
+    else:
+        _check_out(out, query, "flash_attention_decode_devlen")
     with _on_device(query.device):
-        ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, L, HD, num_splits)
+        ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, L, HD, num_splits, flags)
         stream_ptr = _stream_ptr(query.device)
         ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None
         rc = lib.l3_attn_decode_devlen(
@@ -264,7 +308,7 @@ def flash_attention_decode_devlen(query, keys, values, kv_len, num_splits: int =
             _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
             _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
             _l3lib.i64_array((out.stride(0), out.stride(1))),
-            1.0 / math.sqrt(HD), num_splits, kv_len.data_ptr(), stream_ptr)
+            1.0 / math.sqrt(HD), num_splits, flags, kv_len.data_ptr(), stream_ptr)
     if rc != 0:
         _fail(rc, f"B={B} QH={QH} KVH={KVH} L={L} HD={HD}")
     return out
@@ -294,10 +338,16 @@ def rot_embed_append(qkv, freq_table, cache_k, cache_v, pos, n_head: int, out=No
     if not freq_table.is_cuda or freq_table.dtype != torch.float32 or freq_table.dim() != 2 \
             or freq_table.size(1) != HD or not freq_table.is_contiguous():
         raise RuntimeError("freq_table must be a contiguous (rows, HD) float32 GPU tensor")
-    if not pos.is_cuda or pos.dtype != torch.int32 or pos.numel() != 1:
-        raise RuntimeError("pos must be a one-element int32 GPU tensor")
+    if not pos.is_cuda or pos.dtype != torch.int32 or pos.numel() != 1 or pos.device != qkv.device:
+        raise RuntimeError("pos must be a one-element int32 tensor on qkv's GPU")
+    if cache_k.device != qkv.device or cache_v.device != qkv.device or freq_table.device != qkv.device:
+        raise RuntimeError("qkv, freq_table and the caches must be on the same device")
     if out is None:
         out = torch.empty((B, 1, n_head, HD), dtype=qkv.dtype, device=qkv.device)
+    elif not isinstance(out, torch.Tensor) or out.dtype != torch.bfloat16 or out.device != qkv.device \
+            or tuple(out.shape) != (B, 1, n_head, HD) or not out.is_contiguous():
+        raise RuntimeError(f"rot_embed_append: out must be a contiguous bf16 tensor of shape {(B, 1, n_head, HD)} "
+                           f"on {qkv.device}")
     with _on_device(qkv.device):
         rc = lib.l3_rot_embed_append(qkv.data_ptr(), freq_table.data_ptr(), out.data_ptr(), cache_k.data_ptr(),
                                      cache_v.data_ptr(), pos.data_ptr(), B, n_head, KVH, HD, qkv.stride(0),
@@ -471,25 +521,20 @@ def _rows_out(x, rows: int, N: int):
 
 
 def _use_splitk(x, weight) -> bool:
-    """17..64 activation rows against a matrix too small for one workgroup per 128 rows to fill the
-    device: the split-K kernel plus its finishing pass is the faster route (measured at 17, 32 and 64
-    rows, K 2048..8192: up to 16384 matrix rows on 256 compute units; from 32768 on the single launch wins)."""
+    """17..64 activation rows: the split-K kernel plus its finishing pass (one launch serves up to 16)."""
     K = x.shape[-1]
     if K <= 0 or weight.dim() != 2 or not x.is_cuda:
         return False
-    rows = x.numel() // K
-    N = weight.shape[0]
-    if N % 8:          # the finishing pass writes eight columns per lane; the single launch needs only N % 4 == 0
-        return False
-    return rows > _l3lib.L3_LINEAR_FUSED_MAX_ROWS and -(-N // 128) < _cus(x.device)
+    return _l3lib.L3_LINEAR_MAX_ROWS < x.numel() // K <= _l3lib.L3_LINEAR_SPLITK_MAX_ROWS
 
 
 def linear_decode(x, weight):
     """F.linear(x, weight) for at most 64 activation rows (model.py:95,121,134,225 when T == 1):
     one pass over the weight matrix at HBM speed instead of a GEMM.  x (..., K), weight (N, K)
-    -> (..., N).  Up to 16 rows are one launch whatever the matrix; with 17..64 rows (K % 128 == 0
-    then) a matrix whose rows alone fill the device is still one launch, and the matrices of a few
-    thousand rows go through linear_splitk and linear_splitk_finish (N % 8 == 0).  An extension."""
+    -> (..., N).  Up to 16 rows are one launch whatever the matrix; 17..64 rows go through
+    linear_splitk and linear_splitk_finish (N % 8 == 0, K % 128 == 0), which suits matrices of a
+    few thousand rows -- a vocabulary projection at those batch sizes is a library GEMM's job.
+    An extension."""
     lib = _l3lib.load()
     if _use_splitk(x, weight):
         return linear_splitk_finish(linear_splitk(x, weight)).view(*x.shape[:-1], weight.shape[0])
@@ -504,7 +549,7 @@ def linear_decode(x, weight):
 
 
 def linear_swiglu_decode(x, w_gate, w_up):
-    """F.silu(F.linear(x, w_gate)) * F.linear(x, w_up) for at most 64 activation rows in one
+    """F.silu(F.linear(x, w_gate)) * F.linear(x, w_up) for at most 16 activation rows in one
     launch (model.py:134 with w_gate = c_fc2, w_up = c_fc), same rounding points.  An extension."""
     lib = _l3lib.load()
     x2, rows, N, K = _linear_args(x, (w_gate, w_up))

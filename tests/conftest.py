@@ -34,24 +34,18 @@ def gpu():
 
 @pytest.fixture(params=["mfma", "fma"])
 def attn_kernel(request):
-    """Run an attention test once per split-KV kernel (MFMA tiles / FMA dot products)."""
-    from custom_kernels import _l3lib as l3
+    """Run an attention test once per split-KV kernel (MFMA tiles / FMA dot products): the shim's
+    context-local default flags carry the choice into every call of the test."""
+    from custom_kernels import custom_kernels_extension as cke
 
-    lib = l3.load()
-    prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL,
-                                  l3.L3_ATTN_KERNEL_FMA if request.param == "fma" else l3.L3_ATTN_KERNEL_MFMA)
-    yield request.param
-    lib.l3_attn_set_option(l3.L3_ATTN_OPT_KERNEL, prev)
+    with cke.attention_flags(kernel=request.param):
+        yield request.param
 
 
 @pytest.fixture(params=["auto", "wave", "tiled", "pipelined"])
 def prefill_form(request):
     """Run a prefill test once per form of the kernel (the library's own choice, and each forced)."""
-    from custom_kernels import _l3lib as l3
+    from custom_kernels import custom_kernels_extension as cke
 
-    lib = l3.load()
-    value = {"auto": l3.L3_ATTN_PREFILL_AUTO, "wave": l3.L3_ATTN_PREFILL_WAVE, "tiled": l3.L3_ATTN_PREFILL_TILED,
-             "pipelined": l3.L3_ATTN_PREFILL_PIPELINED}
-    prev = lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, value[request.param])
-    yield request.param
-    lib.l3_attn_set_option(l3.L3_ATTN_OPT_PREFILL, prev)
+    with cke.attention_flags(prefill=request.param):
+        yield request.param

@@ -7,6 +7,15 @@ from oracle import bf16_bits_to_f32, bf16_ulp_distance, f32_to_bf16_bits, round_
 
 ATTN_ATOL = 2e-2     # north-star tolerance for attention in bf16
 ATTN_RTOL = 1.6e-2
+# Regression bound, far inside the contract, for N(0,1) inputs: what float32 accumulation, one final
+# bf16 rounding (half an ulp <= 2^-8 relative) and bf16 probabilities in the second product can cost.
+# The last term is 2^-9 * sum_j p_j |v_j|: about 1.6e-3 once a row averages over many tokens (measured
+# maximum over the long shapes: 1.2e-3), up to 2^-9 * max|v| when a couple of tokens carry the row.
+# A kernel that loses a rescale or a term on some path at small magnitude stays inside the contract
+# tolerance; it does not stay inside this.
+ATTN_REG_ATOL = 2e-3
+ATTN_REG_RTOL = 2.0 ** -7
+ATTN_REG_FEW_TOKENS = 2.0 ** -9 * 6.0   # added when a row may attend to fewer than 64 tokens
 
 
 def t2bits(t: torch.Tensor) -> np.ndarray:
@@ -49,7 +58,9 @@ def to_device_like(t: torch.Tensor, device) -> torch.Tensor:
     return moved.as_strided(t.shape, t.stride(), t.storage_offset())
 
 
-def assert_attn_close(out_bits_or_tensor, ref_f64, what=""):
+def assert_attn_close(out_bits_or_tensor, ref_f64, what="", min_kv_len=None, regression=True):
+    """The contract tolerance, and inside it the regression bound; `min_kv_len` is the smallest
+    number of tokens an output row attends to (None = unknown or few)."""
     out = t2f32(out_bits_or_tensor).astype(np.float64) if isinstance(out_bits_or_tensor, torch.Tensor) \
         else bf16_bits_to_f32(out_bits_or_tensor).astype(np.float64)
     ref = np.asarray(ref_f64, dtype=np.float64)
@@ -57,6 +68,12 @@ def assert_attn_close(out_bits_or_tensor, ref_f64, what=""):
     tol = ATTN_ATOL + ATTN_RTOL * np.abs(ref)
     bad = err > tol
     assert not bad.any(), f"{what}: {bad.sum()} of {bad.size} outside atol {ATTN_ATOL}/rtol {ATTN_RTOL}; max err {err.max():.4g}"
+    if regression:
+        atol = ATTN_REG_ATOL + (0.0 if (min_kv_len is not None and min_kv_len >= 64) else ATTN_REG_FEW_TOKENS)
+        worse = err > atol + ATTN_REG_RTOL * np.abs(ref)
+        assert not worse.any(), (f"{what}: inside the contract tolerance but {worse.sum()} of {worse.size} elements are "
+                                 f"outside the regression bound atol {atol:.3g}/rtol {ATTN_REG_RTOL:.3g}; "
+                                 f"max err {err.max():.4g}")
     return float(err.max())
 
 

@@ -39,9 +39,11 @@ C_CALLER = r"""
 int main(void) {
     /* host-logic entry points only: nothing here touches a GPU */
     if (l3_version() < 100) return 1;
-    if (l3_attn_choose_splits(1, 8, 32768, 128, 256) < 2) return 2;
-    if (l3_attn_choose_splits(1, 8, 32768, 96, 256) != L3_ERR_HEAD_SIZE) return 3;
-    if (l3_attn_decode_workspace_bytes(1, 32, 8, 32768, 128, 4) != (size_t)(4 * 32 * 128 * 4 + 4 * 32 * 8)) return 4;
+    if (l3_attn_choose_splits(1, 8, 32768, 128, 256, 0) < 2) return 2;
+    if (l3_attn_choose_splits(1, 8, 32768, 96, 256, 0) != L3_ERR_HEAD_SIZE) return 3;
+    if (l3_attn_decode_workspace_bytes(1, 32, 8, 32768, 128, 4, L3_ATTN_FLAG_KERNEL_FMA) !=
+        (size_t)(4 * 32 * 128 * 4 + 4 * 32 * 8)) return 4;
+    if (l3_attn_choose_splits(1, 8, 32768, 128, 256, 0x4000) != L3_ERR_FLAGS) return 6;
     if (l3_rms_norm(0, 0, 0, 1, 2048, 1e-5f, 0) != L3_ERR_NULL_POINTER) return 5;
     printf("%s\n", l3_strerror(L3_ERR_HEAD_RATIO));
     return 0;
@@ -70,14 +72,17 @@ def test_error_codes_match_header():
         assert getattr(_l3lib, name) == int(val)
         assert _l3lib.strerror(int(val))
     assert int(re.search(r"#define L3_ATTN_MAX_SPLITS (\d+)", text).group(1)) == _l3lib.L3_ATTN_MAX_SPLITS
+    assert int(re.search(r"#define L3_LINEAR_MAX_ROWS (\d+)", text).group(1)) == _l3lib.L3_LINEAR_MAX_ROWS
+    for name, val in re.findall(r"#define (L3_ATTN_FLAG_[A-Z_]+) (0x[0-9a-fA-F]+)", text):
+        assert getattr(_l3lib, name) == int(val, 16)
     assert "unknown" in _l3lib.strerror(-12345)
 
 
 def _attn(q=FAKE, k=FAKE, v=FAKE, out=FAKE, ws=None, ws_bytes=0, B=1, QH=32, KVH=8, S=256, HD=64,
-          qs=(2048, 64), ks=(131072, 64, 512), vs=(131072, 64, 512), os_=(2048, 64), splits=1):
+          qs=(2048, 64), ks=(131072, 64, 512), vs=(131072, 64, 512), os_=(2048, 64), splits=1, flags=0):
     return _l3lib.load().l3_attn_decode(q, k, v, out, ws, ws_bytes, B, QH, KVH, S, HD, _l3lib.i64_array(qs),
                                         _l3lib.i64_array(ks), _l3lib.i64_array(vs), _l3lib.i64_array(os_),
-                                        0.125, splits, None)
+                                        0.125, splits, flags, None)
 
 
 def test_attention_argument_checks_run_before_any_launch():
@@ -95,10 +100,12 @@ def test_attention_argument_checks_run_before_any_launch():
     assert _attn(vs=(131072, 60, 512)) == _l3lib.L3_ERR_STRIDE
     assert _attn(qs=(2048, -64)) == _l3lib.L3_ERR_STRIDE
     assert _attn(k=FAKE + 2) == _l3lib.L3_ERR_ALIGNMENT
+    assert _attn(flags=0x100) == _l3lib.L3_ERR_FLAGS
+    assert _attn(flags=-1) == _l3lib.L3_ERR_FLAGS
     assert _attn(S=1024, ks=(524288, 64, 512), vs=(524288, 64, 512), splits=4) == _l3lib.L3_ERR_WORKSPACE
     assert _attn(S=1024, ks=(524288, 64, 512), vs=(524288, 64, 512), splits=4, ws=FAKE, ws_bytes=16) \
         == _l3lib.L3_ERR_WORKSPACE
-    need = _l3lib.load().l3_attn_decode_workspace_bytes(1, 32, 8, 1024, 64, 4)
+    need = _l3lib.load().l3_attn_decode_workspace_bytes(1, 32, 8, 1024, 64, 4, 0)
     assert _attn(S=1024, ks=(524288, 64, 512), vs=(524288, 64, 512), splits=4, ws=FAKE + 64, ws_bytes=need) \
         == _l3lib.L3_ERR_ALIGNMENT
 
@@ -123,23 +130,23 @@ def test_split_planning():
     for HD, tile in ((64, 64), (128, 32)):
         prev = 0
         for S in (1, 63, 64, 65, 256, 512, 1000, 4096, 32768, 131072):
-            n = lib.l3_attn_choose_splits(1, 8, S, HD, 256)
+            n = lib.l3_attn_choose_splits(1, 8, S, HD, 256, 0)
             assert 1 <= n <= _l3lib.L3_ATTN_MAX_SPLITS
             assert n <= max(1, -(-S // tile)), "no split shorter than one workgroup tile"
             assert n >= prev, "more tokens never means fewer splits at fixed batch"
             prev = n
-            ws = lib.l3_attn_decode_workspace_bytes(1, 32, 8, S, HD, 0)
+            ws = lib.l3_attn_decode_workspace_bytes(1, 32, 8, S, HD, 0, 0)
             if n == 1:
                 assert ws == 0
             else:
                 rows = 32 * n
                 assert rows * (HD + 2) * 4 <= ws <= rows * (HD + 2) * 4 + 512
         # enough (batch, kv head) pairs to fill the device: no split, no combine
-        assert lib.l3_attn_choose_splits(256, 8, 256, HD, 256) == 1
+        assert lib.l3_attn_choose_splits(256, 8, 256, HD, 256, 0) == 1
         # the device size matters
-        assert lib.l3_attn_choose_splits(1, 8, 32768, HD, 64) < lib.l3_attn_choose_splits(1, 8, 32768, HD, 256)
+        assert lib.l3_attn_choose_splits(1, 8, 32768, HD, 64, 0) < lib.l3_attn_choose_splits(1, 8, 32768, HD, 256, 0)
     # many sequences (8 kv heads: one workgroup per sequence and split group, 256 units):
-    plan = lambda B, S, HD: lib.l3_attn_choose_splits(B, 8, S, HD, 256)  # noqa: E731
+    plan = lambda B, S, HD: lib.l3_attn_choose_splits(B, 8, S, HD, 256, 0)  # noqa: E731
     assert plan(3, 32768, 128) == 79            # at most 85 (3 * 85 = 255 workgroups for 256 units), whole tiles: 79 x 416 tokens
     assert plan(4, 4096, 64) == 64              # few sequences: one workgroup per unit
     assert plan(16, 4096, 64) == 11             # from 8 sequences on, three quarters of the units: 12 groups, whole tiles
@@ -149,11 +156,17 @@ def test_split_planning():
     assert plan(96, 512, 64) == 1               # short streams at a quarter of the units or more: no combine
     assert plan(128, 128, 64) == 1 and plan(192, 1024, 128) == 1
     assert plan(100, 4096, 128) == 2            # a long stream is worth the second group
-    assert lib.l3_attn_choose_splits(1, 8, 256, 96, 256) == _l3lib.L3_ERR_HEAD_SIZE
-    assert lib.l3_attn_choose_splits(0, 8, 256, 64, 256) == _l3lib.L3_ERR_SHAPE
-    assert cke.attention_num_splits(16, 8, 4096, 64) == lib.l3_attn_choose_splits(16, 8, 4096, 64, 256)
+    assert lib.l3_attn_choose_splits(1, 8, 256, 96, 256, 0) == _l3lib.L3_ERR_HEAD_SIZE
+    assert lib.l3_attn_choose_splits(0, 8, 256, 64, 256, 0) == _l3lib.L3_ERR_SHAPE
+    assert cke.attention_num_splits(16, 8, 4096, 64) == lib.l3_attn_choose_splits(16, 8, 4096, 64, 256, 0)
     # an explicit request is honoured up to what the length allows
-    assert lib.l3_attn_decode_workspace_bytes(1, 32, 8, 4096, 128, 7) == 32 * 7 * 128 * 4 + 32 * 7 * 8
+    assert lib.l3_attn_decode_workspace_bytes(1, 32, 8, 4096, 128, 7, 0) == 32 * 7 * 128 * 4 + 32 * 7 * 8
+    # the plan belongs to the call: the FMA kernel's differs, and the shim's context carries the flag per thread
+    fma = _l3lib.L3_ATTN_FLAG_KERNEL_FMA
+    assert lib.l3_attn_choose_splits(16, 8, 4096, 64, 256, fma) != lib.l3_attn_choose_splits(16, 8, 4096, 64, 256, 0)
+    with cke.attention_flags(kernel="fma"):
+        assert cke.attention_num_splits(16, 8, 4096, 64) == lib.l3_attn_choose_splits(16, 8, 4096, 64, 256, fma)
+    assert cke.attention_num_splits(16, 8, 4096, 64) == 11
 
 
 def test_shim_rejects_cpu_tensors_and_has_no_fallback():
@@ -180,12 +193,14 @@ def test_missing_library_raises(monkeypatch, tmp_path):
 def test_stage_entry_points_argument_checks():
     lib = _l3lib.load()
     qs, ks = _l3lib.i64_array((2048, 64)), _l3lib.i64_array((131072, 64, 512))
-    assert lib.l3_attn_split(FAKE, FAKE, FAKE, None, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, None) \
+    assert lib.l3_attn_split(FAKE, FAKE, FAKE, None, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, 0, None) \
         == _l3lib.L3_ERR_NULL_POINTER
-    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 32, 8, 256, 80, qs, ks, ks, 0.125, 1, None) \
+    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 32, 8, 256, 80, qs, ks, ks, 0.125, 1, 0, None) \
         == _l3lib.L3_ERR_HEAD_SIZE
-    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE + 4, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, None) \
+    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE + 4, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, 0, None) \
         == _l3lib.L3_ERR_ALIGNMENT
+    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, 2, None) \
+        == _l3lib.L3_ERR_FLAGS
     assert lib.l3_attn_combine(FAKE, FAKE, None, 1, 32, 64, 4, qs, None) == _l3lib.L3_ERR_NULL_POINTER
     assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 1, 32, 96, 4, qs, None) == _l3lib.L3_ERR_HEAD_SIZE
     assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 1, 32, 64, 0, qs, None) == _l3lib.L3_ERR_SPLITS
@@ -199,10 +214,11 @@ def test_prefill_argument_checks():
     lib = _l3lib.load()
     qs, ks = _l3lib.i64_array((131072, 64, 2048)), _l3lib.i64_array((131072, 64, 512))
 
-    def call(q=FAKE, out=FAKE, B=1, QH=32, KVH=8, T=16, S=64, HD=64, q_strides=qs, k_strides=ks):
+    def call(q=FAKE, out=FAKE, B=1, QH=32, KVH=8, T=16, S=64, HD=64, q_strides=qs, k_strides=ks, flags=0):
         return lib.l3_attn_prefill(q, FAKE, FAKE, out, B, QH, KVH, T, S, HD, q_strides, k_strides, k_strides,
-                                   q_strides, 0.125, None)
+                                   q_strides, 0.125, flags, None)
 
+    assert call(flags=0x40) == _l3lib.L3_ERR_FLAGS
     assert call(out=None) == _l3lib.L3_ERR_NULL_POINTER
     assert call(HD=96) == _l3lib.L3_ERR_HEAD_SIZE
     assert call(QH=40) == _l3lib.L3_ERR_HEAD_RATIO      # ratio 5
@@ -224,7 +240,7 @@ def test_linear_decode_argument_checks():
     assert call(M=0) == _l3lib.L3_ERR_SHAPE
     assert call(M=_l3lib.L3_LINEAR_MAX_ROWS + 1) == _l3lib.L3_ERR_SHAPE
     assert call(K=2040, xs=2040, ws=2040) == _l3lib.L3_ERR_SHAPE       # K not a multiple of 32
-    assert call(M=17, K=2080, xs=2080, ws=2080) == _l3lib.L3_ERR_SHAPE # more than 16 rows: K must be a multiple of 128
+    assert call(M=17) == _l3lib.L3_ERR_SHAPE                           # more than one 16-column block of rows
     assert call(N=2046, ys=2048) == _l3lib.L3_ERR_SHAPE                # N not a multiple of 4
     assert call(xs=1024) == _l3lib.L3_ERR_STRIDE                       # rows would overlap
     assert call(ws=2052) == _l3lib.L3_ERR_STRIDE                       # weight rows not 16-byte aligned
@@ -306,7 +322,7 @@ def test_linear_splitk_plan_and_argument_checks():
     assert call(N=16384, ks=2) == _l3lib.L3_ERR_SPLITS # 128-row groups stage at most 512 k
     assert call(ks=17) == _l3lib.L3_ERR_SPLITS
     assert call(nbytes=1024) == _l3lib.L3_ERR_WORKSPACE
-    assert _l3lib.L3_LINEAR_MAX_ROWS == 64 and _l3lib.L3_LINEAR_SPLITK_MAX_ROWS == 64
+    assert _l3lib.L3_LINEAR_MAX_ROWS == 16 and _l3lib.L3_LINEAR_SPLITK_MAX_ROWS == 64
 
     def finish(part=FAKE, ks=4, res=None, y=FAKE, M=64, N=2048, stride=2048):
         return lib.l3_linear_splitk_finish(part, ks, res, y, M, N, stride, None)
@@ -325,3 +341,11 @@ def test_linear_splitk_plan_and_argument_checks():
         == _l3lib.L3_ERR_NULL_POINTER
     assert lib.l3_rot_embed_append_partials(FAKE, 4, FAKE, FAKE, FAKE, FAKE, FAKE, 64, 32, 8, 60, cs, 256, 512, None) \
         == _l3lib.L3_ERR_SHAPE
+
+
+def test_read_stream_argument_checks():
+    lib = _l3lib.load()
+    assert lib.l3_hbm_read_stream(None, 1 << 20, FAKE, 0, None) == _l3lib.L3_ERR_NULL_POINTER
+    assert lib.l3_hbm_read_stream(FAKE, 0, FAKE, 0, None) == _l3lib.L3_ERR_SHAPE
+    assert lib.l3_hbm_read_stream(FAKE, 1000, FAKE, 0, None) == _l3lib.L3_ERR_SHAPE
+    assert lib.l3_hbm_read_stream(FAKE + 8, 1 << 20, FAKE, 0, None) == _l3lib.L3_ERR_ALIGNMENT

@@ -43,7 +43,7 @@ def test_decode_attention_on_the_last_batch_rows_of_a_large_cache(gpu, big_cache
     assert (MAXB - 1) * ck.stride(0) > 2 ** 31 > 31 * ck.stride(0)
     ref = attention_decode_ref(t2f32(q.transpose(1, 2)[rows]), t2f32(k.transpose(1, 2)[rows]),
                                t2f32(v.transpose(1, 2)[rows]))
-    assert_attn_close(out[rows], ref, what="large cache decode")
+    assert_attn_close(out[rows], ref, what="large cache decode", min_kv_len=S)
 
 
 def test_prefill_attention_on_the_last_batch_row_of_a_large_cache(gpu, big_cache):

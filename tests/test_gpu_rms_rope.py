@@ -294,6 +294,25 @@ def test_argmax_first_maximum(gpu, rows, V):
                                   torch.argmax(wide[:, :V].float(), dim=-1).cpu().numpy())
 
 
+def test_argmax_treats_nan_as_the_maximum_like_torch(gpu):
+    """A NaN logit wins (the first one), as in torch.argmax: a numerical blow-up picks the same
+    token on the graph-replayed and the eager path."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    V = 5000
+    x = randn_bf16((6, V), 93)
+    x[0, 4000] = float("nan")                       # one NaN beats every number ...
+    x[1, 4100] = float("nan"); x[1, 17] = float("nan"); x[1, 2500] = float("inf")   # ... the first of several wins, inf included
+    x[2, :] = float("nan")                          # a row of NaNs: index 0
+    x[3, 7] = float("inf"); x[3, 9] = float("inf")  # no NaN: first maximum
+    x[4, :] = float("-inf")                         # all equal: index 0
+    x[5, V - 1] = float("nan")                      # in the last chunk
+    out = cke.argmax(x.to(gpu)).cpu()
+    want = torch.argmax(x.float(), dim=-1)
+    np.testing.assert_array_equal(out.numpy(), want.numpy())
+    np.testing.assert_array_equal(out.numpy(), np.array([4000, 17, 0, 7, 0, V - 1]))
+
+
 @pytest.mark.parametrize("rows,V,L,pos0", [(1, 128256, 256, 127), (64, 128256, 256, 200), (5, 1000, 20, 7), (3, 50, 9, 8)])
 def test_greedy_step_matches_generate_bookkeeping(gpu, rows, V, L, pos0):
     """argmax + the per-token bookkeeping of generate() (model.py:371-378) in place on the device,
