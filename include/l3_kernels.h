@@ -38,7 +38,8 @@ enum {
     L3_ERR_WORKSPACE = -7,      /* workspace NULL or smaller than l3_attn_decode_workspace_bytes */
     L3_ERR_SPLITS = -8,         /* num_splits negative or above L3_ATTN_MAX_SPLITS */
     L3_ERR_HIP = -9,            /* the HIP runtime reported an error at launch */
-    L3_ERR_FLAGS = -10          /* bits set in `flags` that this version does not define */
+    L3_ERR_FLAGS = -10,         /* bits set in `flags` that this version does not define */
+    L3_ERR_SCRATCH = -11        /* l3_attn_decode_static: the problem needs more than L3_ATTN_STATIC_SCRATCH_BYTES */
 };
 
 #define L3_ATTN_MAX_SPLITS 512
@@ -113,6 +114,29 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out,
                    const int64_t q_strides[2], const int64_t k_strides[3],
                    const int64_t v_strides[3], const int64_t out_strides[2],
                    float scale, int num_splits, int flags, void* stream);
+
+/*
+ * l3_attn_decode for callers that cannot allocate device memory and have no workspace to pass
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the
+ * float32 partials live in a static device array of L3_ATTN_STATIC_SCRATCH_BYTES inside the
+ * library instead of a caller's workspace, and the call allocates and frees nothing.  It has no
+ * counterpart in the reference, whose launcher allocates three temporaries per call
+ * (custom_kernels.cu:269-271).  Same arguments, kernels and results (bit for bit) as
+ * l3_attn_decode.  A problem whose plan needs more scratch than the array holds returns
+ * L3_ERR_SCRATCH (size it with l3_attn_decode_workspace_bytes; every BASELINE shape needs under
+ * 5 MiB).  Every GPU the library runs on holds its own copy of the array from the first call on
+ * that GPU until the process ends; the address is looked up once per device on that first call,
+ * so make one call outside stream capture first.  All calls on one GPU share the array: calls
+ * that overlap in time on the same GPU (different streams or threads) race.  Nothing in the
+ * array has to start at zero -- every row a combine reads was written by the same call's split
+ * kernel -- so the previous call's contents are simply overwritten.
+ */
+#define L3_ATTN_STATIC_SCRATCH_BYTES (16u << 20)
+int l3_attn_decode_static(const void* q, const void* k, const void* v, void* out,
+                          int B, int QH, int KVH, int S, int HD,
+                          const int64_t q_strides[2], const int64_t k_strides[3],
+                          const int64_t v_strides[3], const int64_t out_strides[2],
+                          float scale, int num_splits, int flags, void* stream);
 
 /*
  * l3_attn_decode with the KV length read from device memory at run time (*kv_len_dev, clamped to

@@ -44,6 +44,38 @@ size_t attn_workspace_bytes(int B, int QH, int HD, int num_splits) {
 
 }  // namespace
 
+// Scratch of l3_attn_decode_static: the float32 partials and their (max, sum) pairs live in this
+// array instead of a caller's workspace.  Every device the library runs on holds its own copy at
+// its own address for the life of the process; in host code the NAME is only a handle for
+// hipGetSymbolAddress, never an address to hand to a kernel.
+static __device__ __align__(256) unsigned char g_attn_static_scratch[L3_ATTN_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of the current device's copy of the array, looked up once per device (null on failure).
+void* static_scratch_ptr() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr) return ptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ptr = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (ptr) return ptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_attn_static_scratch)) != hipSuccess || !ptr) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    return ptr;
+}
+}  // namespace
+
 int current_device_cus() {
     static std::once_flag once;
     static int cus = 256;
@@ -145,6 +177,7 @@ const char* l3_strerror(int code) {
         case L3_ERR_SPLITS: return "num_splits out of range";
         case L3_ERR_HIP: return "HIP runtime error at kernel launch";
         case L3_ERR_FLAGS: return "unknown bits in flags";
+        case L3_ERR_SCRATCH: return "problem needs more scratch than the static device buffer holds";
         default: return "unknown error code";
     }
 }
@@ -226,7 +259,7 @@ int attn_decode_impl(const void* q, const void* k, const void* v, void* out, voi
                      size_t workspace_bytes, int B, int QH, int KVH, int S, int HD,
                      const int64_t q_strides[2], const int64_t k_strides[3], const int64_t v_strides[3],
                      const int64_t out_strides[2], float scale, int num_splits, int flags, const int* seqlen_dev,
-                     void* stream) {
+                     void* stream, bool static_scratch = false) {
     if (int rc = check_attn_args(q, k, v, out, B, QH, KVH, S, HD, q_strides, k_strides, v_strides, out_strides,
                                  num_splits, true); rc != L3_OK)
         return rc;
@@ -235,7 +268,14 @@ int attn_decode_impl(const void* q, const void* k, const void* v, void* out, voi
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
     const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
     const size_t need = attn_workspace_bytes(B, QH, HD, plan.num_splits);
-    if (need > 0) {
+    if (static_scratch) {
+        // the partials go to this device's copy of the static array; nothing is allocated
+        if (need > L3_ATTN_STATIC_SCRATCH_BYTES) return L3_ERR_SCRATCH;
+        if (need > 0) {
+            workspace = static_scratch_ptr();
+            if (!workspace) return L3_ERR_HIP;
+        }
+    } else if (need > 0) {
         if (!workspace || workspace_bytes < need) return L3_ERR_WORKSPACE;
         if (!aligned(workspace, kWorkspaceAlign)) return L3_ERR_ALIGNMENT;
     }
@@ -261,6 +301,14 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out, void*
                    const int64_t out_strides[2], float scale, int num_splits, int flags, void* stream) {
     return attn_decode_impl(q, k, v, out, workspace, workspace_bytes, B, QH, KVH, S, HD, q_strides, k_strides,
                             v_strides, out_strides, scale, num_splits, flags, nullptr, stream);
+}
+
+int l3_attn_decode_static(const void* q, const void* k, const void* v, void* out, int B, int QH, int KVH, int S,
+                          int HD, const int64_t q_strides[2], const int64_t k_strides[3],
+                          const int64_t v_strides[3], const int64_t out_strides[2], float scale, int num_splits,
+                          int flags, void* stream) {
+    return attn_decode_impl(q, k, v, out, nullptr, 0, B, QH, KVH, S, HD, q_strides, k_strides, v_strides,
+                            out_strides, scale, num_splits, flags, nullptr, stream, true);
 }
 
 int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out, void* workspace,

@@ -20,7 +20,9 @@ L3_ERR_WORKSPACE = -7
 L3_ERR_SPLITS = -8
 L3_ERR_HIP = -9
 L3_ERR_FLAGS = -10
+L3_ERR_SCRATCH = -11
 L3_ATTN_MAX_SPLITS = 512
+L3_ATTN_STATIC_SCRATCH_BYTES = 16 << 20
 L3_LINEAR_MAX_ROWS = 16         # one launch, any matrix shape, optional input norm / SwiGLU / residual / rope epilogue
 L3_LINEAR_SPLITK_MAX_ROWS = 64
 L3_LINEAR_STAGE_ELEMS = 24576   # activations (rows padded by 8) the fused input norm can stage in LDS
@@ -41,6 +43,13 @@ SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v out
          ctypes.c_void_p, ctypes.c_size_t,                                    # workspace, bytes
+         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,  # B QH KVH S HD
+         _c_i64p, _c_i64p, _c_i64p, _c_i64p,                                  # strides
+         ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],        # scale splits flags stream
+    ),
+    "l3_attn_decode_static": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v out
          ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,  # B QH KVH S HD
          _c_i64p, _c_i64p, _c_i64p, _c_i64p,                                  # strides
          ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],        # scale splits flags stream

@@ -21,6 +21,7 @@ import torch
 from . import _l3lib
 
 __all__ = ["flash_attention_decode", "rms_norm", "rot_embed", "attention_num_splits", "attention_flags",
+           "flash_attention_decode_static",
            "flash_attention_split", "flash_attention_combine", "flash_attention_decode_devlen",
            "rot_embed_append", "add_rms_norm", "silu_mul", "argmax", "flash_attention_prefill"]
 
@@ -170,6 +171,29 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0, flags=None)
             _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
             _l3lib.i64_array((out.stride(0), out.stride(1))),
             1.0 / math.sqrt(HD), num_splits, flags, stream_ptr)
+    if rc != 0:
+        _fail(rc, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
+    return out
+
+
+def flash_attention_decode_static(query, keys, values, out, num_splits: int = 0, flags=None):
+    """flash_attention_decode into the caller's ``out`` with the partials in the library's static
+    device scratch: the call allocates nothing (l3_attn_decode_static).  Raises when the problem
+    needs more scratch than the static array holds.  Calls that overlap on one GPU race."""
+    lib = _l3lib.load()
+    flags = _flags(flags)
+    B, QH, KVH, S, HD = _check_qkv(query, keys, values)
+    if keys.device != query.device or values.device != query.device:
+        raise RuntimeError("query, keys and values must be on the same device")
+    _check_out(out, query, "flash_attention_decode_static")
+    with _on_device(query.device):
+        rc = lib.l3_attn_decode_static(
+            query.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr(), B, QH, KVH, S, HD,
+            _l3lib.i64_array((query.stride(0), query.stride(1))),
+            _l3lib.i64_array((keys.stride(0), keys.stride(1), keys.stride(2))),
+            _l3lib.i64_array((values.stride(0), values.stride(1), values.stride(2))),
+            _l3lib.i64_array((out.stride(0), out.stride(1))),
+            1.0 / math.sqrt(HD), num_splits, flags, _stream_ptr(query.device))
     if rc != 0:
         _fail(rc, f"B={B} QH={QH} KVH={KVH} S={S} HD={HD}")
     return out

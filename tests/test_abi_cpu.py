@@ -75,6 +75,8 @@ def test_error_codes_match_header():
     assert int(re.search(r"#define L3_LINEAR_MAX_ROWS (\d+)", text).group(1)) == _l3lib.L3_LINEAR_MAX_ROWS
     for name, val in re.findall(r"#define (L3_ATTN_FLAG_[A-Z_]+) (0x[0-9a-fA-F]+)", text):
         assert getattr(_l3lib, name) == int(val, 16)
+    assert int(re.search(r"#define L3_ATTN_STATIC_SCRATCH_BYTES \((\d+)u << (\d+)\)", text).group(1)) << 20 \
+        == _l3lib.L3_ATTN_STATIC_SCRATCH_BYTES
     assert "unknown" in _l3lib.strerror(-12345)
 
 

@@ -305,6 +305,8 @@ def test_caller_supplied_outputs_are_validated(gpu):
     for bad in bad_outs:
         with pytest.raises(RuntimeError):
             cke.flash_attention_decode_devlen(qg, kg, vg, kv_len, out=bad)
+        with pytest.raises(RuntimeError):
+            cke.flash_attention_decode_static(qg, kg, vg, bad)
     with pytest.raises(RuntimeError):
         cke.flash_attention_decode_devlen(qg, kg, vg, kv_len.cpu())
     qkv = randn_bf16((2, 1, 48 * 64), 45).to(gpu)
