@@ -4,18 +4,22 @@
 Default workload (the headline configuration): decode attention at head_dim 128, batch 1,
 32 query / 8 KV heads, bf16, KV length swept over every power of two from 512 to 32768.
 One step = one pass over the seven lengths (split-KV kernel + combine each).  Inputs are
-resident in HBM before the timed region; each length owns several copies of its K/V and a
-pass uses the next copy, so that >1 GB of other traffic separates two reads of the same
-bytes and the 256 MB Infinity Cache cannot serve them.  The passes are captured in a HIP
-graph (launch-bound otherwise) and replayed; the clock is wall time around the replays with
-a device synchronisation on both sides.
+resident in HBM before the timed region.  Every launch reads K/V from its own region of a 2 GiB
+pool, and a region is read again only after at least 512 MB of other regions have been read,
+so the 256 MB Infinity Cache cannot serve any of it: every figure is HBM-cold.  The
+launches are captured in a HIP graph (launch-bound otherwise) and replayed -- at least 30 ms
+untimed, then at least 50 ms timed, whatever --steps says; the clock is wall time around the
+replays with a device synchronisation on both sides.
 
-Prints ONE JSON line: value = algorithmic GB/s (K+V+Q read, O written) over the timed
-steps; "roofline" prices the same bytes against the 8 TB/s HBM peak from HIP-event timing;
-"cpu_baseline" is stock PyTorch on the host cores for a bounded sample of the same sweep.
+Prints ONE JSON line: value = algorithmic GB/s (K+V+Q read, O written) over the timed steps;
+"roofline" prices the split-KV kernel alone against the 8 TB/s HBM peak from HIP-event timing and
+carries the read bandwidth a pure stream reaches on the same device; "cpu_baseline" is stock
+PyTorch on the host cores for a bounded sample of the same sweep.  The same line carries the rest
+of the target ("north_star": head_dim 64, the batched shapes, RMSNorm, rotary embedding, each
+cold, torch's own attention beside the decode kernel) and the end-to-end tokens/s ("e2e").
 
-Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|prefill|linear|e2e|copy) report the remaining configurations
-in the same format.
+Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|prefill|linear|e2e|copy|readstream) report the
+remaining configurations in the same format.
 """
 
 import argparse
@@ -35,22 +39,32 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 SEED = 42               # the reference's default seed (benchmark_kernel.py:126)
 FORCE_SPLITS = 0        # --splits
 ATTN_FLAGS = 0          # --attn-kernel fma sets L3_ATTN_FLAG_KERNEL_FMA
+COLD_BYTES = 512 << 20  # distinct input bytes between two reads of the same region (Infinity Cache: 256 MB)
+MIN_WARM_S = 0.03       # untimed replays: after an idle spell the first milliseconds run at lower clocks
+MIN_TIMED_S = 0.05
 
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file (summaries and the copy-kernel calibration are in profiles/); keyed by (workload, kernel).
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this file (the summaries, their commands and the copy-kernel calibration are under profiles/).
+# An entry is reported only while the split plan it was measured with is the plan of this run.
 MEASURED_TRAFFIC = {
-    # profiles/attn_splitkv_mfma_c2_sweep_hbm_traffic.md: 38.21 MB fetched + 2.47 MB written per launch
-    ("c2", "attn_splitkv_mfma_kernel"): 40680000,
-    # profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md (largest shape of each workload)
-    ("c3a", "attn_splitkv_mfma_kernel"): 136660000,   # 135.37 MB fetched + 1.29 MB written
-    ("c3b", "attn_splitkv_mfma_kernel"): 135890000,   # 134.39 MB fetched + 1.50 MB written (partials of 11 splits)
-    ("rms", "rms_norm_stream_kernel"): 67270000,      # 4096 x 4096: 33.72 MB fetched + 33.55 MB written
-    ("rope", "rot_embed_rows_kernel"): 68670000,      # 4096 x 32 x 128: 35.12 MB fetched + 33.55 MB written
+    "c2": {"bytes": 40680000, "plan": [1, 32, 64, 128, 256, 256, 256],
+           "profile": "profiles/attn_splitkv_mfma_c2_sweep_hbm_traffic.md"},
+    "c3a": {"bytes": 136660000, "plan": [1], "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
+    "c3b": {"bytes": 135890000, "plan": [11], "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
+    "rms": {"bytes": 67270000, "plan": None, "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
+    "rope": {"bytes": 68670000, "plan": None, "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
 }
 
 
-def attn_kernel_name(lib=None):
+def measured_traffic(name, plan=None):
+    rec = MEASURED_TRAFFIC.get(name)
+    if rec is None or ATTN_FLAGS or FORCE_SPLITS or (rec["plan"] is not None and rec["plan"] != plan):
+        return None, None
+    return rec["bytes"], rec["profile"]
+
+
+def attn_kernel_name():
     from custom_kernels import _l3lib as l3
     return "fma" if ATTN_FLAGS & l3.L3_ATTN_FLAG_KERNEL_FMA else "mfma"
 
@@ -60,44 +74,62 @@ def attn_bytes(B, QH, KVH, S, HD):
     return 2 * B * KVH * S * HD * 2 + 2 * B * QH * HD * 2
 
 
-class AttnCase:
-    """One attention shape with `slots` independent copies of its inputs, pre-allocated outputs
-    and workspace, launched straight through the C ABI (no per-call allocation)."""
+class KVPool:
+    """2 GiB of N(0,1) bf16 (1 GiB for K, 1 GiB for V) that every attention shape carves its
+    rotating input copies from.  `regions` hands out disjoint (B, L, KVH, HD) caches; a launch that
+    walks over them reads each byte once per walk."""
 
-    def __init__(self, torch, lib, l3, dev, B, QH, KVH, S, HD, slots, src_k=None, src_v=None, src_q=None,
-                 cache_len=0):
+    def __init__(self, torch, dev, elems=1 << 29):
+        self.torch = torch
+        self.k = torch.empty(elems, dtype=torch.bfloat16, device=dev).normal_()
+        self.v = torch.empty(elems, dtype=torch.bfloat16, device=dev).normal_()
+        self.next = 0
+
+    def reset(self):
+        self.next = 0
+
+    def region(self, B, L, KVH, HD):
+        per = B * L * KVH * HD
+        if self.next + per > self.k.numel():
+            raise RuntimeError("KV pool exhausted")
+        k = self.k[self.next:self.next + per].view(B, L, KVH, HD)
+        v = self.v[self.next:self.next + per].view(B, L, KVH, HD)
+        self.next += per
+        return k, v
+
+    def capacity(self, B, L, KVH, HD):
+        return (self.k.numel() - self.next) // (B * L * KVH * HD)
+
+
+class AttnCase:
+    """One attention shape with `slots` disjoint copies of its K/V (token-major storage, transposed
+    views: the model's cache layout, benchmark_kernel.py:165-173), a pre-allocated output and
+    workspace, launched straight through the C ABI (no per-call allocation)."""
+
+    def __init__(self, torch, lib, l3, dev, pool, B, QH, KVH, S, HD, slots, cache_len=0):
         self.torch, self.lib = torch, lib
         self.B, self.QH, self.KVH, self.S, self.HD = B, QH, KVH, S, HD
         self.bytes = attn_bytes(B, QH, KVH, S, HD)
-        self.slots = slots
+        L = max(S, cache_len)
+        self.slots = max(1, min(slots, pool.capacity(B, L, KVH, HD)))
         g = torch.Generator().manual_seed(SEED)
-        q = src_q if src_q is not None else torch.randn((B, 1, QH, HD), generator=g).to(torch.bfloat16)
-        k = src_k if src_k is not None else torch.randn((B, S, KVH, HD), generator=g).to(torch.bfloat16)
-        v = src_v if src_v is not None else torch.randn((B, S, KVH, HD), generator=g).to(torch.bfloat16)
-        self.cpu = (q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
-        # token-major storage, transposed views: the model's cache layout (benchmark_kernel.py:165-173)
-        self.q = [q.to(dev).transpose(1, 2) for _ in range(slots)]
-        if cache_len > S:
+        self.q = torch.randn((B, 1, QH, HD), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+        self.k, self.v = [], []
+        for _ in range(self.slots):
+            kc, vc = pool.region(B, L, KVH, HD)
             # the model's layout (model.py:107-111): a (B, L, KVH, HD) cache of which the first S tokens are attended
-            def cache_view(t):
-                full = torch.zeros((B, cache_len, KVH, HD), dtype=torch.bfloat16, device=dev)
-                full[:, :S] = t.to(dev)
-                return full[:, :S].transpose(1, 2)
-            self.k = [cache_view(k) for _ in range(slots)]
-            self.v = [cache_view(v) for _ in range(slots)]
-        else:
-            self.k = [k.to(dev).transpose(1, 2) for _ in range(slots)]
-            self.v = [v.to(dev).transpose(1, 2) for _ in range(slots)]
-        self.out = [torch.empty_like(t) for t in self.q]
+            self.k.append(kc[:, :S].transpose(1, 2))
+            self.v.append(vc[:, :S].transpose(1, 2))
+        self.out = torch.empty_like(self.q)
         # 0 = the library plans for the current device (split count and kernel form)
         self.req_splits = FORCE_SPLITS
         self.num_splits = FORCE_SPLITS or lib.l3_attn_choose_splits(B, KVH, S, HD, 0, ATTN_FLAGS)
         self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.req_splits, ATTN_FLAGS)
         self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
         self.part_o = self.part_ml = None
+        qt, ot = self.q, self.out
         self._args = []
-        for i in range(slots):
-            qt, kt, vt, ot = self.q[i], self.k[i], self.v[i], self.out[i]
+        for kt, vt in zip(self.k, self.v):
             self._args.append((
                 qt.data_ptr(), kt.data_ptr(), vt.data_ptr(), ot.data_ptr(), self.ws.data_ptr(), self.ws_bytes,
                 B, QH, KVH, S, HD,
@@ -122,6 +154,11 @@ class AttnCase:
                                     self.req_splits, ATTN_FLAGS, stream_ptr)
         if rc < 0:
             raise RuntimeError(f"l3_attn_split failed: {rc}")
+
+
+def cold_slots(call_bytes, floor=4):
+    """Copies of a shape's inputs needed so that COLD_BYTES of other data pass between two reads of one copy."""
+    return max(floor, int(math.ceil(COLD_BYTES / call_bytes)) + 1)
 
 
 def capture_graph(torch, fn):
@@ -149,6 +186,29 @@ def event_time_ms(torch, run, reps):
     return start.elapsed_time(end) / reps
 
 
+def timed_replays(torch, graph, min_replays=1, wall=False):
+    """Replays `graph` untimed for MIN_WARM_S, then timed for at least MIN_TIMED_S (and at least
+    min_replays times).  Returns (milliseconds per replay, replays timed).  HIP events on the
+    stream the graph runs on, or -- wall=True -- the host clock with a device synchronisation on
+    both sides."""
+    t0 = time.perf_counter()
+    n_warm = 0
+    while time.perf_counter() - t0 < MIN_WARM_S or n_warm < 2:
+        graph.replay()
+        torch.cuda.synchronize()
+        n_warm += 1
+    est = event_time_ms(torch, graph.replay, 2)
+    reps = max(min_replays, int(math.ceil(MIN_TIMED_S * 1e3 / max(est, 1e-4))))
+    if not wall:
+        return event_time_ms(torch, graph.replay, reps), reps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / reps, reps
+
+
 def time_cpu(fn, min_seconds, min_reps=3, max_reps=100000):
     fn()
     t0 = time.perf_counter()
@@ -161,45 +221,109 @@ def time_cpu(fn, min_seconds, min_reps=3, max_reps=100000):
             return el / n, n
 
 
+def torch_sdpa_us(torch, case, max_calls=24):
+    """torch's own scaled_dot_product_attention (enable_gqa) on the same cold tensors on the same GPU,
+    eager calls timed with events: what the reference's benchmark plots beside its kernel
+    (benchmark_kernel.py:23-28, 110-115).  A reported baseline only."""
+    import torch.nn.functional as F
+
+    try:
+        n = min(case.slots, max_calls)
+        for i in range(min(2, n)):
+            F.scaled_dot_product_attention(case.q, case.k[-1 - i], case.v[-1 - i], enable_gqa=True)
+        idx = [0]
+
+        def one():
+            i = idx[0] % n
+            idx[0] += 1
+            F.scaled_dot_product_attention(case.q, case.k[i], case.v[i], enable_gqa=True)
+        return round(event_time_ms(torch, one, n) * 1e3, 2)
+    except Exception as exc:  # informational only
+        print(f"bench.py: torch SDPA failed for B{case.B} S{case.S} HD{case.HD}: {exc}", file=sys.stderr)
+        return None
+
+
+def measure_attention_shape(torch, lib, l3, dev, pool, B, QH, KVH, S, HD, cache_len=0, with_sdpa=True,
+                            split_stage=False):
+    """One shape alone, HBM-cold: a graph that walks over the shape's copies, replayed."""
+    pool.reset()
+    c = AttnCase(torch, lib, l3, dev, pool, B, QH, KVH, S, HD, cold_slots(attn_bytes(B, QH, KVH, S, HD)), cache_len)
+    launch = c.launch_split_stage if split_stage else c.launch
+    launch(0, torch.cuda.current_stream().cuda_stream)
+    gph = capture_graph(torch, lambda: [launch(s, torch.cuda.current_stream().cuda_stream) for s in range(c.slots)])
+    ms, reps = timed_replays(torch, gph)
+    ms /= c.slots
+    del gph
+    gbps = c.bytes / (ms * 1e-3) / 1e9
+    rec = {"B": B, "HD": HD, "kv_len": S, "splits": c.num_splits, "us": round(ms * 1e3, 3), "GBps": round(gbps, 1),
+           "frac": round(gbps / HBM_PEAK_GBPS, 4), "bytes": c.bytes, "copies": c.slots,
+           "cold": bool(c.bytes * (c.slots - 1) >= COLD_BYTES), "launches_timed": reps * c.slots}
+    if not split_stage and c.num_splits > 1:
+        # the split-KV kernel of the same calls alone: the difference is what the combine launch costs
+        c.launch_split_stage(0, torch.cuda.current_stream().cuda_stream)
+        sg = capture_graph(torch, lambda: [c.launch_split_stage(s, torch.cuda.current_stream().cuda_stream)
+                                           for s in range(c.slots)])
+        rec["split_kernel_us"] = round(timed_replays(torch, sg)[0] / c.slots * 1e3, 3)
+        del sg
+    if with_sdpa:
+        rec["torch_sdpa_us"] = torch_sdpa_us(torch, c)
+    return rec
+
+
+def measure_read_stream(torch, lib, dev, pool, chunk_bytes=128 << 20):
+    """The read bandwidth a pure stream reaches: the library's read-only kernel over the K pool in
+    chunks of chunk_bytes, each chunk cold, graph-replayed like everything else."""
+    src = pool.k
+    total = src.numel() * 2
+    n = max(1, total // chunk_bytes)
+    sink = torch.zeros(16, dtype=torch.int32, device=dev)
+
+    def walk():
+        sp = torch.cuda.current_stream().cuda_stream
+        for i in range(n):
+            rc = lib.l3_hbm_read_stream(src.data_ptr() + i * chunk_bytes, chunk_bytes, sink.data_ptr(), 0, sp)
+            if rc != 0:
+                raise RuntimeError(f"l3_hbm_read_stream failed: {rc}")
+    walk()
+    gph = capture_graph(torch, walk)
+    ms, reps = timed_replays(torch, gph)
+    ms /= n
+    gbps = chunk_bytes / (ms * 1e-3) / 1e9
+    return {"bytes_per_launch": chunk_bytes, "us": round(ms * 1e3, 3), "GBps": round(gbps, 1),
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "launches_timed": reps * n,
+            "kernel": "hbm_read_stream_kernel (16-byte non-temporal loads, no stores, no arithmetic)"}
+
+
+ATTN_WORKLOADS = {
+    # name: (B, HD, KV lengths, label)
+    "c2": (1, 128, [512, 1024, 2048, 4096, 8192, 16384, 32768],
+           "decode attention sweep: B1 QH32 KVH8 HD128 bf16, KV length 512..32768 (x2), split+combine"),
+    "c1": (1, 64, [256], "decode attention: B1 QH32 KVH8 HD64 bf16, KV length 256, split+combine"),
+    "c3a": (256, 64, [256], "batched decode attention: B256 QH32 KVH8 HD64 bf16, KV length 256"),
+    "c3b": (16, 64, [4096], "batched decode attention: B16 QH32 KVH8 HD64 bf16, KV length 4096, split+combine"),
+    "hd64": (1, 64, [512, 1024, 2048, 4096, 8192, 16384, 32768],
+             "decode attention sweep: B1 QH32 KVH8 HD64 bf16, KV length 512..32768 (x2), split+combine"),
+}
+
+
 # ------------------------------------------------------------------------------ workloads
-def run_attention(args, torch, lib, l3, dev, name):
+def run_attention(args, torch, lib, l3, dev, name, pool):
     from oracle.cpu_baseline import attention_cpu
 
     QH, KVH = 32, 8
-    if name == "c2":
-        B, HD, lengths = 1, 128, [512, 1024, 2048, 4096, 8192, 16384, 32768]
-        label = "decode attention sweep: B1 QH32 KVH8 HD128 bf16, KV length 512..32768 (x2), split+combine"
-    elif name == "c1":
-        B, HD, lengths = 1, 64, [256]
-        label = "decode attention: B1 QH32 KVH8 HD64 bf16, KV length 256, split+combine"
-    elif name == "c3a":
-        B, HD, lengths = 256, 64, [256]
-        label = "batched decode attention: B256 QH32 KVH8 HD64 bf16, KV length 256"
-    elif name == "c3b":
-        B, HD, lengths = 16, 64, [4096]
-        label = "batched decode attention: B16 QH32 KVH8 HD64 bf16, KV length 4096, split+combine"
-    elif name == "hd64":
-        B, HD, lengths = 1, 64, [512, 1024, 2048, 4096, 8192, 16384, 32768]
-        label = "decode attention sweep: B1 QH32 KVH8 HD64 bf16, KV length 512..32768 (x2), split+combine"
-    else:
-        raise ValueError(name)
-
+    B, HD, lengths, label = ATTN_WORKLOADS[name]
     if args.lengths:
         lengths = [int(x) for x in args.lengths.split(",")]
         label += f" [lengths overridden: {lengths}]"
-    smax = max(lengths)
-    g = torch.Generator().manual_seed(SEED)
-    q = torch.randn((B, 1, QH, HD), generator=g).to(torch.bfloat16)
-    k = torch.randn((B, smax, KVH, HD), generator=g).to(torch.bfloat16)
-    v = torch.randn((B, smax, KVH, HD), generator=g).to(torch.bfloat16)
-    pass_bytes = sum(attn_bytes(B, QH, KVH, S, HD) for S in lengths)
-    # enough copies that a pass over all of them moves > 1 GiB between two uses of the same bytes
-    slots = max(4, int(math.ceil((1 << 30) / pass_bytes)))
-    slots = min(slots, 64)
     if args.cache_len:
         label += f" [K/V are views of (B, {args.cache_len}, KVH, HD) caches]"
-    cases = [AttnCase(torch, lib, l3, dev, B, QH, KVH, S, HD, slots, src_k=k[:, :S].contiguous(),
-                      src_v=v[:, :S].contiguous(), src_q=q, cache_len=args.cache_len) for S in lengths]
+    pass_bytes = sum(attn_bytes(B, QH, KVH, S, HD) for S in lengths)
+    # a pass reads every length once, each from its own region; enough passes per graph that
+    # COLD_BYTES of other regions separate two reads of one region
+    passes = cold_slots(pass_bytes)
+    pool.reset()
+    cases = [AttnCase(torch, lib, l3, dev, pool, B, QH, KVH, S, HD, passes, args.cache_len) for S in lengths]
+    passes = min(c.slots for c in cases)
 
     def one_pass(slot):
         sp = torch.cuda.current_stream().cuda_stream
@@ -225,59 +349,53 @@ def run_attention(args, torch, lib, l3, dev, name):
             "roofline": None, "cpu_baseline": None, "per_length": detail,
         }
 
-    passes_per_graph = slots
-    graph = capture_graph(torch, lambda: [one_pass(s) for s in range(passes_per_graph)])
-
-    steps = max(passes_per_graph, (args.steps + passes_per_graph - 1) // passes_per_graph * passes_per_graph)
-    warm = max(1, (args.warmup + passes_per_graph - 1) // passes_per_graph)
-    for _ in range(warm):
+    one_pass(0)
+    graph = capture_graph(torch, lambda: [one_pass(s) for s in range(passes)])
+    # the headline: wall clock around the replays, device synchronised on both sides; at least
+    # args.steps passes and at least MIN_TIMED_S, after at least MIN_WARM_S (and args.warmup passes) untimed
+    for _ in range((args.warmup + passes - 1) // passes):
         graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps // passes_per_graph):
-        graph.replay()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / steps
+    ms_graph, reps = timed_replays(torch, graph, min_replays=(args.steps + passes - 1) // passes, wall=True)
+    steps = reps * passes
+    ms_per_step = ms_graph / passes
     value = pass_bytes / (ms_per_step * 1e-3) / 1e9
-
     # HIP-event timing of the same replays (events on the stream the kernels run on)
-    ev_ms = event_time_ms(torch, graph.replay, max(1, steps // passes_per_graph)) / passes_per_graph
+    ev_ms = event_time_ms(torch, graph.replay, reps) / passes
     op_gbps = pass_bytes / (ev_ms * 1e-3) / 1e9
+    del graph
 
-    # The dominant kernel on its own: the split-KV stage of every length, same rotation, graph-replayed.
+    # The dominant kernel on its own: the split-KV stage of every length, same regions, graph-replayed.
     def split_pass(slot):
         sp = torch.cuda.current_stream().cuda_stream
         for c in cases:
             c.launch_split_stage(slot, sp)
 
     split_pass(0)
-    sgraph = capture_graph(torch, lambda: [split_pass(s) for s in range(passes_per_graph)])
-    sgraph.replay()
-    split_ms = event_time_ms(torch, sgraph.replay, max(1, steps // passes_per_graph)) / passes_per_graph
+    sgraph = capture_graph(torch, lambda: [split_pass(s) for s in range(passes)])
+    sms, sreps = timed_replays(torch, sgraph)
+    split_ms = sms / passes
     achieved = pass_bytes / (split_ms * 1e-3) / 1e9
-    split_kernel = "attn_splitkv_mfma_kernel" if attn_kernel_name(lib) == "mfma" else "attn_splitkv_fma_kernel"
+    split_kernel = "attn_splitkv_mfma_kernel" if attn_kernel_name() == "mfma" else "attn_splitkv_fma_kernel"
     del sgraph
+    plan = [c.num_splits for c in cases]
+    traffic, traffic_src = measured_traffic(name, plan)
+    del cases
 
-    # per-length detail: each length alone, rotating over its copies, graph-replayed
-    detail = []
-    for c in cases:
-        reps_in_graph = max(slots, 16)
-        gph = capture_graph(torch, lambda c=c: [c.launch(s, torch.cuda.current_stream().cuda_stream)
-                                                for s in range(reps_in_graph)])
-        gph.replay()
-        ms = event_time_ms(torch, gph.replay, 5) / reps_in_graph
-        gbps = c.bytes / (ms * 1e-3) / 1e9
-        detail.append({"kv_len": c.S, "splits": c.num_splits, "us": round(ms * 1e3, 3), "GBps": round(gbps, 1),
-                       "frac": round(gbps / HBM_PEAK_GBPS, 4), "bytes": c.bytes,
-                       "cold": bool(c.bytes * slots > (300 << 20))})
-        del gph
+    # per-length detail: each length alone over its own cold copies, with torch's attention beside it
+    detail = [measure_attention_shape(torch, lib, l3, dev, pool, B, QH, KVH, S, HD, args.cache_len,
+                                      with_sdpa=not args.no_sdpa) for S in lengths]
 
     cpu = None
     if not args.no_cpu_baseline and name in ("c2", "c1"):
+        g = torch.Generator().manual_seed(SEED)
+        smax = max(lengths)
+        q = torch.randn((B, 1, QH, HD), generator=g).to(torch.bfloat16).transpose(1, 2)
+        k = torch.randn((B, smax, KVH, HD), generator=g).to(torch.bfloat16)
+        v = torch.randn((B, smax, KVH, HD), generator=g).to(torch.bfloat16)
+
         def cpu_pass():
-            for c in cases:
-                attention_cpu(*c.cpu)
+            for S in lengths:
+                attention_cpu(q, k[:, :S].transpose(1, 2), v[:, :S].transpose(1, 2))
         sec, n = time_cpu(cpu_pass, args.cpu_seconds)
         cpu = {"value": round(pass_bytes / sec / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
                "kind": "port", "host_cpus": os.cpu_count(),
@@ -287,95 +405,122 @@ def run_attention(args, torch, lib, l3, dev, name):
     return {
         "metric": "decode_attn_hbm_GBps", "value": round(value, 1), "unit": "GB/s",
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-        "steps": steps, "ms_per_step": round(ms_per_step, 5), "dtype": "bf16",
-        "config": {"workload": label, "kv_copies_per_length": slots, "accumulate": "f32", "launch": "hip graph",
-                   "seed": SEED},
+        "steps": steps, "steps_requested": args.steps, "ms_per_step": round(ms_per_step, 5), "dtype": "bf16",
+        "config": {"workload": label, "kv_regions_per_length": passes, "cold_bytes_between_reuse": COLD_BYTES,
+                   "accumulate": "f32", "launch": "hip graph", "seed": SEED,
+                   "timed_region_s": round(ms_graph * reps / 1e3, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((name, split_kernel)),
-                     "kernel": split_kernel, "launches_per_pass": len(cases),
-                     "avg_launch_us": round(split_ms * 1e3 / len(cases), 3),
-                     "algorithmic_bytes_per_launch": pass_bytes // len(cases),
+                     "traffic": traffic, "traffic_profile": traffic_src,
+                     "kernel": split_kernel, "launches_per_pass": len(lengths), "split_plan": plan,
+                     "avg_launch_us": round(split_ms * 1e3 / len(lengths), 3), "launches_timed": sreps * passes * len(lengths),
+                     "algorithmic_bytes_per_launch": pass_bytes // len(lengths),
                      "split_plus_combine_GBps": round(op_gbps, 1),
                      "split_plus_combine_frac": round(op_gbps / HBM_PEAK_GBPS, 4)},
         "cpu_baseline": cpu, "per_length": detail,
     }
 
 
+def north_star_extras(args, torch, lib, l3, dev, pool):
+    """The rest of the target beside the headline sweep, every entry HBM-cold: head_dim 64 at batch 1,
+    the batched shapes (split + combine together), RMSNorm and rotary embedding at 4096 rows."""
+    QH, KVH = 32, 8
+    sdpa = not args.no_sdpa
+    out = {"hd64_b1": [measure_attention_shape(torch, lib, l3, dev, pool, 1, QH, KVH, S, 64, with_sdpa=sdpa)
+                       for S in (4096, 8192, 16384, 32768)],
+           "c1_b1_hd64_s256": measure_attention_shape(torch, lib, l3, dev, pool, 1, QH, KVH, 256, 64, with_sdpa=sdpa),
+           "c3a_b256_hd64_s256": measure_attention_shape(torch, lib, l3, dev, pool, 256, QH, KVH, 256, 64, with_sdpa=sdpa),
+           "c3b_b16_hd64_s4096": measure_attention_shape(torch, lib, l3, dev, pool, 16, QH, KVH, 4096, 64, with_sdpa=sdpa)}
+    out["rms_norm"] = [rows_record(torch, lib, l3, dev, "rms", 2, 2048, C) for C in (2048, 4096)]
+    out["rot_embed"] = [rows_record(torch, lib, l3, dev, "rope", 2, 2048, HD) for HD in (64, 128)]
+    return out
+
+
+def rows_record(torch, lib, l3, dev, name, B, T, width):
+    """One RMSNorm (width = C) or rotary-embedding (width = HD, 32 heads of a strided qkv view) shape,
+    cold: enough copies of input and output that COLD_BYTES pass between two uses of one copy."""
+    from custom_kernels import precompute_freqs_cis
+
+    g = torch.Generator().manual_seed(SEED)
+    sp = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+    if name == "rms":
+        C = width
+        nbytes = 2 * B * T * C * 2 + C * 2
+        copies = cold_slots(nbytes, floor=2)
+        x0 = torch.randn((B, T, C), generator=g).to(torch.bfloat16).to(dev)
+        xs = [x0] + [torch.empty_like(x0).normal_() for _ in range(copies - 1)]
+        w = (torch.randn((C,), generator=g) * 0.02 + 1).to(torch.bfloat16).to(dev)
+        ys = [torch.empty_like(x) for x in xs]
+        run = lambda: [lib.l3_rms_norm(x.data_ptr(), w.data_ptr(), y.data_ptr(), B * T, C, 1e-5, sp())  # noqa: E731
+                       for x, y in zip(xs, ys)]
+        rec = {"rows": B * T, "C": C}
+        keep = (x0, w)
+    else:
+        HD, NH = width, 32
+        nbytes = 2 * B * T * NH * HD * 2 + T * HD * 4
+        copies = cold_slots(nbytes, floor=2)
+        tab = precompute_freqs_cis(HD, 4096, 500000.0, True, scale_factor=32.0, device=dev)
+        buf0 = torch.randn((B, T, (NH + 16) * HD), generator=g).to(torch.bfloat16).to(dev)
+        bufs = [buf0] + [torch.empty_like(buf0).normal_() for _ in range(copies - 1)]
+        xs = [b[..., : NH * HD].view(B, T, NH, HD) for b in bufs]
+        ys = [torch.empty((B, T, NH, HD), dtype=torch.bfloat16, device=dev) for _ in xs]
+        fr = tab[:T].contiguous()
+        st = l3.i64_array((xs[0].stride(0), xs[0].stride(1), xs[0].stride(2)))
+        run = lambda: [lib.l3_rot_embed(x.data_ptr(), fr.data_ptr(), y.data_ptr(), B, T, NH, HD, st, sp())  # noqa: E731
+                       for x, y in zip(xs, ys)]
+        rec = {"tokens": B * T, "NH": NH, "HD": HD}
+        keep = (xs[0], fr)
+    run()
+    gph = capture_graph(torch, run)
+    ms, reps = timed_replays(torch, gph)
+    ms /= copies
+    del gph
+    rec.update({"us": round(ms * 1e3, 3), "GBps": round(nbytes / ms / 1e6, 1),
+                "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nbytes, "copies": copies,
+                "cold": bool(nbytes * (copies - 1) >= COLD_BYTES), "launches_timed": reps * copies})
+    rec["_keep"] = keep
+    rec["_ms"] = ms
+    return rec
+
+
+def public(rec):
+    return {k: v for k, v in rec.items() if not k.startswith("_")}
+
+
 def run_rows(args, torch, lib, l3, dev, name):
     """RMSNorm / rotary embedding at the largest configured shape (4096 rows / tokens), plus the small ones."""
-    from custom_kernels import custom_kernels_extension as cke
-    from custom_kernels import precompute_freqs_cis
     from oracle.cpu_baseline import rms_norm_cpu, rot_embed_cpu
 
-    detail = []
-    head = None
+    detail, head = [], None
+    for width in ((2048, 4096) if name == "rms" else (64, 128)):
+        for (B, T) in ((1, 1), (1, 64), (1, 256), (2, 2048)):
+            rec = rows_record(torch, lib, l3, dev, name, B, T, width)
+            if B * T == 4096 and width == (4096 if name == "rms" else 128):
+                head = rec
+            detail.append(public(rec))
     if name == "rms":
-        for C in (2048, 4096):
-            for (B, T) in ((1, 1), (1, 64), (1, 256), (2, 2048)):
-                copies = max(2, min(64, (1 << 30) // max(1, 2 * B * T * C * 2)))
-                g = torch.Generator().manual_seed(SEED)
-                xs = [torch.randn((B, T, C), generator=g).to(torch.bfloat16).to(dev) for _ in range(min(copies, 4))]
-                xs = xs + [xs[0].clone() for _ in range(copies - len(xs))]
-                w = (torch.randn((C,), generator=g) * 0.02 + 1).to(torch.bfloat16).to(dev)
-                ys = [torch.empty_like(x) for x in xs]
-                sp = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
-                gph = capture_graph(torch, lambda: [lib.l3_rms_norm(x.data_ptr(), w.data_ptr(), y.data_ptr(), B * T, C,
-                                                                    1e-5, sp()) for x, y in zip(xs, ys)])
-                gph.replay()
-                ms = event_time_ms(torch, gph.replay, 10) / copies
-                nbytes = 2 * B * T * C * 2 + C * 2
-                rec = {"rows": B * T, "C": C, "us": round(ms * 1e3, 3), "GBps": round(nbytes / ms / 1e6, 1),
-                       "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nbytes}
-                detail.append(rec)
-                if C == 4096 and B * T == 4096:
-                    head = (rec, ms, nbytes, lambda x=xs[0].cpu(), w=w.cpu(): rms_norm_cpu(x, w, 1e-5))
         label = "fused RMSNorm: 4096 rows x C 4096 bf16 (2x2048-token prefill), eps 1e-5"
-        metric = "rms_norm_hbm_GBps"
+        metric, kernel = "rms_norm_hbm_GBps", "rms_norm_stream_kernel"
+        x, w = (t.cpu() for t in head["_keep"])
+        cpu_fn = lambda: rms_norm_cpu(x, w, 1e-5)  # noqa: E731
     else:
-        for HD in (64, 128):
-            tab = precompute_freqs_cis(HD, 4096, 500000.0, True, scale_factor=32.0, device=dev)
-            for (B, T) in ((1, 1), (1, 64), (1, 256), (2, 2048)):
-                NH = 32
-                copies = max(2, min(64, (1 << 30) // max(1, 2 * B * T * NH * HD * 2)))
-                g = torch.Generator().manual_seed(SEED)
-                buf0 = torch.randn((B, T, (NH + 16) * HD), generator=g).to(torch.bfloat16).to(dev)
-                bufs = [buf0] + [buf0.clone() for _ in range(copies - 1)]
-                xs = [b[..., : NH * HD].view(B, T, NH, HD) for b in bufs]
-                ys = [torch.empty((B, T, NH, HD), dtype=torch.bfloat16, device=dev) for _ in xs]
-                fr = tab[:T].contiguous()
-                st = l3.i64_array((xs[0].stride(0), xs[0].stride(1), xs[0].stride(2)))
-                sp = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
-                gph = capture_graph(torch, lambda: [lib.l3_rot_embed(x.data_ptr(), fr.data_ptr(), y.data_ptr(), B, T,
-                                                                     NH, HD, st, sp()) for x, y in zip(xs, ys)])
-                gph.replay()
-                ms = event_time_ms(torch, gph.replay, 10) / copies
-                nbytes = 2 * B * T * NH * HD * 2 + T * HD * 4
-                rec = {"tokens": B * T, "NH": NH, "HD": HD, "us": round(ms * 1e3, 3),
-                       "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
-                       "bytes": nbytes}
-                detail.append(rec)
-                if HD == 128 and B * T == 4096:
-                    head = (rec, ms, nbytes, lambda x=xs[0].cpu(), f=fr.cpu(): rot_embed_cpu(x, f))
         label = "fused rotary embedding: 4096 tokens x 32 heads x HD 128 bf16 from a strided qkv view"
-        metric = "rot_embed_hbm_GBps"
-
-    rec, ms, nbytes, cpu_fn = head
+        metric, kernel = "rot_embed_hbm_GBps", "rot_embed_rows_kernel"
+        x, f = (t.cpu() for t in head["_keep"])
+        cpu_fn = lambda: rot_embed_cpu(x, f)  # noqa: E731
     cpu = None
     if not args.no_cpu_baseline:
         sec, n = time_cpu(cpu_fn, min(args.cpu_seconds, 5.0))
-        cpu = {"value": round(nbytes / sec / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
+        cpu = {"value": round(head["bytes"] / sec / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
                "kind": "port", "host_cpus": os.cpu_count(), "sample": f"{n} runs of the same shape in torch on the CPU"}
+    traffic, traffic_src = measured_traffic(name)
     return {
-        "metric": metric, "value": rec["GBps"], "unit": "GB/s", "frac_of_hbm_peak": rec["frac"],
-        "steps": args.steps, "ms_per_step": round(ms, 5), "dtype": "bf16",
+        "metric": metric, "value": head["GBps"], "unit": "GB/s", "frac_of_hbm_peak": head["frac"],
+        "steps": head["launches_timed"], "ms_per_step": round(head["_ms"], 5), "dtype": "bf16",
         "config": {"workload": label, "accumulate": "f32", "launch": "hip graph", "seed": SEED},
-        "roofline": {"bound": "hbm", "achieved": rec["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": rec["frac"],
-                     "traffic": MEASURED_TRAFFIC.get((name, "rms_norm_stream_kernel" if name == "rms"
-                                                      else "rot_embed_rows_kernel")),
-                     "kernel": "rms_norm_stream_kernel" if name == "rms" else "rot_embed_rows_kernel",
-                     "algorithmic_bytes_per_launch": nbytes},
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": head["frac"], "traffic": traffic, "traffic_profile": traffic_src, "kernel": kernel,
+                     "algorithmic_bytes_per_launch": head["bytes"]},
         "cpu_baseline": cpu, "per_shape": detail,
     }
 
@@ -469,7 +614,17 @@ def run_linear(args, torch, lib, l3, dev):
             w0 = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(dev)
             ws = [w0] + [w0.clone() for _ in range(copies - 1)]
             ws2 = [w.clone() for w in ws] if swiglu else None
-            if swiglu:
+            if swiglu and M > 16:
+                # as the end-to-end harness does at these batch sizes: one library GEMM over the stacked
+                # gate|up matrix, then the library's SwiGLU product on its two halves
+                cats = [torch.cat([a, b], dim=0) for a, b in zip(ws, ws2)]
+
+                def run_l3():
+                    for c in cats:
+                        gu = F.linear(x, c)
+                        cke.silu_mul(gu[..., :N], gu[..., N:])
+                run_t = lambda: [F.silu(F.linear(x, a)) * F.linear(x, b) for a, b in zip(ws, ws2)]  # noqa: E731
+            elif swiglu:
                 run_l3 = lambda: [cke.linear_swiglu_decode(x, a, b) for a, b in zip(ws, ws2)]  # noqa: E731
                 run_t = lambda: [F.silu(F.linear(x, a)) * F.linear(x, b) for a, b in zip(ws, ws2)]  # noqa: E731
             else:
@@ -495,7 +650,8 @@ def run_linear(args, torch, lib, l3, dev):
                            "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
                            "bytes": nbytes, "torch_us": round(tms * 1e3, 2),
                            "path": "F.linear (library GEMM)" if library else
-                                   ("l3_linear_swiglu_decode" if swiglu else
+                                   ("F.linear on the stacked matrix + l3_silu_mul_rows" if swiglu and M > 16 else
+                                    "l3_linear_swiglu_decode" if swiglu else
                                     ("l3_linear_splitk + l3_linear_splitk_finish" if M > 16 else "l3_linear_decode"))})
             per_token = 1 if name == "lm_head" else 16
             total_us += ms * 1e3 * per_token
@@ -550,12 +706,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "prefill", "linear", "e2e", "copy"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3a", "c3b", "hd64", "rms", "rope", "prefill",
+                                                         "linear", "e2e", "copy", "readstream"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--single-shot", action="store_true",
                     help="attention workloads: one eager call per length (for profilers), no graph replay")
     ap.add_argument("--no-e2e", action="store_true",
                     help="default workload only: skip the end-to-end tokens/s summary that rides along")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="default workload only: skip the other shapes of the target (head_dim 64, batched, RMSNorm, rotary)")
+    ap.add_argument("--no-sdpa", action="store_true", help="skip torch's scaled_dot_product_attention beside the decode kernel")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="wall time spent on the CPU baseline sample")
     ap.add_argument("--e2e-batch", type=int, default=1)
     ap.add_argument("--attn-kernel", default="default", choices=["default", "mfma", "fma"],
@@ -566,7 +726,7 @@ def main():
                     help="attention workloads: K/V as views of caches this many tokens long (the model's batch stride)")
     args = ap.parse_args()
 
-    global FORCE_SPLITS
+    global FORCE_SPLITS, ATTN_FLAGS
     FORCE_SPLITS = args.splits
     if args.gpus != 1:
         print(f"bench.py: this path runs on one GPU with no sharding; --gpus {args.gpus} is not supported "
@@ -583,13 +743,24 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    global ATTN_FLAGS
     if args.attn_kernel == "fma":
         ATTN_FLAGS = l3.L3_ATTN_FLAG_KERNEL_FMA
-    attn_opts = {"split_kv_kernel": attn_kernel_name(lib)}
+    attn_opts = {"split_kv_kernel": attn_kernel_name()}
+    attention = args.workload in ATTN_WORKLOADS
+    default_line = args.workload == "c2" and not args.lengths and not args.single_shot and not args.cache_len
 
-    if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):
-        res = run_attention(args, torch, lib, l3, dev, args.workload)
+    def cpu_op_table():
+        from oracle import cpu_baseline
+
+        class cpu_ops:
+            rms_norm = staticmethod(cpu_baseline.rms_norm_cpu)
+            rot_embed = staticmethod(cpu_baseline.rot_embed_cpu)
+            flash_attention_decode = staticmethod(cpu_baseline.attention_cpu)
+        return cpu_ops
+
+    pool = KVPool(torch, dev) if attention or args.workload == "readstream" else None
+    if attention:
+        res = run_attention(args, torch, lib, l3, dev, args.workload, pool)
     elif args.workload in ("rms", "rope"):
         res = run_rows(args, torch, lib, l3, dev, args.workload)
     elif args.workload == "prefill":
@@ -598,33 +769,53 @@ def main():
         res = run_linear(args, torch, lib, l3, dev)
     elif args.workload == "copy":
         res = run_copy(args, torch, dev)
+    elif args.workload == "readstream":
+        rs = {str(mb): measure_read_stream(torch, lib, dev, pool, mb << 20) for mb in (16, 64, 128, 512)}
+        head = rs["128"]
+        res = {"metric": "read_stream_hbm_GBps", "value": head["GBps"], "unit": "GB/s", "frac_of_hbm_peak": head["frac"],
+               "steps": head["launches_timed"], "ms_per_step": round(head["us"] / 1e3, 5), "dtype": "u8",
+               "config": {"workload": "pure read stream over a 1 GiB pool in chunks of 128 MiB (16 / 64 / 512 MiB beside it), "
+                                      "each chunk cold", "launch": "hip graph"},
+               "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                            "frac": head["frac"], "traffic": None, "kernel": "hbm_read_stream_kernel",
+                            "algorithmic_bytes_per_launch": head["bytes_per_launch"]},
+               "cpu_baseline": None, "per_chunk_MiB": rs}
     else:
         import llama_arch
 
-        cpu_ops = None
-        if not args.no_cpu_baseline:
-            from oracle import cpu_baseline
-
-            class cpu_ops:
-                rms_norm = staticmethod(cpu_baseline.rms_norm_cpu)
-                rot_embed = staticmethod(cpu_baseline.rot_embed_cpu)
-                flash_attention_decode = staticmethod(cpu_baseline.attention_cpu)
-
-        res = llama_arch.bench_e2e(args, torch, dev, cpu_ops)
+        res = llama_arch.bench_e2e(args, torch, dev, None if args.no_cpu_baseline else cpu_op_table())
 
     line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
             "steps": res.pop("steps"), "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": res.pop("dtype"),
             "data": "synthetic", "config": res.pop("config")}
     line.update(res)
-    if args.workload in ("c1", "c2", "c3a", "c3b", "hd64"):
+    if attention:
         line["config"].update(attn_opts)
-    if args.workload == "c2" and not args.no_e2e and not args.lengths and not args.single_shot:
-        # the second half of the headline metric: greedy decode tokens/s of the 1B architecture
-        # (128 prompt ids + 128 generated tokens, graph-replayed loop; --workload e2e has the detail)
-        import llama_arch
+    if default_line:
+        # the read bandwidth a pure stream reaches here: the practical ceiling the fractions are read against
+        rs = measure_read_stream(torch, lib, dev, pool)
+        line["roofline"]["practical_read_peak"] = rs
+        if not args.no_extras:
+            ns = north_star_extras(args, torch, lib, l3, dev, pool)
+            ns["rms_norm"] = [public(r) for r in ns["rms_norm"]]
+            ns["rot_embed"] = [public(r) for r in ns["rot_embed"]]
+            ns["hd128_b1"] = [r for r in line["per_length"] if r["kv_len"] >= 4096]
+            target = 0.70
+            pts = ns["hd128_b1"] + ns["hd64_b1"] + [ns["c3a_b256_hd64_s256"], ns["c3b_b16_hd64_s4096"]]
+            ns["target_frac"] = target
+            ns["points_at_or_above_target"] = sum(r["frac"] >= target for r in pts)
+            ns["points"] = len(pts)
+            line["north_star"] = ns
+        del pool
+        torch.cuda.empty_cache()
+        if not args.no_e2e:
+            # the second half of the headline metric: greedy decode tokens/s of the 1B architecture
+            # (128 prompt ids + 128 generated tokens; --workload e2e has the detail)
+            import llama_arch
 
-        line["e2e_tokens_per_s"] = llama_arch.e2e_summary(torch, dev)
+            line["e2e"] = llama_arch.e2e_summary(torch, dev, cpu_ops=None if args.no_cpu_baseline else cpu_op_table())
+            line["e2e_tokens_per_s"] = {k: v["tok_per_s"] for k, v in line["e2e"].items() if k.startswith("bs")}
     line["device"] = torch.cuda.get_device_name(0)
     print(json.dumps(line), flush=True)
 

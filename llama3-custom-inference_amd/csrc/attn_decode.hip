@@ -85,8 +85,8 @@ attn_splitkv_fma_kernel(const AttnParams p) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int tok = min(tbase + u * G + g, t_end - 1);
-            kr[u] = load16(kbase + int64_t(tok) * p.k_st);
-            vr[u] = load16(vbase + int64_t(tok) * p.v_st);
+            kr[u] = load16_stream(kbase + int64_t(tok) * p.k_st);   // K/V are read once: a stream
+            vr[u] = load16_stream(vbase + int64_t(tok) * p.v_st);
         }
     };
 

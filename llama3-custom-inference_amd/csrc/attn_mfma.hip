@@ -92,7 +92,7 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     for (int nb = 0; nb < NB; ++nb) O[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = kMaskedScore;  // running maximum of the raw scores (common to the four k groups of a head)
     float l_part = 0.f;          // this lane's share of the softmax denominator
-    mfma_tile_loop<HD, LOADS>(kbase, vbase, p.k_st, p.v_st, s_slab[wave], qfrag, t_begin + (COOP ? wave * WT : 0),
+    mfma_tile_loop<HD, LOADS, true>(kbase, vbase, p.k_st, p.v_st, s_slab[wave], qfrag, t_begin + (COOP ? wave * WT : 0),
                               t_end, STEP, t_end, t_end, c, O, m_run, l_part);
 
     // ---- this wavefront's result.  O[nb][r] is dim 16*nb + 4*fg + r of head fn; the softmax

@@ -54,7 +54,9 @@ struct MfmaTile {
 // wave-uniform; tiles below it skip the masking).  On return O[nb][r] is dim 16*nb + 4*fg + r of
 // column fn (unnormalised), m_run the column's running maximum of the raw scores (shared by its
 // four k groups) and l_part this lane's share of the column's softmax denominator.
-template <int HD, int LOADS = 8>
+// STREAM: K/V are read once by the whole grid (decode), so they are loaded non-temporally; the
+// prefill form, whose column groups re-read the same tiles from cache, keeps plain loads.
+template <int HD, int LOADS = 8, bool STREAM = false>
 __device__ __forceinline__ void mfma_tile_loop(const uint16_t* kbase, const uint16_t* vbase, int64_t k_st,
                                                int64_t v_st, unsigned char* slab,
                                                const bf16x8_t (&qfrag)[MfmaTile<HD>::KC], int t_first, int t_end,
@@ -82,14 +84,14 @@ __device__ __forceinline__ void mfma_tile_loop(const uint16_t* kbase, const uint
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int tok = min(tbase + u * G + ld_row, t_end - 1);  // clamped rows are masked below
-            kr[u] = load16(kbase + int64_t(tok) * k_st);
+            kr[u] = STREAM ? load16_stream(kbase + int64_t(tok) * k_st) : load16(kbase + int64_t(tok) * k_st);
         }
     };
     auto issue_v = [&](int tbase) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int tok = min(tbase + u * G + ld_row, t_end - 1);
-            vr[u] = load16(vbase + int64_t(tok) * v_st);
+            vr[u] = STREAM ? load16_stream(vbase + int64_t(tok) * v_st) : load16(vbase + int64_t(tok) * v_st);
         }
     };
 

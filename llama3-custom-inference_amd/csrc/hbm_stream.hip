@@ -24,7 +24,7 @@ hbm_read_stream_kernel(const uint4* __restrict__ src, int64_t n16, uint32_t* __r
 #pragma unroll
         for (int u = 0; u < kStreamUnroll; ++u) {
             const int64_t i = base + u * kStreamThreads + threadIdx.x;
-            v[u] = (i < n16) ? src[i] : make_uint4(0u, 0u, 0u, 0u);
+            v[u] = (i < n16) ? load16_stream(reinterpret_cast<const uint16_t*>(src + i)) : make_uint4(0u, 0u, 0u, 0u);
         }
 #pragma unroll
         for (int u = 0; u < kStreamUnroll; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;

@@ -86,7 +86,7 @@ linear_splitk_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
 #pragma unroll
         for (int j = 0; j < NWC; ++j) {
 #pragma unroll
-            for (int s = 0; s < SPC; ++s) rw[j][s] = load16(wp + ((c0 + w0 + j) * SPC + s) * 32);
+            for (int s = 0; s < SPC; ++s) rw[j][s] = load16_stream(wp + ((c0 + w0 + j) * SPC + s) * 32);
         }
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {

@@ -108,8 +108,8 @@ rms_norm_stream_kernel(const uint16_t* __restrict__ x, const uint16_t* __restric
     for (int j = 0; j < MAXV; ++j) {
         const int vi = lane + j * kWaveSize;
         if (vi < nvec) {
-            cur[j] = load16(x + row * int64_t(C) + vi * 8);
-            if constexpr (ADD) rcur[j] = load16(res + row * int64_t(C) + vi * 8);
+            cur[j] = load16_stream(x + row * int64_t(C) + vi * 8);
+            if constexpr (ADD) rcur[j] = load16_stream(res + row * int64_t(C) + vi * 8);
             wv[j] = load16(w + vi * 8);
         }
     }
@@ -122,8 +122,8 @@ rms_norm_stream_kernel(const uint16_t* __restrict__ x, const uint16_t* __restric
             for (int j = 0; j < MAXV; ++j) {
                 const int vi = lane + j * kWaveSize;
                 if (vi < nvec) {
-                    nxt[j] = load16(x + nrow * int64_t(C) + vi * 8);
-                    if constexpr (ADD) rnxt[j] = load16(res + nrow * int64_t(C) + vi * 8);
+                    nxt[j] = load16_stream(x + nrow * int64_t(C) + vi * 8);
+                    if constexpr (ADD) rnxt[j] = load16_stream(res + nrow * int64_t(C) + vi * 8);
                 }
             }
         }

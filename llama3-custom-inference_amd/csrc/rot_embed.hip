@@ -70,7 +70,7 @@ rot_embed_rows_kernel(const uint16_t* __restrict__ x, const float* __restrict__ 
     const uint16_t* xp = x + b * sb + t * st + int64_t(hq * HG) * sh + c * 8;
     uint4 xv[HG];
 #pragma unroll
-    for (int i = 0; i < HG; ++i) xv[i] = load16(xp + i * sh);
+    for (int i = 0; i < HG; ++i) xv[i] = load16_stream(xp + i * sh);
     const float4 f0 = fp[0];
     const float4 f1 = fp[1];
     uint16_t* yp = y + ((b * T + t) * NH + hq * HG) * HD + c * 8;

@@ -62,15 +62,22 @@ class _Tokenizer:
 
 
 class LlamaDecoder:
-    def __init__(self, config: LlamaConfig, ops, device, dtype=torch.bfloat16, seed: int = 42):
+    def __init__(self, config: LlamaConfig, ops, device, dtype=torch.bfloat16, seed: int = 42, weights_from=None):
+        """`weights_from`: another LlamaDecoder of the same configuration whose weights are copied
+        (to this device) instead of being drawn again from the seed."""
         self.config, self.ops, self.device, self.dtype = config, ops, torch.device(device), dtype
         self.tokenizer = _Tokenizer()
         c = config
         hd = c.n_embd // c.n_head
         self.hd = hd
         g = torch.Generator().manual_seed(seed)
+        donor = iter(weights_from._weights()) if weights_from is not None else None
 
         def w(*shape):
+            if donor is not None:
+                t = next(donor)
+                assert tuple(t.shape) == tuple(shape)
+                return t.to(device=self.device, dtype=dtype)
             return (torch.randn(shape, generator=g, dtype=torch.float32) * 0.02).to(dtype).to(self.device)
 
         self.wte = w(c.vocab_size, c.n_embd)          # tied with the lm_head (model.py:190)
@@ -97,6 +104,13 @@ class LlamaDecoder:
         # nn.Linear calls with at most this many activation rows (the decode step) go through the
         # library's weight-streaming kernels when the operator module has them; 0 = always F.linear
         self.decode_linear_rows = 16 if hasattr(ops, "linear_decode") else 0
+
+    def _weights(self):
+        """The random-init matrices in the order __init__ draws them."""
+        yield self.wte
+        for L in self.layers:
+            for name in ("c_attn", "c_proj", "c_fc", "c_fc2", "mlp_proj"):
+                yield L[name]
 
     def set_decode_linear_rows(self, rows: int):
         self.decode_linear_rows = rows if hasattr(self.ops, "linear_decode") else 0
@@ -478,22 +492,48 @@ def timed_generate(model, batch, input_len, gen_len, seed=42, sync=None, graphed
     return gen_len * batch / dt, dt, out
 
 
-def e2e_summary(torch_mod, dev, batches=(1, 64), input_len=128, gen_len=128, repeats=2):
-    """Graph-replayed greedy decode of the end-to-end configuration, tokens/s per batch size (best of
-    `repeats` after one warm-up generation that also records the graph): the short form that rides
-    along with the default attention benchmark."""
+def e2e_summary(torch_mod, dev, batches=(1, 64), input_len=128, gen_len=128, repeats=2, cpu_ops=None):
+    """The end-to-end configuration in short form, for the default benchmark line: per batch size the
+    graph-replayed greedy decode (best of `repeats` after one warm-up generation that also records the
+    graph) in tokens/s and microseconds per generated token, the eager loop beside it, and how many of the
+    generated tokens the two loops agree on; with `cpu_ops` (an operator table working on CPU tensors) a
+    shortened batch-1 generation of the same model on the host cores."""
+    import os
+
     from custom_kernels import custom_kernels_extension as cke
 
+    sync = torch_mod.cuda.synchronize
+    cfg = LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=max(batches))
+    model = LlamaDecoder(cfg, cke, dev)
     out = {}
     for batch in batches:
-        cfg = LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=batch)
-        model = LlamaDecoder(cfg, cke, dev)
-        timed_generate(model, batch, input_len, gen_len, seed=1, graphed=True)
-        best = max(timed_generate(model, batch, input_len, gen_len, sync=torch_mod.cuda.synchronize, graphed=True)[0]
-                   for _ in range(repeats))
-        out[f"bs{batch}"] = round(best, 1)
-        del model
-        torch_mod.cuda.empty_cache()
+        timed_generate(model, batch, input_len, 2, seed=1)                       # eager warm-up
+        eager_tps, _, eager_toks = timed_generate(model, batch, input_len, gen_len, sync=sync)
+        timed_generate(model, batch, input_len, gen_len, seed=1, graphed=True)   # records the graph
+        best, toks = 0.0, None
+        for _ in range(repeats):
+            tps, _, t = timed_generate(model, batch, input_len, gen_len, sync=sync, graphed=True)
+            if tps > best:
+                best, toks = tps, t
+        same = sum(a == b for ra, rb in zip(eager_toks, toks) for a, b in zip(ra, rb))
+        out[f"bs{batch}"] = {"tok_per_s": round(best, 1), "us_per_generated_token_step": round(1e6 * batch / best, 1),
+                             "eager_tok_per_s": round(eager_tps, 1),
+                             "graphed_vs_eager_same_tokens": f"{same}/{batch * gen_len}",
+                             "weight_stream_frac_of_hbm_peak": round(2471628800 * best / batch / 8e12, 4)}
+    out["config"] = (f"Llama-3.2-1B architecture, random init, {input_len} prompt ids + {gen_len} greedy tokens, "
+                     "prefill included, decode loop replayed from a HIP graph")
+    if cpu_ops is not None:
+        cpu_model = LlamaDecoder(LlamaConfig(max_model_len=input_len + gen_len, max_gen_batch_size=1), cpu_ops, "cpu",
+                                 weights_from=model)
+        short = 8
+        tps, dt, _ = timed_generate(cpu_model, 1, input_len, short)
+        out["cpu_baseline"] = {"value": round(tps, 2), "unit": "tokens/s", "cores": torch_mod.get_num_threads(),
+                               "kind": "port", "host_cpus": os.cpu_count(),
+                               "sample": f"same model and prompts on the CPU with torch ops, batch 1, {input_len} prompt "
+                                         f"ids + {short} greedy tokens in {dt:.1f} s (shortened generation)"}
+        del cpu_model
+    del model
+    torch_mod.cuda.empty_cache()
     return out
 
 
