@@ -99,7 +99,8 @@ size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int
  *   q, out : (B, QH, 1, HD) bf16; q_strides / out_strides = {batch, head} strides
  *   k, v   : (B, KVH, S, HD) bf16; k_strides / v_strides = {batch, head, token} strides.
  *            Token rows must start on 16-byte boundaries (base pointers 16-byte aligned,
- *            strides multiples of 8).  q and out need 16-byte aligned rows as well.
+ *            strides multiples of 8, token stride below 2^24 elements).  q and out need
+ *            16-byte aligned rows as well.
  *   scale  : softmax scale; the reference uses 1/sqrt(HD) (custom_kernels.cu:253)
  *   num_splits : 0 = automatic, otherwise 1..L3_ATTN_MAX_SPLITS (the kernel may use fewer
  *            when S is short); results do not depend on it beyond float32 rounding

@@ -42,7 +42,7 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     __shared__ __align__(16) unsigned char s_slab[kMfmaWaves][SLAB];
 
     const int lane = threadIdx.x & (kWaveSize - 1);
-    const int wave = threadIdx.x / kWaveSize;
+    const int wave = wave_uniform(int(threadIdx.x) / kWaveSize);   // scalar: everything derived from it is wave-uniform
     const int fn = lane & 15;        // role in an MFMA operand: row/column index ...
     const int fg = lane >> 4;        // ... and k group
 
@@ -83,16 +83,15 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
         qfrag[m] = __builtin_bit_cast(bf16x8_t, qv);
     }
 
-    const int ld_c = lane % T::LPR;  // this lane's 16-byte chunk of a token row in the global loads
-    const uint16_t* kbase = p.k + b * p.k_sb + kvh * p.k_sh + ld_c * 8;
-    const uint16_t* vbase = p.v + b * p.v_sb + kvh * p.v_sh + ld_c * 8;
+    const int64_t k_head = b * p.k_sb + kvh * p.k_sh;   // token 0 of this kv head, in elements
+    const int64_t v_head = b * p.v_sb + kvh * p.v_sh;
 
     f32x4_t O[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) O[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = kMaskedScore;  // running maximum of the raw scores (common to the four k groups of a head)
     float l_part = 0.f;          // this lane's share of the softmax denominator
-    mfma_tile_loop<HD, LOADS, true>(kbase, vbase, p.k_st, p.v_st, s_slab[wave], qfrag, t_begin + (COOP ? wave * WT : 0),
+    mfma_tile_loop<HD, LOADS, true>(p.k, p.v, k_head, v_head, p.k_st, p.v_st, s_slab[wave], qfrag, t_begin + (COOP ? wave * WT : 0),
                               t_end, STEP, t_end, t_end, c, O, m_run, l_part);
 
     // ---- this wavefront's result.  O[nb][r] is dim 16*nb + 4*fg + r of head fn; the softmax

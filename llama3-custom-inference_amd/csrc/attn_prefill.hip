@@ -26,7 +26,7 @@ attn_prefill_mfma_kernel(const PrefillParams p) {
     __shared__ __align__(16) unsigned char s_slab[kMfmaWaves][SLAB];
 
     const int lane = threadIdx.x & (kWaveSize - 1);
-    const int wave = threadIdx.x / kWaveSize;
+    const int wave = wave_uniform(int(threadIdx.x) / kWaveSize);
     const int fn = lane & 15;   // column of the MFMA tiles
     const int fg = lane >> 4;   // k group
 
@@ -59,16 +59,15 @@ attn_prefill_mfma_kernel(const PrefillParams p) {
         qfrag[m] = __builtin_bit_cast(bf16x8_t, qv);
     }
 
-    const int ld_c = lane % T::LPR;
-    const uint16_t* kbase = p.k + b * p.k_sb + kvh * p.k_sh + ld_c * 8;
-    const uint16_t* vbase = p.v + b * p.v_sb + kvh * p.v_sh + ld_c * 8;
+    const int64_t k_head = b * p.k_sb + kvh * p.k_sh;   // token 0 of this kv head, in elements
+    const int64_t v_head = b * p.v_sb + kvh * p.v_sh;
 
     f32x4_t O[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) O[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = kMaskedScore;
     float l_part = 0.f;
-    mfma_tile_loop<HD>(kbase, vbase, p.k_st, p.v_st, s_slab[wave], qfrag, 0, t_end, WT, col_limit, col_limit_min,
+    mfma_tile_loop<HD>(p.k, p.v, k_head, v_head, p.k_st, p.v_st, s_slab[wave], qfrag, 0, t_end, WT, col_limit, col_limit_min,
                        p.scale_log2e, O, m_run, l_part);
 
     l_part += __shfl_xor(l_part, 16, kWaveSize);

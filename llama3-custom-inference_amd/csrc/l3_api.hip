@@ -221,6 +221,8 @@ int check_attn_args(const void* q, const void* k, const void* v, const void* out
         if (kv_dims[i] == 1) continue;
         if (k_strides[i] < 0 || v_strides[i] < 0 || k_strides[i] % 8 || v_strides[i] % 8) return L3_ERR_STRIDE;
     }
+    // a tile's rows are addressed with 32-bit byte offsets from the tile's first token
+    if (S > 1 && (k_strides[2] >= kAttnMaxTokenStride || v_strides[2] >= kAttnMaxTokenStride)) return L3_ERR_STRIDE;
     if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || (need_out && !aligned(out, 16)))
         return L3_ERR_ALIGNMENT;
     return L3_OK;
@@ -339,6 +341,7 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
         if (kv_dims[i] != 1 && (k_strides[i] < 0 || v_strides[i] < 0 || k_strides[i] % 8 || v_strides[i] % 8))
             return L3_ERR_STRIDE;
     }
+    if (S > 1 && (k_strides[2] >= kAttnMaxTokenStride || v_strides[2] >= kAttnMaxTokenStride)) return L3_ERR_STRIDE;
     if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 16)) return L3_ERR_ALIGNMENT;
     PrefillParams p;
     p.q = static_cast<const uint16_t*>(q);

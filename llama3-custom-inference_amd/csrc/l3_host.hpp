@@ -23,6 +23,10 @@ constexpr int kAttnImplMfma = 1;
 
 constexpr int kMfmaWaves = 8;  // wavefronts per workgroup of the MFMA kernel
 
+// K/V token strides (elements) must stay below this: the MFMA kernels address the rows of a tile
+// (at most 64 tokens) with 32-bit byte offsets from the tile's first token.
+constexpr int64_t kAttnMaxTokenStride = int64_t(1) << 24;
+
 // Granularity of a split in tokens.  FMA kernel: one main-loop trip of its 4-wave workgroup
 // (4 x 8 KiB of K+V).  MFMA kernel: one tile of a wavefront (16 KiB of K+V).
 constexpr int attn_tile_tokens(int HD, int impl) {
