@@ -32,7 +32,7 @@ namespace {
 // workgroups per CU.
 template <int HD, bool COOP, int LOADS = 8>
 __global__ void __launch_bounds__(kMfmaWaves * kWaveSize, 2)
-attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg) {
+attn_splitkv_mfma_kernel(const int R, const int hpw_log2, const AttnParams p) {
     using T = MfmaTile<HD, LOADS>;
     constexpr int WT = T::WT, KC = T::KC, NB = T::NB, SLAB = T::SLAB;
     constexpr int STEP = COOP ? kMfmaWaves * WT : WT;  // token stride between a wavefront's tiles
@@ -46,31 +46,23 @@ attn_splitkv_mfma_kernel(const AttnParams p, const int R, const int heads_per_wg
     const int fn = lane & 15;        // role in an MFMA operand: row/column index ...
     const int fg = lane >> 4;        // ... and k group
 
-    int b, kvh, split;
+    // Grid: x = kv head (COOP) or group of 2^hpw_log2 adjacent kv heads, y = batch, z = split (COOP)
+    // or group of splits -- no division on the way to the first load.
+    const int b = blockIdx.y;
+    int kvh, split;
     if constexpr (COOP) {
-        // workgroup -> (batch, kv head, split), kv head fastest
-        int bid = blockIdx.x;
-        kvh = bid % p.KVH;
-        bid /= p.KVH;
-        b = bid % p.B;
-        split = bid / p.B;
+        kvh = blockIdx.x;
+        split = blockIdx.z;
     } else {
-        // workgroup -> (batch, group of heads_per_wg adjacent kv heads, group of splits); its eight
-        // wavefronts -> heads_per_wg heads x (8 / heads_per_wg) consecutive splits
-        const int head_groups = p.KVH / heads_per_wg;
-        const int splits_per_wg = kMfmaWaves / heads_per_wg;
-        int bid = blockIdx.x;
-        const int hg = bid % head_groups;
-        bid /= head_groups;
-        b = bid % p.B;
-        const int sg = bid / p.B;
-        kvh = hg * heads_per_wg + wave % heads_per_wg;
-        split = sg * splits_per_wg + wave / heads_per_wg;
-        if (split >= p.num_splits) return;  // whole wavefront; no barrier follows
+        // the eight wavefronts -> 2^hpw_log2 heads x (8 >> hpw_log2) consecutive splits
+        kvh = (int(blockIdx.x) << hpw_log2) + (wave & ((1 << hpw_log2) - 1));
+        split = (int(blockIdx.z) << (3 - hpw_log2)) + (wave >> hpw_log2);
     }
     const int t_begin = split * p.tokens_per_split;
     const int S = p.seqlen_dev ? max(1, min(*p.seqlen_dev, p.S)) : p.S;  // wave-uniform; a length below 1 counts as 1
-    if (t_begin >= S) return;  // split beyond a device-side KV length (whole workgroup when COOP): the combine skips it
+    // A split past the plan (last workgroup of the streaming form: whole wavefront, no barrier follows)
+    // or past a device-side KV length (whole workgroup when COOP): the combine skips it.
+    if (split >= p.num_splits || t_begin >= S) return;
     const int t_end = min(S, t_begin + p.tokens_per_split);
     const float c = p.scale_log2e;
 
@@ -176,29 +168,48 @@ int attn_mfma_heads_per_wg(int KVH) {
     return 1;
 }
 
-int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipStream_t stream) {
+int launch_attn_splitkv_mfma(const AttnParams& params, int HD, int R, bool coop, hipStream_t stream) {
     if (R < 1 || R > kAttnMaxRatio) return int(hipErrorInvalidValue);
     const dim3 block(kMfmaWaves * kWaveSize);
-    if (coop) {
-        const dim3 grid(unsigned(p.B) * unsigned(p.KVH) * unsigned(p.num_splits));
-        if (HD == 64 && p.tokens_per_split <= 2 * kMfmaWaves * 32) {
-            hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, true, 4>), grid, block, 0, stream, p, R, 1);
-        } else if (HD == 64) {
-            hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, true>), grid, block, 0, stream, p, R, 1);
-        } else {
-            hipLaunchKernelGGL((attn_splitkv_mfma_kernel<128, true>), grid, block, 0, stream, p, R, 1);
-        }
-        return int(hipGetLastError());
-    }
-    const int hpw = attn_mfma_heads_per_wg(p.KVH);
+    const int hpw = attn_mfma_heads_per_wg(params.KVH);
+    int hpw_log2 = 0;
+    while ((1 << hpw_log2) < hpw) ++hpw_log2;
     const int spw = kMfmaWaves / hpw;
-    const dim3 grid(unsigned(p.B) * unsigned(p.KVH / hpw) * unsigned((p.num_splits + spw - 1) / spw));
-    if (HD == 64) {
-        hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, false>), grid, block, 0, stream, p, R, hpw);
-    } else {
-        hipLaunchKernelGGL((attn_splitkv_mfma_kernel<128, false>), grid, block, 0, stream, p, R, hpw);
+    // The batch index is the grid's y dimension (at most 65535): larger batches go out in slices, each
+    // with its pointers moved to the slice's first sequence.
+    constexpr int kMaxGridY = 65535;
+    for (int b0 = 0; b0 < params.B; b0 += kMaxGridY) {
+        AttnParams p = params;
+        p.B = (params.B - b0 < kMaxGridY) ? params.B - b0 : kMaxGridY;
+        p.q += b0 * p.q_sb;
+        p.k += b0 * p.k_sb;
+        p.v += b0 * p.v_sb;
+        if (p.out) p.out += b0 * p.o_sb;
+        if (p.part_o) {
+            const int64_t row0 = int64_t(b0) * p.QH * p.num_splits;
+            p.part_o += row0 * HD;
+            p.part_ml += row0;
+        }
+        if (coop) {
+            const dim3 grid(unsigned(p.KVH), unsigned(p.B), unsigned(p.num_splits));
+            if (HD == 64 && p.tokens_per_split <= 2 * kMfmaWaves * 32) {
+                hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, true, 4>), grid, block, 0, stream, R, 0, p);
+            } else if (HD == 64) {
+                hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, true>), grid, block, 0, stream, R, 0, p);
+            } else {
+                hipLaunchKernelGGL((attn_splitkv_mfma_kernel<128, true>), grid, block, 0, stream, R, 0, p);
+            }
+        } else {
+            const dim3 grid(unsigned(p.KVH / hpw), unsigned(p.B), unsigned((p.num_splits + spw - 1) / spw));
+            if (HD == 64) {
+                hipLaunchKernelGGL((attn_splitkv_mfma_kernel<64, false>), grid, block, 0, stream, R, hpw_log2, p);
+            } else {
+                hipLaunchKernelGGL((attn_splitkv_mfma_kernel<128, false>), grid, block, 0, stream, R, hpw_log2, p);
+            }
+        }
+        if (const hipError_t e = hipGetLastError(); e != hipSuccess) return int(e);
     }
-    return int(hipGetLastError());
+    return 0;
 }
 
 }  // namespace l3

@@ -42,21 +42,23 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
 // Compute units of the current device, 256 when no device can be queried.
 int current_device_cus();
 
+// What a wavefront needs before it can issue its first K/V load comes first, so that it sits in the
+// first 64 bytes of the kernel arguments (one scalar-cache miss instead of three in a row).
 struct AttnParams {
+    int B, QH, KVH, S;
+    int num_splits, tokens_per_split;
+    const int* seqlen_dev;  // when set, the KV length is read from here (<= S, which then only bounds the plan)
     const uint16_t* q;
     const uint16_t* k;
     const uint16_t* v;
+    int64_t k_sb, k_sh, k_st;
+    int64_t v_sb, v_sh, v_st;
+    int64_t q_sb, q_sh;
+    float scale_log2e;
     uint16_t* out;
     float* part_o;    // [B][QH][num_splits][HD] unnormalised partial outputs; null = write `out` directly
     float2* part_ml;  // [B][QH][num_splits] (max in log2 units, sum of exp2)
-    int B, QH, KVH, S;
-    const int* seqlen_dev;  // when set, the KV length is read from here (<= S, which then only bounds the plan)
-    int num_splits, tokens_per_split;
-    int64_t q_sb, q_sh;
-    int64_t k_sb, k_sh, k_st;
-    int64_t v_sb, v_sh, v_st;
     int64_t o_sb, o_sh;
-    float scale_log2e;
 };
 
 struct PrefillParams {

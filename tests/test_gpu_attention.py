@@ -165,6 +165,30 @@ def test_inputs_are_not_modified_and_errors_are_raised(gpu):
         cke.flash_attention_decode(*make_qkv(1, 10, 2, 16, 64, device=gpu))
     with pytest.raises(RuntimeError, match="BFloat16"):
         cke.flash_attention_decode(q.float(), k, v)
+    # a token stride of 2^24 elements or more is refused (a tile's rows are addressed with 32-bit
+    # offsets); nothing is read through the view
+    wide = torch.zeros((1 << 24) + 8 * 64, device=gpu, dtype=torch.bfloat16).as_strided((1, 8, 2, 64), (0, 64, 1 << 24, 1))
+    with pytest.raises(RuntimeError, match="stride"):
+        cke.flash_attention_decode(q, wide, wide)
+
+
+def test_more_sequences_than_one_grid_dimension_holds(gpu):
+    """The batch index is a grid dimension of at most 65535 entries; a larger batch goes out in slices.
+    Every sequence, those of the second slice included, must match the oracle."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    B, QH, KVH, S, HD = 65535 + 70, 2, 1, 40, 64
+    q, k, v = make_qkv(B, QH, KVH, S, HD, seed=77)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    for splits in (1, 2):
+        out = cke.flash_attention_decode(qg, kg, vg, splits)
+        torch.cuda.synchronize()
+        tail = slice(B - 200, B)
+        ref = attention_decode_ref(t2f32(q[tail]), t2f32(k[tail]), t2f32(v[tail]))
+        assert_attn_close(out[tail], ref, what=f"last 200 of {B} sequences, splits {splits}", min_kv_len=S)
+        head = slice(0, 64)
+        ref = attention_decode_ref(t2f32(q[head]), t2f32(k[head]), t2f32(v[head]))
+        assert_attn_close(out[head], ref, what=f"first 64 of {B} sequences, splits {splits}", min_kv_len=S)
 
 
 def test_runs_on_the_current_stream(gpu):
