@@ -67,6 +67,26 @@ def test_many_sequences_with_few_splits(gpu, attn_kernel, B, QH, KVH, S, HD, spl
     _run(gpu, B, QH, KVH, S, HD, seed=B + splits, splits=splits)
 
 
+@pytest.mark.parametrize("B,QH,KVH,S,HD", [(1, 32, 8, 513, 128), (1, 32, 8, 1000, 128), (1, 32, 8, 2048, 128),
+                                            (1, 32, 8, 4097, 128), (1, 32, 8, 8192, 128), (1, 32, 8, 600, 64),
+                                            (1, 32, 8, 1024, 64), (1, 32, 8, 3000, 64), (1, 32, 8, 4096, 64),
+                                            (3, 8, 2, 777, 128), (2, 32, 8, 1500, 64), (5, 6, 3, 290, 128),
+                                            (1, 8, 1, 5000, 128), (64, 8, 2, 300, 128)])
+def test_medium_sequences_over_few_heads(gpu, attn_kernel, B, QH, KVH, S, HD):
+    """The plan's own choice for medium lengths over few (batch, kv head) pairs: with the MFMA kernel,
+    cooperative workgroups over several splits (one merged partial row per workgroup) plus the combine.
+    Checked against the oracle and against a forced split count, which takes the streaming form."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    if attn_kernel == "mfma":
+        assert cke.attention_num_splits(B, KVH, S, HD, 256) > 1
+    out, ref, _ = _run(gpu, B, QH, KVH, S, HD, seed=S + HD)
+    qg, kg, vg = make_qkv(B, QH, KVH, S, HD, seed=S + HD, device=gpu)
+    forced = cke.flash_attention_decode(qg, kg, vg, 5)
+    torch.cuda.synchronize()
+    assert (out.float() - forced.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, np.abs(ref).max())
+
+
 @pytest.mark.parametrize("HD", [64, 128])
 @pytest.mark.parametrize("splits", [1, 2, 5, 16, 512])
 def test_result_independent_of_split_count(gpu, HD, splits):
