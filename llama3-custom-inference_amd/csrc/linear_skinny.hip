@@ -48,8 +48,8 @@ __device__ __forceinline__ void store_qkv_pair(const LinearParams& p, int m, int
 // Elements of LDS the staged activations may take (rows are padded by 8 elements).
 constexpr int kXldsMaxElems = 24576;
 
-// RW = weight rows per wavefront.  16: the plain mapping above.  4 (at most 4 activation rows, one
-// matrix): the 16 rows and the 16 columns of a matrix instruction are both split into four k
+// RW = weight rows per wavefront.  16: the plain mapping above.  4 (at most 4 activation rows):
+// the 16 rows and the 16 columns of a matrix instruction are both split into four k
 // ranges -- tile row i is weight row i % 4 over k range i / 4, tile column j is activation row
 // j % 4 over k range j / 4 -- so one instruction covers 4 weight rows x 128 k, the blocks on the
 // diagonal (i / 4 == j / 4) hold the products and the rest is ignored.  Four times as many
@@ -58,7 +58,7 @@ template <int NW, int CBLK, int U, bool SWIGLU, bool XLDS, int RW>
 __global__ void __launch_bounds__(NW * kWaveSize)
 linear_skinny_kernel(const LinearParams p) {
     static_assert(!XLDS || CBLK == 1, "activations are staged in LDS only for up to 16 rows");
-    static_assert(RW == 16 || (RW == 4 && CBLK == 1 && !SWIGLU), "the four-row mapping is for one matrix");
+    static_assert(RW == 16 || (RW == 4 && CBLK == 1), "the four-row mapping takes at most four activation rows");
     constexpr int KQ = 16 / RW;                            // k ranges per matrix instruction
     constexpr int KSTEP = 32 * KQ;                         // k covered by one step
     constexpr int ACC = SWIGLU ? 2 : 1;
@@ -218,19 +218,31 @@ linear_skinny_kernel(const LinearParams p) {
         // range l / 16 against activation row (l % 16) % 4 over k range (l % 16) / 4.  The lanes
         // whose two k ranges agree hold products; they meet, with the other wavefronts of the row
         // group, in LDS, and the group's first wavefront finishes its 4 x 4 results.
-        float* part = &s_red[wave][0][0][0];
         if ((fn >> 2) == fg) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) part[(fg * 4 + (fn & 3)) * 4 + t] = acc[0][0][t];
+            for (int a = 0; a < ACC; ++a) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) s_red[wave][a][0][(fg * 4 + (fn & 3)) * 4 + t] = acc[a][0][t];
+            }
         }
         __syncthreads();
         if (kslice != 0 || lane >= 16) return;
         const int m = lane >> 2, t = lane & 3;             // activation row, weight row within the group
         const int n = n0 + t;
-        float o = 0.f;
-        for (int w = 0; w < sk; ++w) {
+        float oa[ACC];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) o += s_red[wave + w][0][0][(q * 4 + m) * 4 + t];
+        for (int a = 0; a < ACC; ++a) {
+            oa[a] = 0.f;
+            for (int w = 0; w < sk; ++w) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) oa[a] += s_red[wave + w][a][0][(q * 4 + m) * 4 + t];
+            }
+        }
+        float o = oa[0];
+        if constexpr (SWIGLU) {
+            const float g = __uint_as_float(f32_to_bf16_bits(oa[0]) << 16);
+            const float u = __uint_as_float(f32_to_bf16_bits(oa[ACC - 1]) << 16);
+            o = silu_rounded(g) * u;
         }
         if (p.rope_table) {   // the even lane of a pair takes its partner's value and stores both
             const float o1 = __shfl_xor(o, 1, kWaveSize);
@@ -342,10 +354,20 @@ int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t s
     if (p.M > 16) return int(hipErrorInvalidValue);   // one 16-column MFMA block of activation rows (checked by the caller)
     const bool stage = p.norm_w != nullptr;   // the caller has checked linear_skinny_can_stage
     const int row_blocks = (p.N + 15) / 16;
-    // a matrix with too few 16-row blocks to fill the device, and at most four activation rows:
-    // four weight rows per wavefront
-    if (!swiglu && p.M <= 4 && p.K % 128 == 0 && row_blocks < 2 * num_cus) {
-        p.sk = linear_skinny_plan(p.N, p.K, 8, num_cus, 4, 128);
+    // At most four activation rows: four weight rows per wavefront, each read 256 contiguous bytes at a
+    // time.  A matrix with too few 16-row blocks to fill the device gets its K split by the plan; a
+    // large one (the vocabulary projection: 105 -> 86 us at 128256 x 2048) two wavefronts per row
+    // group (one: 92 us, four: 125 us).
+    if (p.M <= 4 && p.K % 128 == 0) {
+        if (row_blocks < 2 * num_cus) {
+            p.sk = linear_skinny_plan(p.N, p.K, 8, num_cus, 4, 128);
+        } else {
+            p.sk = (p.K / 128 >= 16) ? 2 : 1;
+        }
+        if (swiglu) {
+            return stage ? launch_variant<8, 1, 8, true, true, 4>(p, stream)
+                         : launch_variant<8, 1, 8, true, false, 4>(p, stream);
+        }
         return stage ? launch_variant<8, 1, 8, false, true, 4>(p, stream)
                      : launch_variant<8, 1, 8, false, false, 4>(p, stream);
     }
