@@ -432,6 +432,10 @@ def north_star_extras(args, torch, lib, l3, dev, pool):
            "c1_b1_hd64_s256": measure_attention_shape(torch, lib, l3, dev, pool, 1, QH, KVH, 256, 64, with_sdpa=sdpa),
            "c3a_b256_hd64_s256": measure_attention_shape(torch, lib, l3, dev, pool, 256, QH, KVH, 256, 64, with_sdpa=sdpa),
            "c3b_b16_hd64_s4096": measure_attention_shape(torch, lib, l3, dev, pool, 16, QH, KVH, 4096, 64, with_sdpa=sdpa)}
+    # beyond the configured sweep: where batch 1 crosses the target as the stream grows against the fixed
+    # cost of two launches
+    out["longer_kv_b1"] = [measure_attention_shape(torch, lib, l3, dev, pool, 1, QH, KVH, S, HD, with_sdpa=sdpa)
+                           for HD in (128, 64) for S in (65536, 131072)]
     out["rms_norm"] = [rows_record(torch, lib, l3, dev, "rms", 2, 2048, C) for C in (2048, 4096)]
     out["rot_embed"] = [rows_record(torch, lib, l3, dev, "rope", 2, 2048, HD) for HD in (64, 128)]
     return out
@@ -808,6 +812,7 @@ def main():
             ns["target_frac"] = target
             ns["points_at_or_above_target"] = sum(r["frac"] >= target for r in pts)
             ns["points"] = len(pts)
+            ns["longer_kv_points_at_or_above_target"] = sum(r["frac"] >= target for r in ns["longer_kv_b1"])
             line["north_star"] = ns
         del pool
         torch.cuda.empty_cache()

@@ -125,9 +125,10 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
             // head's token range, merged through LDS into ONE partial row per workgroup), spread over
             // the units with at least two tiles each.  Against the streaming form this measured
             // 6.7 instead of 8.6 us at 1024 tokens and 11.5 instead of 12.4 us at 8192 (head size 128,
-            // batch 1, 8 kv heads); from two tiles per wavefront on the streaming form's whole-row
-            // reads win (head size 64, whose per-head rows are 128 bytes: from one tile per wavefront).
-            const int64_t coop_tiles = int64_t(HD == 128 ? kMfmaWaves : kMfmaWaves / 2) * wgs;
+            // batch 1, 8 kv heads) and 13.6 instead of 14.2 us at 12288; from two tiles per wavefront on
+            // (16384: 17.9 against 16.2 us) the streaming form's whole-row reads win (head size 64, whose
+            // per-head rows are 128 bytes: from one tile per wavefront).
+            const int64_t coop_tiles = int64_t(HD == 128 ? kMfmaWaves * 3 / 2 : kMfmaWaves / 2) * wgs;
             if (tiles <= coop_tiles) {
                 int coop_splits = std::min(wgs, ceil_div(tiles, 2));
                 if (coop_splits > L3_ATTN_MAX_SPLITS) coop_splits = L3_ATTN_MAX_SPLITS;
@@ -161,7 +162,19 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
                 groups = 2;
             }
         } else {
-            groups = int64_t(num_cus) / wgs_per_split_group;
+            // Few workgroups per split group (batch 1 of a long sequence): four fifths of the units, each
+            // with a longer stream, beat one workgroup on every unit (16384 tokens at head size 128: 171
+            // workgroups of three tiles per wavefront 16.0 us, 256 of two 16.9 us; 32768: 205 of five
+            // 25.5 us, 256 of four 26.2 us) -- fewer starts and ends, fewer partials for the combine --
+            // as long as the rounding to whole tiles leaves at least three fifths of the units busy.
+            groups = (int64_t(num_cus) * 4 + 4) / 5 / wgs_per_split_group;
+            if (groups < 1) groups = 1;
+            int64_t split_tiles = ceil_div(tiles, int(std::min<int64_t>(groups * spg, tiles)));
+            while (split_tiles > 1 &&
+                   ceil_div(tiles, int(split_tiles)) / spg * wgs_per_split_group * 5 < int64_t(num_cus) * 3) {
+                --split_tiles;
+            }
+            groups = ceil_div(ceil_div(tiles, int(split_tiles)), spg);
         }
         splits = int(groups * spg);
     } else {
