@@ -149,7 +149,9 @@ def test_split_planning():
         assert lib.l3_attn_choose_splits(1, 8, 32768, HD, 64, 0) < lib.l3_attn_choose_splits(1, 8, 32768, HD, 256, 0)
     # many sequences (8 kv heads: one workgroup per sequence and split group, 256 units):
     plan = lambda B, S, HD: lib.l3_attn_choose_splits(B, 8, S, HD, 256, 0)  # noqa: E731
-    assert plan(3, 32768, 128) == 79            # at most 85 (3 * 85 = 255 workgroups for 256 units), whole tiles: 79 x 416 tokens
+    assert plan(3, 32768, 128) == 64            # four fifths of the units (68 groups of 3 workgroups at most), whole tiles: 64 x 512 tokens
+    assert plan(1, 32768, 128) == 205 and plan(1, 16384, 128) == 171   # 5 and 3 tiles per wavefront
+    assert plan(1, 12288, 128) == 32 and plan(1, 8192, 64) == 32       # cooperative form: one workgroup per unit
     assert plan(4, 4096, 64) == 64              # few sequences: one workgroup per unit
     assert plan(16, 4096, 64) == 11             # from 8 sequences on, three quarters of the units: 12 groups, whole tiles
     assert plan(48, 4096, 128) == 4
