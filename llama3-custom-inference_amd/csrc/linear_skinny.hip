@@ -66,7 +66,7 @@ linear_skinny_kernel(const LinearParams p) {
     extern __shared__ __align__(16) uint16_t s_x[];        // XLDS: M rows of K + 8 elements
 
     const int lane = threadIdx.x & (kWaveSize - 1);
-    const int wave = threadIdx.x / kWaveSize;
+    const int wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x) / kWaveSize);   // scalar: what derives from it is wave-uniform
     const int fn = lane & 15;
     const int fg = lane >> 4;
 
