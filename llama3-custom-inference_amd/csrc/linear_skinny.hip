@@ -357,7 +357,11 @@ int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t s
     // At most four activation rows: four weight rows per wavefront, each read 256 contiguous bytes at a
     // time.  A matrix with too few 16-row blocks to fill the device gets its K split by the plan; a
     // large one (the vocabulary projection: 105 -> 86 us at 128256 x 2048) two wavefronts per row
-    // group (one: 92 us, four: 125 us).
+    // group (one: 92 us, four: 125 us).  A ring of four k steps per wavefront: eight cost 0.1 us per
+    // small matrix and 0.3 us on the gate|up pair, sixteen 2 ... 50 us; more bytes in flight per compute
+    // unit than the memory system wants slow it down (a ring kept full across rounds, with exact load
+    // counts instead of a wait for the whole ring per round, made the vocabulary projection 89 us
+    // instead of 77).
     if (p.M <= 4 && p.K % 128 == 0) {
         if (row_blocks < 2 * num_cus) {
             p.sk = linear_skinny_plan(p.N, p.K, 8, num_cus, 4, 128);
@@ -365,11 +369,11 @@ int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t s
             p.sk = (p.K / 128 >= 16) ? 2 : 1;
         }
         if (swiglu) {
-            return stage ? launch_variant<8, 1, 8, true, true, 4>(p, stream)
-                         : launch_variant<8, 1, 8, true, false, 4>(p, stream);
+            return stage ? launch_variant<8, 1, 4, true, true, 4>(p, stream)
+                         : launch_variant<8, 1, 4, true, false, 4>(p, stream);
         }
-        return stage ? launch_variant<8, 1, 8, false, true, 4>(p, stream)
-                     : launch_variant<8, 1, 8, false, false, 4>(p, stream);
+        return stage ? launch_variant<8, 1, 4, false, true, 4>(p, stream)
+                     : launch_variant<8, 1, 4, false, false, 4>(p, stream);
     }
     // few row blocks and a long K (the MLP's down projection): sixteen wavefronts share a row block
     const bool big_wg = !swiglu && row_blocks < num_cus && p.K / 32 >= 128;
