@@ -42,7 +42,7 @@ linear_splitk_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict_
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
-    const int wave = tid / kWaveSize;
+    const int wave = wave_uniform(tid / kWaveSize);   // scalar: what derives from it is wave-uniform
     const int fn = lane & 15;
     const int fg = lane >> 4;
 
