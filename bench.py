@@ -15,8 +15,9 @@ Prints ONE JSON line: value = algorithmic GB/s (K+V+Q read, O written) over the 
 "roofline" prices the split-KV kernel alone against the 8 TB/s HBM peak from HIP-event timing and
 carries the read bandwidth a pure stream reaches on the same device; "cpu_baseline" is stock
 PyTorch on the host cores for a bounded sample of the same sweep.  The same line carries the rest
-of the target ("north_star": head_dim 64, the batched shapes, RMSNorm, rotary embedding, each
-cold, torch's own attention beside the decode kernel) and the end-to-end tokens/s ("e2e").
+of the target ("north_star": head_dim 64, the batched shapes, longer KV lengths, RMSNorm, rotary
+embedding, each cold; beside every attention shape torch's own attention on the same GPU and the
+time a kernel that only reads takes for the same bytes) and the end-to-end tokens/s ("e2e").
 
 Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|prefill|linear|e2e|copy|readstream) report the
 remaining configurations in the same format.
@@ -268,6 +269,9 @@ def measure_attention_shape(torch, lib, l3, dev, pool, B, QH, KVH, S, HD, cache_
         del sg
     if with_sdpa:
         rec["torch_sdpa_us"] = torch_sdpa_us(torch, c)
+    if not split_stage:
+        # what a kernel that only reads takes for the same number of bytes, cold, launched the same way
+        rec["read_stream_us"] = measure_read_stream(torch, lib, dev, pool, (c.bytes + 255) // 256 * 256)["us"]
     return rec
 
 
