@@ -112,6 +112,14 @@ class LlamaDecoder:
             for name in ("c_attn", "c_proj", "c_fc", "c_fc2", "mlp_proj"):
                 yield L[name]
 
+    def prefill_pass_mode(self):
+        """How generate_graphed ran its prompt passes so far: 'recorded' (HIP graph, checked against the
+        eager pass), 'eager' (the recording did not reproduce the eager logits) or 'none yet'."""
+        entries = [e for loop in self._graphs.values() for e in loop.prefill_graphs.values()]
+        if not entries:
+            return "none yet"
+        return "recorded" if all(e[0] is not None for e in entries) else "eager"
+
     def set_decode_linear_rows(self, rows: int):
         self.decode_linear_rows = rows if hasattr(self.ops, "linear_decode") else 0
         self._graphs.clear()   # recorded decode steps contain the previous choice
@@ -249,14 +257,14 @@ class LlamaDecoder:
             h = self.ops.rms_norm(x, L["ln_2"], c.norm_eps)
             x = x + self._mlp(L, h)
         x = self.ops.rms_norm(x, self.ln_f, c.norm_eps)
-        return self._linear(x[:, [-1], :], self.wte).float()
+        return self._linear(x[:, -1:, :].contiguous(), self.wte).float()
 
     # ------------------------------------------------------------------------- generate
     @torch.inference_mode()
     def generate_graphed(self, prompt_tokens, max_gen_len, echo=False, ignore_eos=False):
-        """generate() with the per-token loop replayed from a HIP graph: prefill of the common
-        prompt prefix runs eagerly (model.py:365 with T = min_prompt_len), every later position is
-        one graph replay.  Needs ops with rot_embed_append / flash_attention_decode_devlen."""
+        """generate() with the per-token loop replayed from a HIP graph: the prefill of the common
+        prompt prefix (model.py:365 with T = min_prompt_len) is one recorded pass, every later position
+        one replay of the recorded decode step.  Needs ops with rot_embed_append / flash_attention_decode_devlen."""
         c = self.config
         bsz = len(prompt_tokens)
         min_prompt_len = min(len(t) for t in prompt_tokens)
@@ -275,8 +283,8 @@ class LlamaDecoder:
         loop.tokens.copy_(host)
         loop.text_mask.copy_(host != pad_id)
         loop.eos.zero_()
-        # position min_prompt_len: eager prefill + the usual bookkeeping
-        logits = self.forward(loop.tokens[:, :min_prompt_len], start_pos=0)
+        # position min_prompt_len: prefill (recorded once per prompt length) + the usual bookkeeping
+        logits = loop.prefill(self, min_prompt_len)
         nxt = torch.argmax(logits[:, -1], dim=-1)
         if min_prompt_len < total_len:
             keep = loop.text_mask[:, min_prompt_len]
@@ -371,6 +379,7 @@ class GraphedDecodeLoop:
         self.eos = _t.zeros(batch, dtype=_t.bool, device=dev)
         self.stop = _t.tensor(list(model.tokenizer.stop_tokens), device=dev)
         self.graph = None
+        self.prefill_graphs = {}   # prompt length -> (recorded prefill or None when it failed its check, logits)
 
     def step(self, m: "LlamaDecoder"):
         c, B = m.config, self.B
@@ -435,6 +444,44 @@ class GraphedDecodeLoop:
         self.tok.copy_(nxt.unsqueeze(1))
         self.pos += 1
         self.kv_len += 1
+
+    def prefill(self, m: "LlamaDecoder", T: int):
+        """Logits of the prompt's first T positions (model.py:365 with start_pos 0) for the tokens in
+        self.tokens.  The eager pass costs ~260 launches from Python (3.3 ms at batch 1, against 0.64 ms
+        for a decode step), so it is recorded too, once per prompt length.  A recorded pass is used only
+        after it has reproduced the eager logits bit for bit on two replays with eager work in between
+        (library GEMMs may record nodes that misbehave on later replays); otherwise the eager pass stays."""
+        import gc
+
+        entry = self.prefill_graphs.get(T)
+        if entry is None:
+            dev = m.device
+            ref = m.forward(self.tokens[:, :T], start_pos=0).clone()   # eager: also the warm-up for the capture
+            torch.cuda.synchronize(dev)
+            graph, out = None, None
+            gc.collect()
+            gc_was_enabled = gc.isenabled()
+            gc.disable()
+            try:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    out = m.forward(self.tokens[:, :T], start_pos=0)
+            finally:
+                if gc_was_enabled:
+                    gc.enable()
+            ok = True
+            for _ in range(2):
+                graph.replay()
+                torch.cuda.synchronize(dev)
+                ok = ok and bool(torch.equal(out, ref))
+                again = m.forward(self.tokens[:, :T], start_pos=0)      # eager work between the replays
+                ok = ok and bool(torch.equal(again, ref))
+            entry = (graph, out) if ok else (None, None)
+            self.prefill_graphs[T] = entry
+        if entry[0] is None:
+            return m.forward(self.tokens[:, :T], start_pos=0)
+        entry[0].replay()
+        return entry[1]
 
     def capture(self, m: "LlamaDecoder"):
         import gc
@@ -519,6 +566,7 @@ def e2e_summary(torch_mod, dev, batches=(1, 64), input_len=128, gen_len=128, rep
         out[f"bs{batch}"] = {"tok_per_s": round(best, 1), "us_per_generated_token_step": round(1e6 * batch / best, 1),
                              "eager_tok_per_s": round(eager_tps, 1),
                              "graphed_vs_eager_same_tokens": f"{same}/{batch * gen_len}",
+                             "prefill_pass": model.prefill_pass_mode(),
                              "weight_stream_frac_of_hbm_peak": round(2471628800 * best / batch / 8e12, 4)}
     out["config"] = (f"Llama-3.2-1B architecture, random init, {input_len} prompt ids + {gen_len} greedy tokens, "
                      "prefill included, decode loop replayed from a HIP graph")
@@ -579,6 +627,7 @@ def bench_e2e(args, torch_mod, dev, cpu_ops=None):
         same = sum(a == b for ra, rb in zip(rec.pop("eager_tokens"), rec.pop("graphed_tokens")) for a, b in zip(ra, rb))
         rec["graphed_vs_eager_same_tokens"] = f"{same}/{batch * gen_len}"
         rec["prefill"] = model.prefill_backend
+        rec["prefill_pass"] = model.prefill_pass_mode()
         results[batch] = rec
         del model
         torch_mod.cuda.empty_cache()

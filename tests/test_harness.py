@@ -142,6 +142,19 @@ def test_graphed_decode_loop_matches_eager(gpu, batch):
                 common += 1
             assert common >= 15, f"graphed and eager streams diverge after {common} tokens: {a} vs {b}"
     assert len(m._graphs) >= 1 and all(g.graph is not None for g in m._graphs.values())
+    # the prompt pass of generate_graphed: whichever way it runs (recorded, or eager when the recording
+    # failed its own check), new prompts through it give the eager pass's logits, replay after replay
+    assert m.prefill_pass_mode() in ("recorded", "eager")
+    print(f"prompt pass: {m.prefill_pass_mode()}", flush=True)
+    with torch.inference_mode():
+        for loop in m._graphs.values():
+            for T in list(loop.prefill_graphs):
+                for seed in (7, 8, 9):
+                    g = torch.Generator().manual_seed(seed)
+                    loop.tokens[:, :T] = torch.randint(0, 900, (loop.tokens.shape[0], T), generator=g).to(gpu)
+                    got = loop.prefill(m, T).clone()
+                    want = m.forward(loop.tokens[:, :T], start_pos=0)
+                    assert torch.equal(got, want), f"prompt pass T={T} seed={seed}"
 
 
 # ---- the end-to-end configuration at its own size (Llama-3.2-1B architecture, model.py:153-166;
