@@ -36,34 +36,26 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
-template <int HD, int CB, int NW>
-struct PrefillTile {
-    static constexpr int NT = NW * kWaveSize;      // threads
-    static constexpr int TK = 64;                  // tokens per K/V tile
-    static constexpr int LPR = HD / 8;             // 16-byte chunks per token row
-    static constexpr int CHUNKS = TK * LPR;        // chunks per K (or V) tile
-    static constexpr int U = CHUNKS / NT;          // chunks per thread per operand
-    static constexpr int NG = TK / 16;
-    static constexpr int KC = HD / 32;
-    static constexpr int NB = HD / 16;
-    static constexpr int KS = TK / 32;
-    static constexpr int KPITCH = HD * 2 + 16;
-    static constexpr int VPITCH = HD * 2 + 32;
-    static constexpr int KBYTES = TK * KPITCH;
-    static constexpr int VBYTES = TK * VPITCH;
-    static constexpr int STAGE = KBYTES + VBYTES;  // one buffer: a K tile followed by a V tile
-    static_assert(CHUNKS % NT == 0, "tile must divide evenly over the workgroup");
-};
-
-// Two wavefronts per SIMD whatever the workgroup size: a 4-wave workgroup could otherwise be given
-// 512 registers per wavefront, and then only one workgroup would fit a compute unit.
-template <int HD, int CB, int NW>
-__global__ void __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// Tiled form.  Few registers on purpose (128 at head size 64): WPE wavefronts per SIMD, i.e. several
+// independent workgroups per compute unit whose matrix, vector and LDS phases, barriers, start-up and
+// drain cover each other.  K/V tiles go from global memory straight into LDS
+// (global_load_lds_dwordx4: a wavefront-wide load lands in 1 KiB of consecutive LDS), so rows are
+// not padded; instead the 16-byte chunk c of token row r sits at chunk position c ^ key(r), which
+// spreads the rows that an operand read touches together over all banks.  The two stages are separate
+// arrays, so that the compiler can tell a read of one from the load in flight into the other.
+template <int HD, int CB, int NW, int TK, int WPE>
+__global__ void __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 attn_prefill_tiled_kernel(const PrefillParams p) {
-    using T = PrefillTile<HD, CB, NW>;
-    constexpr int NT = T::NT, TK = T::TK, LPR = T::LPR, U = T::U, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
-    constexpr int KPITCH = T::KPITCH, VPITCH = T::VPITCH, KBYTES = T::KBYTES, STAGE = T::STAGE;
-    __shared__ __align__(16) unsigned char s_tiles[2 * STAGE];
+    constexpr int NG = TK / 16, KS = TK / 32, KC = HD / 32, NB = HD / 16;
+    constexpr int CPR = HD / 8;                  // 16-byte chunks per token row
+    constexpr int ROWB = HD * 2;                 // bytes per token row
+    constexpr int KBYTES = TK * ROWB;            // a K tile; a stage is a K tile followed by a V tile
+    constexpr int STAGE = 2 * KBYTES;
+    constexpr int LOADS = TK * CPR / kWaveSize;  // wavefront-wide loads per operand tile
+    static_assert(LOADS % NW == 0, "a tile must divide evenly over the wavefronts");
+    constexpr int IPW = LOADS / NW;
+    __shared__ __align__(1024) unsigned char s_stage0[STAGE];
+    __shared__ __align__(1024) unsigned char s_stage1[STAGE];
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWaveSize - 1);
@@ -107,28 +99,42 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         }
     }
 
-    // global -> LDS staging: chunk (tid + u*NT) of a tile is 16 bytes of token row chunk / LPR
-    const uint16_t* kbase = p.k + b * p.k_sb + kvh * p.k_sh + (tid % LPR) * 8;
-    const uint16_t* vbase = p.v + b * p.v_sb + kvh * p.v_sh + (tid % LPR) * 8;
-    const int ld_row = tid / LPR;
-    constexpr int ROWS_PER_LOAD = NT / LPR;
-    uint4 kr[U], vr[U];
-    auto issue = [&](int t0) {
+    // global -> LDS: load j of a wavefront covers slots inst*64 .. +63 of the tile, slot = row * CPR + position
+    const uint16_t* kb = p.k + b * p.k_sb + kvh * p.k_sh;
+    const uint16_t* vb = p.v + b * p.v_sb + kvh * p.v_sh;
+    auto swz_key = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
+    auto dma = [&](int t0, unsigned char* stage) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int tok = min(t0 + u * ROWS_PER_LOAD + ld_row, p.S - 1);  // rows past the data are masked
-            kr[u] = load16(kbase + int64_t(tok) * p.k_st);
-            vr[u] = load16(vbase + int64_t(tok) * p.v_st);
+        for (int j = 0; j < IPW; ++j) {
+            const int inst = wave * IPW + j;
+            const int slot = inst * kWaveSize + lane;
+            const int row = slot / CPR;
+            const int chunk = (slot % CPR) ^ swz_key(row);
+            const int tok = min(t0 + row, p.S - 1);   // rows past the data are clamped to a valid row and masked
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(kb + int64_t(tok) * p.k_st + chunk * 8),
+                L3_LDS_PTR(void, stage + inst * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(vb + int64_t(tok) * p.v_st + chunk * 8),
+                L3_LDS_PTR(void, stage + KBYTES + inst * 1024), 16, 0, 0);
         }
     };
-    auto stash = [&](unsigned char* stage) {
+    // operand addresses within a stage.  K: lane (fn, fg) reads chunk 4m + fg of row 16 tg + fn, whose
+    // key depends on fn alone.  V (transposing read): lane reads 8 bytes of row 32 ks + 4 fg + (fn >> 2)
+    // (+16) in the 32-byte column block nb, i.e. chunk 2 nb + ((lane & 3) >> 1); the key depends on the
+    // lane alone as well.  One address per m / nb, the rest is instruction offsets.
+    int ak[KC], av[NB];   // byte offsets within a stage
+    {
+        const int kkey = swz_key(fn);
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int row = u * ROWS_PER_LOAD + ld_row;
-            *reinterpret_cast<uint4*>(stage + row * KPITCH + (tid % LPR) * 16) = kr[u];
-            *reinterpret_cast<uint4*>(stage + KBYTES + row * VPITCH + (tid % LPR) * 16) = vr[u];
+        for (int m = 0; m < KC; ++m) ak[m] = fn * ROWB + (((m * 4 + fg) ^ kkey) << 4);
+        const int vrow = 4 * fg + (fn >> 2);
+        const int vkey = swz_key(vrow);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            av[nb] = KBYTES + vrow * ROWB + (((nb * 2 + ((lane & 3) >> 1)) ^ vkey) << 4) + (lane & 1) * 8;
         }
-    };
+    }
 
     f32x4_t O[CB][NB];
     float m_run[CB], l_part[CB];
@@ -141,118 +147,111 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     }
     const float c = p.scale_log2e;
 
-    issue(0);
-    stash(s_tiles);
-    __syncthreads();
-
-    int buf = 0;
-    for (int t0 = 0; t0 < wg_t_end; t0 += TK) {
-        const int tn = t0 + TK;
-        const bool more = tn < wg_t_end;   // workgroup-uniform
-        if (more) issue(tn);
-
-        if (t0 < wave_t_end) {             // wave-uniform: some column of this wavefront sees the tile
-            const unsigned char* stage = s_tiles + buf * STAGE;
-            const unsigned char* rd_k = stage + fn * KPITCH + fg * 16;
-            const unsigned char* rd_v = stage + KBYTES + (4 * fg + (fn >> 2)) * VPITCH + (lane & 3) * 8;
-
-            // ---- S = K Q^T for the CB column blocks
-            f32x4_t S[CB][NG];
+    // One tile on its LDS stage: S = K Q^T, the online softmax of S, O^T += V^T P.
+    auto tile = [&](const unsigned char* stage, int t0) __attribute__((always_inline)) {
+        f32x4_t S[CB][NG];
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
+        for (int tg = 0; tg < NG; ++tg) {
 #pragma unroll
-                for (int tg = 0; tg < NG; ++tg) S[cb][tg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            }
+            for (int m = 0; m < KC; ++m) {
+                const uint4 a = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
 #pragma unroll
-            for (int tg = 0; tg < NG; ++tg) {
-#pragma unroll
-                for (int m = 0; m < KC; ++m) {
-                    const uint4 a = *reinterpret_cast<const uint4*>(rd_k + tg * 16 * KPITCH + m * 64);
-#pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        S[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                                            qfrag[cb][m], S[cb][tg], 0, 0, 0);
-                    }
-                }
-            }
-
-            // ---- causal mask (only tiles that reach past the wavefront's first position) and softmax
-            const bool mask_tile = tn > wave_limit_min;
-            bf16x8_t pfrag[CB][KS];
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-                if (mask_tile) {
-#pragma unroll
-                    for (int tg = 0; tg < NG; ++tg) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            if (t0 + tg * 16 + 4 * fg + j >= col_limit[cb]) S[cb][tg][j] = kMaskedScore;
-                        }
-                    }
-                }
-                float mloc = S[cb][0][0];
-#pragma unroll
-                for (int tg = 0; tg < NG; ++tg) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) mloc = fmaxf(mloc, S[cb][tg][j]);
-                }
-                mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWaveSize));
-                mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWaveSize));
-                if (__builtin_amdgcn_ballot_w64(mloc > m_run[cb]) != 0) {
-                    const float m_new = fmaxf(m_run[cb], mloc);
-                    const float alpha = fast_exp2((m_run[cb] - m_new) * c);
-                    l_part[cb] *= alpha;
-#pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) O[cb][nb] *= alpha;
-                    m_run[cb] = m_new;
-                }
-                const float mc = m_run[cb] * c;
-                float psum = 0.f;
-#pragma unroll
-                for (int tg = 0; tg < NG; ++tg) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float pj = fast_exp2(fmaf(S[cb][tg][j], c, -mc));
-                        S[cb][tg][j] = pj;
-                        psum += pj;
-                    }
-                }
-                l_part[cb] += psum;
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    uint4 pw;
-                    pw.x = pack_bf16x2(S[cb][2 * ks][0], S[cb][2 * ks][1]);
-                    pw.y = pack_bf16x2(S[cb][2 * ks][2], S[cb][2 * ks][3]);
-                    pw.z = pack_bf16x2(S[cb][2 * ks + 1][0], S[cb][2 * ks + 1][1]);
-                    pw.w = pack_bf16x2(S[cb][2 * ks + 1][2], S[cb][2 * ks + 1][3]);
-                    pfrag[cb][ks] = __builtin_bit_cast(bf16x8_t, pw);
-                }
-            }
-
-            // ---- O^T += V^T P; the k slots of a 32-token step pair (fg, i) with token 4*fg + i of the
-            //      step's first 16-token group for i < 4 and of its second group for i >= 4
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        L3_LDS_PTR(s16x4_t, rd_v + (2 * ks) * 16 * VPITCH + nb * 32));
-                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        L3_LDS_PTR(s16x4_t, rd_v + (2 * ks + 1) * 16 * VPITCH + nb * 32));
-                    const s16x8_t vv = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv),
-                                                                            pfrag[cb][ks], O[cb][nb], 0, 0, 0);
-                    }
+                for (int cb = 0; cb < CB; ++cb) {
+                    const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[cb][tg];
+                    S[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[cb][m],
+                                                                        acc, 0, 0, 0);
                 }
             }
         }
 
-        // the other buffer was last read before the previous barrier: refill it, then meet
-        if (more) stash(s_tiles + (buf ^ 1) * STAGE);
+        // causal mask (only tiles that reach past the wavefront's first position) and softmax
+        const bool mask_tile = t0 + TK > wave_limit_min;
+        bf16x8_t pfrag[CB][KS];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            if (mask_tile) {
+#pragma unroll
+                for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (t0 + tg * 16 + 4 * fg + j >= col_limit[cb]) S[cb][tg][j] = kMaskedScore;
+                    }
+                }
+            }
+            float mloc = S[cb][0][0];
+#pragma unroll
+            for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) mloc = fmaxf(mloc, S[cb][tg][j]);
+            }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWaveSize));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWaveSize));
+            if (__builtin_amdgcn_ballot_w64(mloc > m_run[cb]) != 0) {
+                const float m_new = fmaxf(m_run[cb], mloc);
+                const float alpha = fast_exp2((m_run[cb] - m_new) * c);
+                l_part[cb] *= alpha;
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) O[cb][nb] *= alpha;
+                m_run[cb] = m_new;
+            }
+            const float mc = m_run[cb] * c;
+            float psum = 0.f;
+#pragma unroll
+            for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float pj = fast_exp2(fmaf(S[cb][tg][j], c, -mc));
+                    S[cb][tg][j] = pj;
+                    psum += pj;
+                }
+            }
+            l_part[cb] += psum;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                uint4 pw;
+                pw.x = pack_bf16x2(S[cb][2 * ks][0], S[cb][2 * ks][1]);
+                pw.y = pack_bf16x2(S[cb][2 * ks][2], S[cb][2 * ks][3]);
+                pw.z = pack_bf16x2(S[cb][2 * ks + 1][0], S[cb][2 * ks + 1][1]);
+                pw.w = pack_bf16x2(S[cb][2 * ks + 1][2], S[cb][2 * ks + 1][3]);
+                pfrag[cb][ks] = __builtin_bit_cast(bf16x8_t, pw);
+            }
+        }
+
+        // O^T += V^T P; the k slots of a 32-token step pair (fg, i) with token 4*fg + i of the step's first
+        // 16-token group for i < 4 and of its second group for i >= 4
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
+                const s16x8_t vv = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pfrag[cb][ks],
+                                                                        O[cb][nb], 0, 0, 0);
+                }
+            }
+        }
+    };
+    // One barrier per tile: the loads of tile i + 1 are issued before the arithmetic on tile i and land in
+    // the other stage, which was last read before the previous barrier.
+    auto step = [&](auto parity_tag, int t0) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(parity_tag)::value;
+        if (t0 + TK < wg_t_end) dma(t0 + TK, PAR ? s_stage0 : s_stage1);   // workgroup-uniform
+        if (t0 < wave_t_end) tile(PAR ? s_stage1 : s_stage0, t0);          // wave-uniform
+        __builtin_amdgcn_s_waitcnt(0xF70);   // vmcnt(0): this wavefront's part of the next stage has landed
         __syncthreads();
-        buf ^= 1;
+    };
+
+    dma(0, s_stage0);
+    __builtin_amdgcn_s_waitcnt(0xF70);
+    __syncthreads();
+    for (int t0 = 0; t0 < wg_t_end; t0 += 2 * TK) {
+        step(std::integral_constant<int, 0>{}, t0);
+        if (t0 + TK < wg_t_end) step(std::integral_constant<int, 1>{}, t0 + TK);
     }
 
 #pragma unroll
@@ -291,20 +290,16 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
 template <int HD, int CB, int NW>
 __global__ void __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attn_prefill_pipe_kernel(const PrefillParams p) {
-    using T = PrefillTile<HD, CB, NW>;
-    constexpr int TK = T::TK, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
-    // K/V tiles go from global memory straight into LDS (global_load_lds_dwordx4: a wavefront-wide
-    // load lands in 1 KiB of consecutive LDS), so rows cannot be padded; instead the 16-byte chunk c
-    // of token row r sits at chunk position c ^ key(r), which spreads the rows that an operand
-    // read touches together over all banks.
+    constexpr int TK = 64;                      // tokens per K/V tile
+    constexpr int NG = TK / 16, KC = HD / 32, NB = HD / 16, KS = TK / 32;
+    // K/V tiles reach LDS as in the tiled kernel: direct loads, swizzled rows.
     constexpr int CPR = HD / 8;                 // 16-byte chunks per token row
     constexpr int ROWB = HD * 2;                // bytes per token row
     constexpr int KBYTES = TK * ROWB;           // a K tile; a stage is a K tile followed by a V tile
     constexpr int STAGE = 2 * KBYTES;
     constexpr int IPW = CPR / NW;               // wavefront-wide loads per wavefront and tile
     static_assert(CPR % NW == 0, "a tile must divide evenly over the wavefronts");
-    // Two separate arrays, so that the compiler can tell a read of one stage from the load in flight
-    // into the other and does not wait for that load before every LDS read.
+    // (with a single array the compiler waits for the load in flight before every LDS read)
     __shared__ __align__(1024) unsigned char s_stage0[STAGE];
     __shared__ __align__(1024) unsigned char s_stage1[STAGE];
 
@@ -630,27 +625,28 @@ attn_prefill_pipe_kernel(const PrefillParams p) {
     }
 }
 
-template <int HD, int CB, int NW>
-int launch_tiled(const PrefillParams& p, bool pipelined, hipStream_t stream) {
+template <class Kernel>
+int launch_blocks(Kernel kernel, const PrefillParams& p, int waves, int col_blocks, hipStream_t stream) {
     const int R = p.QH / p.KVH;
-    const int wg_pos = NW * CB * (16 / R);
+    const int wg_pos = waves * col_blocks * (16 / R);
     const int wgs_per_head = (p.T + wg_pos - 1) / wg_pos;
     const dim3 grid(unsigned(p.B) * unsigned(p.KVH) * unsigned(wgs_per_head));
-    if (pipelined) {
-        hipLaunchKernelGGL((attn_prefill_pipe_kernel<HD, CB, NW>), grid, dim3(NW * kWaveSize), 0, stream, p);
-    } else {
-        hipLaunchKernelGGL((attn_prefill_tiled_kernel<HD, CB, NW>), grid, dim3(NW * kWaveSize), 0, stream, p);
-    }
+    hipLaunchKernelGGL(kernel, grid, dim3(waves * kWaveSize), 0, stream, p);
     return int(hipGetLastError());
 }
 
 }  // namespace
 
-int prefill_tiled_positions_per_wg(int HD, int R) { return prefill_tiled_waves(HD) * kPrefillTiledColBlocks * (16 / R); }
-
 int launch_attn_prefill_tiled(const PrefillParams& p, int HD, bool pipelined, hipStream_t stream) {
-    if (HD == 64) return launch_tiled<64, kPrefillTiledColBlocks, prefill_tiled_waves(64)>(p, pipelined, stream);
-    return launch_tiled<128, kPrefillTiledColBlocks, prefill_tiled_waves(128)>(p, pipelined, stream);
+    constexpr int CB = kPrefillColBlocks, TW = kPrefillTiledWaves;
+    if (pipelined) {
+        if (HD == 64) return launch_blocks(attn_prefill_pipe_kernel<64, CB, prefill_pipe_waves(64)>, p, prefill_pipe_waves(64), CB, stream);
+        return launch_blocks(attn_prefill_pipe_kernel<128, CB, prefill_pipe_waves(128)>, p, prefill_pipe_waves(128), CB, stream);
+    }
+    // tiles of 64 tokens; four wavefronts per SIMD at head size 64 (four workgroups per compute unit), two
+    // at 128 (two workgroups: a stage pair is 64 KiB)
+    if (HD == 64) return launch_blocks(attn_prefill_tiled_kernel<64, CB, TW, 64, 4>, p, TW, CB, stream);
+    return launch_blocks(attn_prefill_tiled_kernel<128, CB, TW, 64, 2>, p, TW, CB, stream);
 }
 
 }  // namespace l3
