@@ -99,23 +99,38 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         }
     }
 
-    // global -> LDS: load j of a wavefront covers slots inst*64 .. +63 of the tile, slot = row * CPR + position
-    const uint16_t* kb = p.k + b * p.k_sb + kvh * p.k_sh;
-    const uint16_t* vb = p.v + b * p.v_sb + kvh * p.v_sh;
+    // global -> LDS: load j of a wavefront covers slots inst*64 .. +63 of the tile, slot = row * CPR + position.
+    // An address is a scalar tile base plus a 32-bit lane offset that does not change from tile to tile
+    // (token strides are below 2^24 elements); rows past the data are clamped to the last row and masked.
+    const char* kb = reinterpret_cast<const char*>(p.k) + wave_uniform((b * p.k_sb + kvh * p.k_sh) * 2);
+    const char* vb = reinterpret_cast<const char*>(p.v) + wave_uniform((b * p.v_sb + kvh * p.v_sh) * 2);
+    const int64_t k_pitch = wave_uniform(int(p.k_st)) * int64_t(2);   // bytes from a token to the next
+    const int64_t v_pitch = wave_uniform(int(p.v_st)) * int64_t(2);
+    const int wave_u = wave_uniform(wave);
     auto swz_key = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
+    uint32_t krow[IPW], vrow[IPW], chunk16[IPW];
+#pragma unroll
+    for (int j = 0; j < IPW; ++j) {
+        const int slot = (wave_u * IPW + j) * kWaveSize + lane;
+        const int row = slot / CPR;
+        krow[j] = uint32_t(row) * uint32_t(k_pitch);
+        vrow[j] = uint32_t(row) * uint32_t(v_pitch);
+        chunk16[j] = uint32_t((slot % CPR) ^ swz_key(row)) * 16u;
+    }
     auto dma = [&](int t0, unsigned char* stage) {
+        const int last_row = min(p.S - 1 - t0, TK - 1);                  // scalar
+        const char* kt = kb + int64_t(t0) * k_pitch;
+        const char* vt = vb + int64_t(t0) * v_pitch;
+        const uint32_t k_last = uint32_t(last_row) * uint32_t(k_pitch);
+        const uint32_t v_last = uint32_t(last_row) * uint32_t(v_pitch);
 #pragma unroll
         for (int j = 0; j < IPW; ++j) {
-            const int inst = wave * IPW + j;
-            const int slot = inst * kWaveSize + lane;
-            const int row = slot / CPR;
-            const int chunk = (slot % CPR) ^ swz_key(row);
-            const int tok = min(t0 + row, p.S - 1);   // rows past the data are clamped to a valid row and masked
+            const int inst = wave_u * IPW + j;
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(kb + int64_t(tok) * p.k_st + chunk * 8),
+                (const __attribute__((address_space(1))) void*)(kt + (min(krow[j], k_last) + chunk16[j])),
                 L3_LDS_PTR(void, stage + inst * 1024), 16, 0, 0);
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(vb + int64_t(tok) * p.v_st + chunk * 8),
+                (const __attribute__((address_space(1))) void*)(vt + (min(vrow[j], v_last) + chunk16[j])),
                 L3_LDS_PTR(void, stage + KBYTES + inst * 1024), 16, 0, 0);
         }
     };
@@ -136,16 +151,27 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         }
     }
 
-    f32x4_t O[CB][NB];
-    float m_run[CB], l_part[CB];
+    // The softmax denominator rides on the matrix pipe: V^T gets a block of rows that are all ones, so
+    // that L = ones . P accumulates the column sums of P (every entry of L[cb] is the whole column's sum,
+    // over all four k groups) next to O.  The vector pipe, which bounds this kernel at head size 64, is
+    // spared one addition per score; P enters both sums rounded to bf16, so the weights of a column add
+    // up to one exactly.
+    f32x4_t O[CB][NB], L[CB];
+    float m_run[CB];
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
         m_run[cb] = kMaskedScore;
-        l_part[cb] = 0.f;
+        L[cb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) O[cb][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
     const float c = p.scale_log2e;
+    // The running maximum only follows the scores when one of them exceeds it by more than 2^8 (in the
+    // exponent's units): until then the exponentials are taken against the stale maximum -- they stay
+    // below 256, which bf16 and the float32 sums hold as well as values below 1 -- and the accumulators
+    // need no rescaling.  O / L is the same quotient either way.
+    const float slack = 8.0f / c;
+    const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
 
     // One tile on its LDS stage: S = K Q^T, the online softmax of S, O^T += V^T P.
     auto tile = [&](const unsigned char* stage, int t0) __attribute__((always_inline)) {
@@ -184,28 +210,21 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) mloc = fmaxf(mloc, S[cb][tg][j]);
             }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWaveSize));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWaveSize));
-            if (__builtin_amdgcn_ballot_w64(mloc > m_run[cb]) != 0) {
+            mloc = column_max(mloc);
+            if (__builtin_amdgcn_ballot_w64(mloc > m_run[cb] + slack) != 0) {
                 const float m_new = fmaxf(m_run[cb], mloc);
                 const float alpha = fast_exp2((m_run[cb] - m_new) * c);
-                l_part[cb] *= alpha;
+                L[cb] *= alpha;
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) O[cb][nb] *= alpha;
                 m_run[cb] = m_new;
             }
             const float mc = m_run[cb] * c;
-            float psum = 0.f;
 #pragma unroll
             for (int tg = 0; tg < NG; ++tg) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float pj = fast_exp2(fmaf(S[cb][tg][j], c, -mc));
-                    S[cb][tg][j] = pj;
-                    psum += pj;
-                }
+                for (int j = 0; j < 4; ++j) S[cb][tg][j] = fast_exp2(fmaf(S[cb][tg][j], c, -mc));   // masked scores give exactly 0
             }
-            l_part[cb] += psum;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 uint4 pw;
@@ -214,6 +233,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
                 pw.z = pack_bf16x2(S[cb][2 * ks + 1][0], S[cb][2 * ks + 1][1]);
                 pw.w = pack_bf16x2(S[cb][2 * ks + 1][2], S[cb][2 * ks + 1][3]);
                 pfrag[cb][ks] = __builtin_bit_cast(bf16x8_t, pw);
+                L[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pfrag[cb][ks], L[cb], 0, 0, 0);
             }
         }
 
@@ -256,13 +276,10 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
 
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
-        float l = l_part[cb];
-        l += __shfl_xor(l, 16, kWaveSize);
-        l += __shfl_xor(l, 32, kWaveSize);
         if (col_limit[cb] > 0) {
             const int qi = wave_first_qi + cb * ppw + fn / R;
             const int qh = kvh * R + fn % R;
-            const float inv = 1.0f / l;
+            const float inv = 1.0f / L[cb][0];
             uint16_t* orow = p.out + b * p.o_sb + int64_t(qh) * p.o_sh + int64_t(qi) * p.o_st + fg * 4;
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
@@ -346,26 +363,38 @@ attn_prefill_pipe_kernel(const PrefillParams p) {
         }
     }
 
-    // global -> LDS: load j of a wavefront covers slots inst*64 .. +63 of the tile, slot = row * CPR + position
-    const uint16_t* kb = p.k + b * p.k_sb + kvh * p.k_sh;
-    const uint16_t* vb = p.v + b * p.v_sb + kvh * p.v_sh;
+    // global -> LDS, addressed as in the tiled kernel (scalar tile base + loop-invariant lane offset)
+    const char* kb = reinterpret_cast<const char*>(p.k) + wave_uniform((b * p.k_sb + kvh * p.k_sh) * 2);
+    const char* vb = reinterpret_cast<const char*>(p.v) + wave_uniform((b * p.v_sb + kvh * p.v_sh) * 2);
+    const int64_t k_pitch = wave_uniform(int(p.k_st)) * int64_t(2);
+    const int64_t v_pitch = wave_uniform(int(p.v_st)) * int64_t(2);
+    const int wave_u = wave_uniform(wave);
     auto swz_key = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
-    // the stage of iteration `it`: K of tile it, V of tile it - 2 (rows outside the data are clamped
-    // to a valid row and never used)
+    uint32_t krow[IPW], vrow[IPW], chunk16[IPW];
+#pragma unroll
+    for (int j = 0; j < IPW; ++j) {
+        const int slot = (wave_u * IPW + j) * kWaveSize + lane;
+        const int row = slot / CPR;
+        krow[j] = uint32_t(row) * uint32_t(k_pitch);
+        vrow[j] = uint32_t(row) * uint32_t(v_pitch);
+        chunk16[j] = uint32_t((slot % CPR) ^ swz_key(row)) * 16u;
+    }
+    // the stage of iteration `it`: K of tile it, V of tile it - 2 (tiles outside the data are replaced by
+    // valid rows that are never used)
     auto dma = [&](int it, unsigned char* stage) {
+        const int tk = min(it * TK, p.S - 1), tv = min(max(it - 2, 0) * TK, p.S - 1);   // scalar
+        const char* kt = kb + int64_t(tk) * k_pitch;
+        const char* vt = vb + int64_t(tv) * v_pitch;
+        const uint32_t k_last = uint32_t(min(p.S - 1 - tk, TK - 1)) * uint32_t(k_pitch);
+        const uint32_t v_last = uint32_t(min(p.S - 1 - tv, TK - 1)) * uint32_t(v_pitch);
 #pragma unroll
         for (int j = 0; j < IPW; ++j) {
-            const int inst = wave * IPW + j;
-            const int slot = inst * kWaveSize + lane;
-            const int row = slot / CPR;
-            const int chunk = (slot % CPR) ^ swz_key(row);
-            const int tok_k = min(it * TK + row, p.S - 1);
-            const int tok_v = min(max((it - 2) * TK + row, 0), p.S - 1);
+            const int inst = wave_u * IPW + j;
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(kb + int64_t(tok_k) * p.k_st + chunk * 8),
+                (const __attribute__((address_space(1))) void*)(kt + (min(krow[j], k_last) + chunk16[j])),
                 L3_LDS_PTR(void, stage + inst * 1024), 16, 0, 0);
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(vb + int64_t(tok_v) * p.v_st + chunk * 8),
+                (const __attribute__((address_space(1))) void*)(vt + (min(vrow[j], v_last) + chunk16[j])),
                 L3_LDS_PTR(void, stage + KBYTES + inst * 1024), 16, 0, 0);
         }
     };
