@@ -60,15 +60,13 @@ const char* l3_strerror(int code);
  *                            the same thing; the flag exists so that the comparison can be repeated
  *                            (the reference has one kernel and no counterpart of this choice).
  *   L3_ATTN_FLAG_PREFILL_*   prefill: force one form of l3_attn_prefill instead of the choice by
- *                            prompt length -- WAVE (every wavefront streams K/V on its own), TILED
- *                            (a workgroup shares K/V tiles; a tile's three phases run in turn) or
- *                            PIPELINED (the same tiling with the phases of three tiles interleaved).
- * Any other bit gives L3_ERR_FLAGS.
+ *                            prompt length -- WAVE (every wavefront streams K/V on its own) or
+ *                            TILED (a workgroup shares K/V tiles).
+ * Any other bit, or both prefill bits at once, gives L3_ERR_FLAGS.
  */
 #define L3_ATTN_FLAG_KERNEL_FMA 0x1
 #define L3_ATTN_FLAG_PREFILL_WAVE 0x10
 #define L3_ATTN_FLAG_PREFILL_TILED 0x20
-#define L3_ATTN_FLAG_PREFILL_PIPELINED 0x30
 #define L3_ATTN_FLAG_PREFILL_MASK 0x30
 
 /*

@@ -96,7 +96,10 @@ int current_device_cus() {
 namespace {
 // The split-KV kernel a call's flags ask for (the library keeps no such choice between calls).
 int attn_impl_of(int flags) { return (flags & L3_ATTN_FLAG_KERNEL_FMA) ? kAttnImplFma : kAttnImplMfma; }
-bool attn_flags_ok(int flags) { return (flags & ~(L3_ATTN_FLAG_KERNEL_FMA | L3_ATTN_FLAG_PREFILL_MASK)) == 0; }
+bool attn_flags_ok(int flags) {
+    return (flags & ~(L3_ATTN_FLAG_KERNEL_FMA | L3_ATTN_FLAG_PREFILL_MASK)) == 0 &&
+           (flags & L3_ATTN_FLAG_PREFILL_MASK) != L3_ATTN_FLAG_PREFILL_MASK;
+}
 }  // namespace
 
 AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl) {
@@ -389,37 +392,19 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     p.v_sb = v_strides[0]; p.v_sh = v_strides[1]; p.v_st = v_strides[2];
     p.o_sb = out_strides[0]; p.o_sh = out_strides[1]; p.o_st = out_strides[2];
     p.scale_log2e = scale * 1.4426950408889634f;
-    // Which form (graph-timed sweeps over B 1 ... 256, T 16 ... 8192, head ratios 1, 3, 4 and 8; the rule
-    // stays within ~5 % of the best form on all of them):
-    // * a prompt that does not exceed one workgroup of the tiled form per kv head, with few enough
-    //   wavefronts for the device to hold them all at once: independent wavefronts, no barrier;
-    // * otherwise K/V tiles are shared by a workgroup, and the number of 4-wave workgroups decides between
-    //   the two kernels.  Head size 64: the tiled kernel keeps four workgroups on a compute unit that
-    //   cover one another and is 6-25 % faster from three per unit on, and for short prompts whatever
-    //   their number; with fewer, longer ones a wavefront has to overlap its own phases, which the
-    //   pipelined kernel does (B 1, T 2048: 38 against 45 us).  Head size 128: the tiled kernel's finer
-    //   grain (32 instead of 64 positions per workgroup at head ratio 4) shortens the longest workgroup,
-    //   which bounds launches of few workgroups (B 1, T 2048: 62 against 73 us), and fills the device
-    //   sooner when prompts are short; for long prompts in many workgroups the pipelined kernel's 8-wave
-    //   workgroups, which fetch each K/V tile once for twice the columns, win by 1-10 %.
+    // Which form (graph-timed sweeps over B 1 ... 256, T 16 ... 8192, head ratios 1, 3, 4 and 8): a prompt
+    // that does not exceed one workgroup of the tiled form per kv head, with few enough wavefronts for the
+    // device to hold them all at once, runs as independent wavefronts with no barrier (4.2 against 4.8 us
+    // for 16 tokens, 5.6 against 6.9 us for 32 at head size 128); everything else shares K/V tiles.
     int form = flags & L3_ATTN_FLAG_PREFILL_MASK;
     if (form == 0) {
         const int R = QH / KVH;
-        const int wg_pos = prefill_tiled_positions_per_wg(R);
-        const int64_t cus = current_device_cus();
         const int64_t private_waves = int64_t(B) * KVH * ((int64_t(T) * R + 15) / 16);
-        if (T <= wg_pos && private_waves <= 4 * cus) {
-            form = L3_ATTN_FLAG_PREFILL_WAVE;
-        } else {
-            const int64_t wgs = int64_t(B) * KVH * ((T + wg_pos - 1) / wg_pos);
-            const bool pipelined = HD == 64 ? (wgs < 3 * cus && T >= 512) : (wgs > 3 * cus && T >= 2048);
-            form = pipelined ? L3_ATTN_FLAG_PREFILL_PIPELINED : L3_ATTN_FLAG_PREFILL_TILED;
-        }
+        const bool tiny = T <= prefill_tiled_positions_per_wg(R) && private_waves <= 4 * int64_t(current_device_cus());
+        form = tiny ? L3_ATTN_FLAG_PREFILL_WAVE : L3_ATTN_FLAG_PREFILL_TILED;
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int rc = (form == L3_ATTN_FLAG_PREFILL_WAVE)
-                       ? launch_attn_prefill(p, HD, st)
-                       : launch_attn_prefill_tiled(p, HD, form == L3_ATTN_FLAG_PREFILL_PIPELINED, st);
+    const int rc = (form == L3_ATTN_FLAG_PREFILL_WAVE) ? launch_attn_prefill(p, HD, st) : launch_attn_prefill_tiled(p, HD, st);
     return rc == 0 ? L3_OK : L3_ERR_HIP;
 }
 

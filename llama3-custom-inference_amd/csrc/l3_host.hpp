@@ -114,15 +114,12 @@ int launch_linear_splitk_finish(const float* part, int ksplit, const uint16_t* r
                                 int64_t y_stride, hipStream_t stream);
 int launch_linear_skinny(LinearParams p, bool swiglu, int num_cus, hipStream_t stream);
 int launch_attn_prefill(const PrefillParams& p, int HD, hipStream_t stream);        // a wavefront per column group
-// Workgroups of the two prefill kernels that share K/V tiles: 16-column blocks per wavefront, and
-// wavefronts per workgroup.  The tiled kernel uses 4-wave workgroups, several per compute unit; the
-// pipelined one 4 at head size 64 (two per unit) and 8 at 128, where the K/V tiles are twice as large
-// and one workgroup that fetches them once for twice the columns is faster.
+// Workgroups of the tiled prefill kernel: 16-column blocks per wavefront, wavefronts per workgroup
+// (small workgroups, several per compute unit).
 constexpr int kPrefillColBlocks = 2;
 constexpr int kPrefillTiledWaves = 4;
-constexpr int prefill_pipe_waves(int HD) { return HD == 64 ? 4 : 8; }
 constexpr int prefill_tiled_positions_per_wg(int R) { return kPrefillTiledWaves * kPrefillColBlocks * (16 / R); }
-int launch_attn_prefill_tiled(const PrefillParams& p, int HD, bool pipelined, hipStream_t stream);  // K/V tiles shared by a workgroup
+int launch_attn_prefill_tiled(const PrefillParams& p, int HD, hipStream_t stream);  // K/V tiles shared by a workgroup
 int launch_attn_splitkv_fma(const AttnParams& p, int HD, int R, hipStream_t stream);
 int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipStream_t stream);
 int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream);

@@ -29,7 +29,6 @@ L3_LINEAR_STAGE_ELEMS = 24576   # activations (rows padded by 8) the fused input
 L3_ATTN_FLAG_KERNEL_FMA = 0x1
 L3_ATTN_FLAG_PREFILL_WAVE = 0x10
 L3_ATTN_FLAG_PREFILL_TILED = 0x20
-L3_ATTN_FLAG_PREFILL_PIPELINED = 0x30
 L3_ATTN_FLAG_PREFILL_MASK = 0x30
 
 # name -> (restype, argtypes); mirrors include/l3_kernels.h line by line

@@ -97,13 +97,13 @@ def _workspace(device, stream_ptr: int, nbytes: int):
 _attn_flags = contextvars.ContextVar("l3_attn_flags", default=0)
 
 _FLAG_NAMES = {"mfma": 0, "fma": _l3lib.L3_ATTN_FLAG_KERNEL_FMA, "auto": 0, "wave": _l3lib.L3_ATTN_FLAG_PREFILL_WAVE,
-               "tiled": _l3lib.L3_ATTN_FLAG_PREFILL_TILED, "pipelined": _l3lib.L3_ATTN_FLAG_PREFILL_PIPELINED}
+               "tiled": _l3lib.L3_ATTN_FLAG_PREFILL_TILED}
 
 
 @contextlib.contextmanager
 def attention_flags(kernel: str = "mfma", prefill: str = "auto"):
     """Within the block, attention calls of this thread that pass no ``flags`` use the named
-    split-KV kernel ("mfma" / "fma") and prefill form ("auto" / "wave" / "tiled" / "pipelined").
+    split-KV kernel ("mfma" / "fma") and prefill form ("auto" / "wave" / "tiled").
     For measurements and tests; the defaults are the library's own choices."""
     token = _attn_flags.set(_FLAG_NAMES[kernel] | _FLAG_NAMES[prefill])
     try:

@@ -223,6 +223,7 @@ def test_prefill_argument_checks():
                                    q_strides, 0.125, flags, None)
 
     assert call(flags=0x40) == _l3lib.L3_ERR_FLAGS
+    assert call(flags=0x30) == _l3lib.L3_ERR_FLAGS          # both prefill bits: no such form
     assert call(out=None) == _l3lib.L3_ERR_NULL_POINTER
     assert call(HD=96) == _l3lib.L3_ERR_HEAD_SIZE
     assert call(QH=40) == _l3lib.L3_ERR_HEAD_RATIO      # ratio 5

@@ -79,7 +79,7 @@ def _draw_prefill_cases(n, seed):
         B = int(rng.integers(1, 4))
         T = int(rng.choice((int(rng.integers(2, 40)), int(rng.integers(40, 300)), int(rng.integers(300, 700)))))
         past = int(rng.choice((0, 0, 1, 50, 130)))          # tokens already in the cache
-        form = str(rng.choice(("auto", "wave", "tiled", "pipelined")))
+        form = str(rng.choice(("auto", "wave", "tiled")))
         cases.append((i, B, R * KVH, KVH, T, T + past, HD, form))
     return cases
 
