@@ -413,6 +413,27 @@ def test_prefill_against_oracle(gpu, prefill_form, HD, B, QH, KVH, T, S):
     assert_attn_close(out, ref, what=f"prefill T={T} S={S} HD={HD}")
 
 
+@pytest.mark.parametrize("HD", [64, 128])
+@pytest.mark.parametrize("gain", [3.0, 8.0])
+def test_prefill_wide_score_range(gpu, prefill_form, HD, gain):
+    """Scores spread over tens of powers of two (queries scaled up), and one key that dominates every
+    query from token 700 on: the running maximum moves both by less and by more than the tiled kernel's
+    2^8 rescaling slack, early and late in a row."""
+    from custom_kernels import custom_kernels_extension as cke
+    from oracle import attention_prefill_ref
+
+    B, QH, KVH, T = 1, 8, 2, 900
+    print(f"prefill wide range form={prefill_form} HD={HD} gain={gain}", flush=True)
+    q = (randn_bf16((B, T, QH, HD), 91).float() * gain).to(torch.bfloat16)
+    k = randn_bf16((B, T, KVH, HD), 92)
+    v = randn_bf16((B, T, KVH, HD), 93)
+    k[0, 700, 1] = (q[0, 800, 5].float() / gain * 2.0).to(torch.bfloat16)   # aligned with one query, large for all of its group
+    out = cke.flash_attention_prefill(q.to(gpu).transpose(1, 2), k.to(gpu).transpose(1, 2), v.to(gpu).transpose(1, 2))
+    torch.cuda.synchronize()
+    ref = attention_prefill_ref(t2f32(q.transpose(1, 2)), t2f32(k.transpose(1, 2)), t2f32(v.transpose(1, 2)))
+    assert_attn_close(out, ref, what=f"prefill wide range HD={HD} gain={gain}")
+
+
 def test_prefill_forms_agree_on_a_long_prompt(gpu):
     """2048 tokens (the auto choice is the tiled form): the tiled and the wavefront-private form against
     each other, and sampled rows against the float64 oracle."""
