@@ -39,7 +39,8 @@ enum {
     L3_ERR_SPLITS = -8,         /* num_splits negative or above L3_ATTN_MAX_SPLITS */
     L3_ERR_HIP = -9,            /* the HIP runtime reported an error at launch */
     L3_ERR_FLAGS = -10,         /* bits set in `flags` that this version does not define */
-    L3_ERR_SCRATCH = -11        /* l3_attn_decode_static: the problem needs more than L3_ATTN_STATIC_SCRATCH_BYTES */
+    L3_ERR_SCRATCH = -11,       /* l3_attn_decode_static: the problem needs more than L3_ATTN_STATIC_SCRATCH_BYTES */
+    L3_ERR_SCALE = -12          /* attention: the softmax scale is not a positive finite number */
 };
 
 #define L3_ATTN_MAX_SPLITS 512
@@ -99,7 +100,8 @@ size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int
  *            Token rows must start on 16-byte boundaries (base pointers 16-byte aligned,
  *            strides multiples of 8, token stride below 2^24 elements).  q and out need
  *            16-byte aligned rows as well.
- *   scale  : softmax scale; the reference uses 1/sqrt(HD) (custom_kernels.cu:253)
+ *   scale  : softmax scale, positive and finite (L3_ERR_SCALE otherwise); the reference uses
+ *            1/sqrt(HD) (custom_kernels.cu:253)
  *   num_splits : 0 = automatic, otherwise 1..L3_ATTN_MAX_SPLITS (the kernel may use fewer
  *            when S is short); results do not depend on it beyond float32 rounding
  *   workspace : >= l3_attn_decode_workspace_bytes(...) bytes, 256-byte aligned; may be NULL

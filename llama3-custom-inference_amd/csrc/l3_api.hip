@@ -21,6 +21,8 @@ constexpr int kVersion = 100;  // 0.1.0
 constexpr size_t kWorkspaceAlign = 256;
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+// The kernels track the maximum of the raw scores and scale it afterwards, which needs a positive scale.
+bool scale_ok(float scale) { return scale > 0.0f && scale <= 3.0e38f; }
 
 bool ratio_supported(int R) { return R == 1 || R == 2 || R == 3 || R == 4 || R == 8; }
 
@@ -216,6 +218,7 @@ const char* l3_strerror(int code) {
         case L3_ERR_HIP: return "HIP runtime error at kernel launch";
         case L3_ERR_FLAGS: return "unknown bits in flags";
         case L3_ERR_SCRATCH: return "problem needs more scratch than the static device buffer holds";
+        case L3_ERR_SCALE: return "softmax scale must be positive and finite";
         default: return "unknown error code";
     }
 }
@@ -304,6 +307,7 @@ int attn_decode_impl(const void* q, const void* k, const void* v, void* out, voi
                                  num_splits, true); rc != L3_OK)
         return rc;
     if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
+    if (!scale_ok(scale)) return L3_ERR_SCALE;
     const int impl = attn_impl_of(flags);
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
     const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
@@ -369,6 +373,7 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
         return L3_ERR_NULL_POINTER;
     if (int rc = check_attn_shape(B, QH, KVH, S, HD); rc != L3_OK) return rc;
     if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
+    if (!scale_ok(scale)) return L3_ERR_SCALE;
     if (T <= 0 || T > S) return L3_ERR_SHAPE;
     if (int64_t(B) * KVH * ((int64_t(T) + 1) / 2 + kMfmaWaves) >= (int64_t(1) << 31)) return L3_ERR_SHAPE;  // grid
     const int q_dims[3] = {B, QH, T};
@@ -418,6 +423,7 @@ int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, fl
         return rc;
     if (!aligned(part_o, 16) || !aligned(part_ml, 8)) return L3_ERR_ALIGNMENT;
     if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
+    if (!scale_ok(scale)) return L3_ERR_SCALE;
     const int impl = attn_impl_of(flags);
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
     const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);

@@ -21,6 +21,7 @@ L3_ERR_SPLITS = -8
 L3_ERR_HIP = -9
 L3_ERR_FLAGS = -10
 L3_ERR_SCRATCH = -11
+L3_ERR_SCALE = -12
 L3_ATTN_MAX_SPLITS = 512
 L3_ATTN_STATIC_SCRATCH_BYTES = 16 << 20
 L3_LINEAR_MAX_ROWS = 16         # one launch, any matrix shape, optional input norm / SwiGLU / residual / rope epilogue

@@ -81,10 +81,10 @@ def test_error_codes_match_header():
 
 
 def _attn(q=FAKE, k=FAKE, v=FAKE, out=FAKE, ws=None, ws_bytes=0, B=1, QH=32, KVH=8, S=256, HD=64,
-          qs=(2048, 64), ks=(131072, 64, 512), vs=(131072, 64, 512), os_=(2048, 64), splits=1, flags=0):
+          qs=(2048, 64), ks=(131072, 64, 512), vs=(131072, 64, 512), os_=(2048, 64), splits=1, flags=0, scale=0.125):
     return _l3lib.load().l3_attn_decode(q, k, v, out, ws, ws_bytes, B, QH, KVH, S, HD, _l3lib.i64_array(qs),
                                         _l3lib.i64_array(ks), _l3lib.i64_array(vs), _l3lib.i64_array(os_),
-                                        0.125, splits, flags, None)
+                                        scale, splits, flags, None)
 
 
 def test_attention_argument_checks_run_before_any_launch():
@@ -104,6 +104,8 @@ def test_attention_argument_checks_run_before_any_launch():
     assert _attn(k=FAKE + 2) == _l3lib.L3_ERR_ALIGNMENT
     assert _attn(flags=0x100) == _l3lib.L3_ERR_FLAGS
     assert _attn(flags=-1) == _l3lib.L3_ERR_FLAGS
+    for bad in (0.0, -0.125, float("nan"), float("inf")):     # the kernels scale a maximum of raw scores
+        assert _attn(scale=bad) == _l3lib.L3_ERR_SCALE
     assert _attn(S=1024, ks=(524288, 64, 512), vs=(524288, 64, 512), splits=4) == _l3lib.L3_ERR_WORKSPACE
     assert _attn(S=1024, ks=(524288, 64, 512), vs=(524288, 64, 512), splits=4, ws=FAKE, ws_bytes=16) \
         == _l3lib.L3_ERR_WORKSPACE
@@ -218,9 +220,11 @@ def test_prefill_argument_checks():
     lib = _l3lib.load()
     qs, ks = _l3lib.i64_array((131072, 64, 2048)), _l3lib.i64_array((131072, 64, 512))
 
-    def call(q=FAKE, out=FAKE, B=1, QH=32, KVH=8, T=16, S=64, HD=64, q_strides=qs, k_strides=ks, flags=0):
+    def call(q=FAKE, out=FAKE, B=1, QH=32, KVH=8, T=16, S=64, HD=64, q_strides=qs, k_strides=ks, flags=0, scale=0.125):
         return lib.l3_attn_prefill(q, FAKE, FAKE, out, B, QH, KVH, T, S, HD, q_strides, k_strides, k_strides,
-                                   q_strides, 0.125, flags, None)
+                                   q_strides, scale, flags, None)
+
+    assert call(scale=0.0) == _l3lib.L3_ERR_SCALE
 
     assert call(flags=0x40) == _l3lib.L3_ERR_FLAGS
     assert call(flags=0x30) == _l3lib.L3_ERR_FLAGS          # both prefill bits: no such form
