@@ -17,7 +17,8 @@ carries the read bandwidth a pure stream reaches on the same device; "cpu_baseli
 PyTorch on the host cores for a bounded sample of the same sweep.  The same line carries the rest
 of the target ("north_star": head_dim 64, the batched shapes, longer KV lengths, RMSNorm, rotary
 embedding, each cold; beside every attention shape torch's own attention on the same GPU and the
-time a kernel that only reads takes for the same bytes) and the end-to-end tokens/s ("e2e").
+time a kernel that only reads takes for the same bytes), the causal prefill kernel on three prompt
+shapes against the MFMA peak ("prefill") and the end-to-end tokens/s ("e2e").
 
 Other workloads (--workload c1|c3a|c3b|hd64|rms|rope|prefill|linear|e2e|copy|readstream) report the
 remaining configurations in the same format.
@@ -535,6 +536,43 @@ def run_rows(args, torch, lib, l3, dev, name):
     }
 
 
+def prefill_summary(torch, dev):
+    """The causal prefill kernel in short form, for the default line: the library's own choice of form on
+    the 1B and 8B prompt shapes and a long prompt, against the dense bf16 MFMA peak with the causal flop
+    count; torch's scaled_dot_product_attention on the same tensors beside it (--workload prefill has
+    every form)."""
+    import torch.nn.functional as F
+    from custom_kernels import custom_kernels_extension as cke
+
+    out = []
+    for (B, QH, KVH, T, HD) in [(2, 32, 8, 2048, 64), (1, 32, 8, 2048, 128), (1, 32, 8, 8192, 128)]:
+        g = torch.Generator().manual_seed(SEED)
+        q = torch.randn((B, T, QH, HD), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+        k = torch.randn((B, T, KVH, HD), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+        v = torch.randn((B, T, KVH, HD), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+        flops = 4.0 * B * QH * HD * (T * (T + 1) / 2)
+        reps = 8
+        cke.flash_attention_prefill(q, k, v)
+        gph = capture_graph(torch, lambda: [cke.flash_attention_prefill(q, k, v) for _ in range(reps)])
+        t_warm = time.perf_counter()    # untimed: after an idle spell the first milliseconds run at lower clocks
+        while time.perf_counter() - t_warm < 0.03:
+            gph.replay()
+            torch.cuda.synchronize()
+        ms = event_time_ms(torch, gph.replay, 5) / reps
+        del gph
+        try:
+            F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+            sd_us = round(1e3 * event_time_ms(torch, lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True,
+                                                                                            enable_gqa=True), 10), 2)
+        except Exception as exc:  # informational only
+            sd_us = None
+            print(f"bench.py: torch SDPA failed for {B, QH, KVH, T, HD}: {exc}", file=sys.stderr)
+        out.append({"B": B, "QH": QH, "KVH": KVH, "T": T, "HD": HD, "us": round(ms * 1e3, 2),
+                    "TFLOPs": round(flops / ms / 1e9, 1), "frac_of_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4),
+                    "torch_sdpa_us": sd_us})
+    return out
+
+
 def run_prefill(args, torch, lib, l3, dev):
     """Causal prefill attention (T query tokens against T cached tokens).  Compute-bound: priced
     against the dense bf16 MFMA peak with the causal flop count 4*HD per (query, attended token)
@@ -817,6 +855,8 @@ def main():
             ns["points"] = len(pts)
             ns["longer_kv_points_at_or_above_target"] = sum(r["frac"] >= target for r in ns["longer_kv_b1"])
             line["north_star"] = ns
+            # the next row after the hot path: causal prefill attention (compute-bound, against the MFMA peak)
+            line["prefill"] = prefill_summary(torch, dev)
         del pool
         torch.cuda.empty_cache()
         if not args.no_e2e:
