@@ -334,7 +334,8 @@ int attn_decode_impl(const void* q, const void* k, const void* v, void* out, voi
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     int err = launch_split_stage(p, HD, QH / KVH, impl, plan.coop, st);
-    if (err == 0 && plan.num_splits > 1) err = launch_attn_combine(p, HD, st);
+    const int groups = (impl == kAttnImplMfma && !plan.coop && B <= 65535) ? KVH / attn_mfma_heads_per_wg(KVH) : 0;
+    if (err == 0 && plan.num_splits > 1) err = launch_attn_combine(p, HD, groups, st);
     return err == 0 ? L3_OK : L3_ERR_HIP;
 }
 }  // namespace
@@ -453,7 +454,7 @@ int l3_attn_combine(const float* part_o, const float* part_ml, void* out, int B,
     p.B = B; p.QH = QH;
     p.num_splits = n;
     p.o_sb = out_strides[0]; p.o_sh = out_strides[1];
-    return launch_attn_combine(p, HD, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+    return launch_attn_combine(p, HD, 0, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 
 int l3_rms_norm(const void* x, const void* w, void* y, int64_t rows, int C, float eps, void* stream) {

@@ -122,7 +122,9 @@ constexpr int prefill_tiled_positions_per_wg(int R) { return kPrefillTiledWaves 
 int launch_attn_prefill_tiled(const PrefillParams& p, int HD, hipStream_t stream);  // K/V tiles shared by a workgroup
 int launch_attn_splitkv_fma(const AttnParams& p, int HD, int R, hipStream_t stream);
 int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipStream_t stream);
-int launch_attn_combine(const AttnParams& p, int HD, hipStream_t stream);
+// producer_groups: head groups per batch entry of the streaming MFMA split kernel that wrote the partials (its
+// grid's x extent), 0 when another kernel or a caller produced them
+int launch_attn_combine(const AttnParams& p, int HD, int producer_groups, hipStream_t stream);
 int launch_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups, hipStream_t stream);
 int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
                     bool vec_ok, hipStream_t stream);

@@ -48,11 +48,15 @@ def test_head_ratios(gpu, HD, QH, KVH, splits):
 @pytest.mark.parametrize("B,QH,KVH,S,HD,splits", [(40, 32, 8, 300, 64, 2), (40, 32, 8, 300, 128, 3),
                                                    (130, 8, 8, 97, 64, 2), (33, 32, 4, 1000, 128, 31),
                                                    (515, 2, 2, 70, 64, 2), (36, 32, 8, 2100, 128, 32),
-                                                   (100, 32, 8, 1024, 128, 0)])
+                                                   (100, 32, 8, 1024, 128, 0),
+                                                   (4, 64, 16, 500, 64, 3), (2, 32, 32, 300, 128, 2),
+                                                   (16, 16, 4, 400, 64, 5), (8, 24, 8, 350, 128, 4)])
 def test_many_sequences_with_few_splits(gpu, attn_kernel, B, QH, KVH, S, HD, splits):
     """A thousand or more (batch, query head) pairs with 2 ... 32 splits each: the combine runs with a
-    wavefront per pair (515 x 2 pairs do not fill its last workgroup); the last case takes the plan's
-    own choice for 100 long sequences (two splits with the MFMA kernel)."""
+    wavefront per pair (515 x 2 pairs do not fill its last workgroup); the case with 0 splits takes the plan's
+    own choice for 100 long sequences (two splits with the MFMA kernel); the last four (and the first two)
+    have (head groups x batch) a multiple of 8, where the combine deals its pairs to the XCD whose split
+    workgroups wrote them: one, two and four head groups of eight kv heads, four kv heads, head ratio 3."""
     if splits == 0:
         from custom_kernels import custom_kernels_extension as cke
         assert cke.attention_num_splits(B, KVH, S, HD, 256) == (2 if attn_kernel == "mfma" else 1)
