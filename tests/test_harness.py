@@ -157,6 +157,25 @@ def test_graphed_decode_loop_matches_eager(gpu, batch):
                     assert torch.equal(got, want), f"prompt pass T={T} seed={seed}"
 
 
+def test_prompt_pass_falls_back_to_eager_when_its_recording_fails_the_check(gpu, monkeypatch):
+    """A recorded prompt pass that does not reproduce the eager logits must not be used: with the
+    comparison forced to fail, generate_graphed keeps the eager pass and still matches generate()."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    cfg = tiny_config(n_head=8, n_kv_head=2, n_embd=512, max_gen_batch_size=4, max_model_len=64)
+    m = la.LlamaDecoder(cfg, cke, gpu, seed=5)
+    m.tokenizer.pad_id, m.tokenizer.stop_tokens = 999, (998,)
+    prompts = la.random_prompts(2, 9, 900, 4, exclude=())
+    eager = m.generate(prompts, max_gen_len=12, ignore_eos=True)
+    monkeypatch.setattr(torch, "equal", lambda a, b: False)
+    graphed = m.generate_graphed(prompts, max_gen_len=12, ignore_eos=True)
+    torch.cuda.synchronize()
+    monkeypatch.undo()
+    assert m.prefill_pass_mode() == "eager"
+    for a, b in zip(eager, graphed):
+        assert a[:8] == b[:8], f"streams diverge early: {a} vs {b}"
+
+
 # ---- the end-to-end configuration at its own size (Llama-3.2-1B architecture, model.py:153-166;
 #      benchmark_model.py:69-85 drives it with 128 prompt ids and 128 generated tokens)
 @pytest.fixture(scope="module")
