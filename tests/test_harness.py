@@ -157,6 +157,7 @@ def test_graphed_decode_loop_matches_eager(gpu, batch):
                     assert torch.equal(got, want), f"prompt pass T={T} seed={seed}"
 
 
+@pytest.mark.gpu
 def test_prompt_pass_falls_back_to_eager_when_its_recording_fails_the_check(gpu, monkeypatch):
     """A recorded prompt pass that does not reproduce the eager logits must not be used: with the
     comparison forced to fail, generate_graphed keeps the eager pass and still matches generate()."""
