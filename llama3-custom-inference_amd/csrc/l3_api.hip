@@ -120,7 +120,11 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
         const int64_t units = int64_t(B) * KVH;
         if (units <= 2 * int64_t(num_cus)) {
             const int wgs = int(std::max<int64_t>(1, num_cus / units));   // workgroups a head can have, one per unit
-            if (tiles <= kMfmaWaves || (tiles <= 2 * kMfmaWaves && wgs < 2)) {
+            // (Head size 64 with at least four workgroups to spare per head: up to six tiles only; its wavefronts
+            // work through half tiles one after the other, 4.1 us at 256 tokens but 5.6 / 6.0 us at 448 / 512,
+            // where four splits and a combine take 5.4 us.)
+            const int one_launch_tiles = (HD == 64 && wgs >= 4) ? 6 : kMfmaWaves;
+            if (tiles <= one_launch_tiles || (tiles <= 2 * kMfmaWaves && wgs < 2)) {
                 plan.coop = true;
                 plan.num_splits = 1;
                 plan.tokens_per_split = tiles * tile;

@@ -154,6 +154,8 @@ def test_split_planning():
     assert plan(3, 32768, 128) == 64            # four fifths of the units (68 groups of 3 workgroups at most), whole tiles: 64 x 512 tokens
     assert plan(1, 32768, 128) == 205 and plan(1, 16384, 128) == 171   # 5 and 3 tiles per wavefront
     assert plan(1, 12288, 128) == 32 and plan(1, 8192, 64) == 32       # cooperative form: one workgroup per unit
+    assert plan(1, 256, 64) == 1 and plan(1, 384, 64) == 1 and plan(1, 448, 64) == 4 and plan(1, 512, 64) == 4   # one launch up to six tiles
+    assert plan(1, 256, 128) == 1 and plan(1, 512, 128) == 8
     assert plan(4, 4096, 64) == 64              # few sequences: one workgroup per unit
     assert plan(16, 4096, 64) == 11             # from 8 sequences on, three quarters of the units: 12 groups, whole tiles
     assert plan(48, 4096, 128) == 4
