@@ -169,6 +169,16 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
                 groups = 1;   // a quarter of the units busy, but no partials and no second launch
             } else if (groups == 1 && !short_stream && int64_t(num_cus) / wgs_per_split_group >= 2) {
                 groups = 2;
+            } else if (groups > 1) {
+                // Splits are whole tiles: with few tiles the rounding can halve the workgroup count (16 tiles
+                // over 12 groups become 8 groups of two).  Shorter splits then, down to one tile, until
+                // three fifths of the units are busy (B 16 x 1024 tokens at head size 64: 11.0 -> 8.9 us).
+                int64_t split_tiles = ceil_div(tiles, int(std::min<int64_t>(groups * spg, tiles)));
+                while (split_tiles > 1 &&
+                       ceil_div(ceil_div(tiles, int(split_tiles)), spg) * wgs_per_split_group * 5 < int64_t(num_cus) * 3) {
+                    --split_tiles;
+                }
+                groups = ceil_div(ceil_div(tiles, int(split_tiles)), spg);
             }
         } else {
             // Few workgroups per split group (batch 1 of a long sequence): four fifths of the units, each

@@ -158,6 +158,8 @@ def test_split_planning():
     assert plan(1, 256, 128) == 1 and plan(1, 512, 128) == 8
     assert plan(4, 4096, 64) == 64              # few sequences: one workgroup per unit
     assert plan(16, 4096, 64) == 11             # from 8 sequences on, three quarters of the units: 12 groups, whole tiles
+    assert plan(16, 1024, 64) == 16             # 16 tiles over 12 groups would round to 8 splits, half the units: one tile each instead
+    assert plan(8, 2048, 64) == 32
     assert plan(48, 4096, 128) == 4
     assert plan(64, 4096, 128) == 3
     assert plan(96, 2048, 64) == 2
