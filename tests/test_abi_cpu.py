@@ -129,6 +129,32 @@ def test_rms_norm_and_rot_embed_argument_checks():
     assert lib.l3_rot_embed(FAKE + 2, FAKE, FAKE, 1, 5, 32, 64, st, None) == _l3lib.L3_ERR_ALIGNMENT
 
 
+def test_split_plan_invariants_over_random_shapes():
+    """Whatever the shape, the device size or the kernel: between one split and one per tile, never above the
+    limit, the same answer twice, and a workspace that holds exactly the partial rows of that many splits."""
+    import random
+
+    lib = _l3lib.load()
+    rng = random.Random(7)
+    fma = _l3lib.L3_ATTN_FLAG_KERNEL_FMA
+    for _ in range(3000):
+        HD = rng.choice((64, 128))
+        KVH = rng.choice((1, 2, 3, 4, 8, 16, 32))
+        R = rng.choice((1, 2, 3, 4, 8))
+        B = rng.choice((1, 1, 2, 3, 7, 8, 16, 33, 64, 100, 256, 1000))
+        S = rng.choice((1, 31, 64, 100, 256, 257, 448, 512, 1000, 4096, 5000, 16384, 32768, 100000, 131072))
+        cus = rng.choice((64, 104, 256, 304))
+        flags = rng.choice((0, 0, 0, fma))
+        n = lib.l3_attn_choose_splits(B, KVH, S, HD, cus, flags)
+        what = f"B={B} KVH={KVH} S={S} HD={HD} cus={cus} flags={flags}: {n}"
+        assert 1 <= n <= _l3lib.L3_ATTN_MAX_SPLITS, what
+        assert n <= max(1, -(-S // 16)), what                      # no kernel's tile is shorter than 16 tokens
+        assert n == lib.l3_attn_choose_splits(B, KVH, S, HD, cus, flags), what
+        ws = lib.l3_attn_decode_workspace_bytes(B, KVH * R, KVH, S, HD, n, flags)
+        rows = B * KVH * R * n
+        assert (ws == 0 if n == 1 else rows * (HD + 2) * 4 <= ws <= rows * (HD + 2) * 4 + 512), what
+
+
 def test_split_planning():
     lib = _l3lib.load()
     for HD, tile in ((64, 64), (128, 32)):
