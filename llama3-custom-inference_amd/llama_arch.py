@@ -445,6 +445,8 @@ class GraphedDecodeLoop:
         self.pos += 1
         self.kv_len += 1
 
+    MAX_PREFILL_GRAPHS = 4
+
     def prefill(self, m: "LlamaDecoder", T: int):
         """Logits of the prompt's first T positions (model.py:365 with start_pos 0) for the tokens in
         self.tokens.  The eager pass costs ~260 launches from Python (3.3 ms at batch 1, against 0.64 ms
@@ -455,6 +457,10 @@ class GraphedDecodeLoop:
 
         entry = self.prefill_graphs.get(T)
         if entry is None:
+            # a recording keeps its activations' memory for as long as it lives: only the last few prompt
+            # lengths stay recorded
+            while len(self.prefill_graphs) >= self.MAX_PREFILL_GRAPHS:
+                self.prefill_graphs.pop(next(iter(self.prefill_graphs)))
             dev = m.device
             ref = m.forward(self.tokens[:, :T], start_pos=0).clone()   # eager: also the warm-up for the capture
             torch.cuda.synchronize(dev)

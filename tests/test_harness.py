@@ -146,6 +146,7 @@ def test_graphed_decode_loop_matches_eager(gpu, batch):
     # failed its own check), new prompts through it give the eager pass's logits, replay after replay
     assert m.prefill_pass_mode() in ("recorded", "eager")
     print(f"prompt pass: {m.prefill_pass_mode()}", flush=True)
+    assert all(len(loop.prefill_graphs) <= loop.MAX_PREFILL_GRAPHS for loop in m._graphs.values())
     with torch.inference_mode():
         for loop in m._graphs.values():
             for T in list(loop.prefill_graphs):
@@ -155,6 +156,27 @@ def test_graphed_decode_loop_matches_eager(gpu, batch):
                     got = loop.prefill(m, T).clone()
                     want = m.forward(loop.tokens[:, :T], start_pos=0)
                     assert torch.equal(got, want), f"prompt pass T={T} seed={seed}"
+
+
+@pytest.mark.gpu
+def test_only_the_last_few_prompt_lengths_stay_recorded(gpu):
+    """Six prompt lengths on one decode loop (same batch, same total length): every generation matches the
+    eager one, and the loop holds no more recorded prompt passes than its limit."""
+    from custom_kernels import custom_kernels_extension as cke
+
+    cfg = tiny_config(n_head=8, n_kv_head=2, n_embd=512, max_gen_batch_size=2, max_model_len=64)
+    m = la.LlamaDecoder(cfg, cke, gpu, seed=6)
+    m.tokenizer.pad_id, m.tokenizer.stop_tokens = 999, (998,)
+    for n in range(5, 11):
+        prompts = la.random_prompts(1, n, 900, n, exclude=())
+        print(f"prompt length {n}", flush=True)
+        eager = m.generate(prompts, max_gen_len=30 - n, ignore_eos=True)
+        graphed = m.generate_graphed(prompts, max_gen_len=30 - n, ignore_eos=True)
+        torch.cuda.synchronize()
+        assert eager[0][:8] == graphed[0][:8], f"streams diverge early: {eager[0]} vs {graphed[0]}"
+    assert len(m._graphs) == 1
+    loop = next(iter(m._graphs.values()))
+    assert len(loop.prefill_graphs) == loop.MAX_PREFILL_GRAPHS and 10 in loop.prefill_graphs and 5 not in loop.prefill_graphs
 
 
 @pytest.mark.gpu
