@@ -62,6 +62,8 @@ class _Tokenizer:
 
 
 class LlamaDecoder:
+    MAX_DECODE_LOOPS = 8    # (batch, total length) pairs whose recorded decode loops are kept
+
     def __init__(self, config: LlamaConfig, ops, device, dtype=torch.bfloat16, seed: int = 42, weights_from=None):
         """`weights_from`: another LlamaDecoder of the same configuration whose weights are copied
         (to this device) instead of being drawn again from the seed."""
@@ -274,6 +276,8 @@ class LlamaDecoder:
         key = (bsz, total_len)
         loop = self._graphs.get(key)
         if loop is None:
+            while len(self._graphs) >= self.MAX_DECODE_LOOPS:      # recorded loops hold device memory
+                self._graphs.pop(next(iter(self._graphs)))
             loop = GraphedDecodeLoop(self, bsz, total_len)
             self._graphs[key] = loop
         pad_id = self.tokenizer.pad_id
