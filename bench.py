@@ -108,8 +108,11 @@ class AttnCase:
     views: the model's cache layout, benchmark_kernel.py:165-173), a pre-allocated output and
     workspace, launched straight through the C ABI (no per-call allocation)."""
 
-    def __init__(self, torch, lib, l3, dev, pool, B, QH, KVH, S, HD, slots, cache_len=0):
+    def __init__(self, torch, lib, l3, dev, pool, B, QH, KVH, S, HD, slots, cache_len=0, splits=None, flags=None):
         self.torch, self.lib = torch, lib
+        splits = FORCE_SPLITS if splits is None else splits
+        flags = ATTN_FLAGS if flags is None else flags
+        self.flags = flags
         self.B, self.QH, self.KVH, self.S, self.HD = B, QH, KVH, S, HD
         self.bytes = attn_bytes(B, QH, KVH, S, HD)
         L = max(S, cache_len)
@@ -124,10 +127,16 @@ class AttnCase:
             self.v.append(vc[:, :S].transpose(1, 2))
         self.out = torch.empty_like(self.q)
         # 0 = the library plans for the current device (split count and kernel form)
-        self.req_splits = FORCE_SPLITS
-        self.num_splits = FORCE_SPLITS or lib.l3_attn_choose_splits(B, KVH, S, HD, 0, ATTN_FLAGS)
-        self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.req_splits, ATTN_FLAGS)
-        self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
+        self.req_splits = splits
+        self.num_splits = splits or lib.l3_attn_choose_splits(B, KVH, S, HD, 0, flags)
+        self.ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, self.req_splits, flags)
+        self.ws = torch.empty(max(self.ws_bytes, l3.L3_ATTN_COUNTER_BYTES), dtype=torch.uint8, device=dev)
+        if flags & l3.L3_ATTN_FLAG_WS_COUNTERS:
+            # the workspace starts with the arrival counters of the single-launch form (zeroed once, here)
+            rc = lib.l3_attn_workspace_init(self.ws.data_ptr(), self.ws.numel(), torch.cuda.current_stream().cuda_stream)
+            if rc != 0:
+                raise RuntimeError(f"l3_attn_workspace_init failed: {rc}")
+            torch.cuda.synchronize()
         self.part_o = self.part_ml = None
         qt, ot = self.q, self.out
         self._args = []
@@ -137,7 +146,7 @@ class AttnCase:
                 B, QH, KVH, S, HD,
                 l3.i64_array((qt.stride(0), qt.stride(1))), l3.i64_array((kt.stride(0), kt.stride(1), kt.stride(2))),
                 l3.i64_array((vt.stride(0), vt.stride(1), vt.stride(2))), l3.i64_array((ot.stride(0), ot.stride(1))),
-                1.0 / math.sqrt(HD), self.req_splits, ATTN_FLAGS))
+                1.0 / math.sqrt(HD), self.req_splits, flags))
 
     def launch(self, slot, stream_ptr):
         rc = self.lib.l3_attn_decode(*self._args[slot % self.slots], stream_ptr)
@@ -153,7 +162,7 @@ class AttnCase:
             self.part_ml = self.torch.empty((self.B, self.QH, n, 2), dtype=self.torch.float32, device=self.ws.device)
         rc = self.lib.l3_attn_split(a[0], a[1], a[2], self.part_o.data_ptr(), self.part_ml.data_ptr(),
                                     self.B, self.QH, self.KVH, self.S, self.HD, a[11], a[12], a[13], a[15],
-                                    self.req_splits, ATTN_FLAGS, stream_ptr)
+                                    self.req_splits, self.flags, stream_ptr)
         if rc < 0:
             raise RuntimeError(f"l3_attn_split failed: {rc}")
 

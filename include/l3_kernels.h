@@ -63,9 +63,23 @@ const char* l3_strerror(int code);
  *   L3_ATTN_FLAG_PREFILL_*   prefill: force one form of l3_attn_prefill instead of the choice by
  *                            prompt length -- WAVE (every wavefront streams K/V on its own) or
  *                            TILED (a workgroup shares K/V tiles).
- * Any other bit, or both prefill bits at once, gives L3_ERR_FLAGS.
+ *   L3_ATTN_FLAG_WS_COUNTERS decode: the workspace starts with L3_ATTN_COUNTER_BYTES of arrival counters
+ *                            that l3_attn_workspace_init prepared (see there); the library may then merge
+ *                            the split partials inside the split launch instead of launching a combine.
+ *   L3_ATTN_FLAG_TWO_LAUNCHES decode: always split kernel + combine kernel, also where the counters would
+ *                            allow a single launch (for comparisons; same results).
+ *   L3_ATTN_FLAG_FORM_*      decode with an explicit num_splits: run that count as cooperative workgroups
+ *                            (COOP: a workgroup per (batch, kv head, split)) or streamed (STREAM, the default
+ *                            for an explicit count: a wavefront per (batch, kv head, split)).  The automatic
+ *                            plan chooses the form itself.
+ * Any other bit, or both bits of a two-bit field at once, gives L3_ERR_FLAGS.
  */
 #define L3_ATTN_FLAG_KERNEL_FMA 0x1
+#define L3_ATTN_FLAG_WS_COUNTERS 0x2
+#define L3_ATTN_FLAG_FORM_COOP 0x4
+#define L3_ATTN_FLAG_FORM_STREAM 0x8
+#define L3_ATTN_FLAG_FORM_MASK 0xc
+#define L3_ATTN_FLAG_TWO_LAUNCHES 0x40
 #define L3_ATTN_FLAG_PREFILL_WAVE 0x10
 #define L3_ATTN_FLAG_PREFILL_TILED 0x20
 #define L3_ATTN_FLAG_PREFILL_MASK 0x30
@@ -115,6 +129,30 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out,
                    const int64_t q_strides[2], const int64_t k_strides[3],
                    const int64_t v_strides[3], const int64_t out_strides[2],
                    float scale, int num_splits, int flags, void* stream);
+
+/*
+ * Single-launch decode attention: prepares a workspace whose first L3_ATTN_COUNTER_BYTES hold the arrival
+ * counters with which the split kernel itself merges the partials of a (batch, kv head) -- the workgroup
+ * that finishes a head last does it, out of the L2 of the XCD all workgroups of that head were placed on --
+ * so that no combine kernel is launched (the reference always launches two kernels: custom_kernels.cu:274-275).
+ *   l3_attn_workspace_init  zeroes the counters on `stream` and, on the first call per device, runs a probe
+ *       launch that confirms the placement rule the scheme rests on (workgroup i of a grid runs on XCD i % 8)
+ *       and WAITS for it: call it at set-up, outside stream capture.  workspace: 256-byte aligned, at least
+ *       L3_ATTN_COUNTER_BYTES.  Every later l3_attn_decode / l3_attn_decode_devlen call on that workspace must
+ *       pass L3_ATTN_FLAG_WS_COUNTERS (sizes from l3_attn_decode_workspace_bytes with the same flag); the
+ *       counters are zero again when a call's kernels have finished, nothing else may write them, and calls
+ *       that share a workspace must not overlap in time.  Where the probe did not confirm the rule, or the
+ *       grid of a call does not keep a head on one XCD (B x KVH not a multiple of 8, more than 32 splits,
+ *       more than 1023 (batch, kv head) pairs), the call runs split kernel + combine as without the flag.
+ *   l3_attn_merge_in_launch_available  1 when the probe has confirmed the rule on the current device.
+ *   l3_attn_placement_errors  number of workgroups that found themselves on another XCD than the rule says
+ *       since the counters were prepared (always 0 on a device that passed the probe; a diagnostic that
+ *       synchronises): workspace = a prepared workspace, or NULL for l3_attn_decode_static's array.
+ */
+#define L3_ATTN_COUNTER_BYTES (128u << 10)
+int l3_attn_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+int l3_attn_merge_in_launch_available(void);
+int64_t l3_attn_placement_errors(const void* workspace);
 
 /*
  * l3_attn_decode for callers that cannot allocate device memory and have no workspace to pass

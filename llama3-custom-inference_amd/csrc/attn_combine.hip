@@ -12,14 +12,13 @@
 // loads of its (max, sum) pairs AND of its partial rows back to back, before it knows any
 // weight, and only then reduces.  Each wavefront merges up to 32 splits per pass with its own
 // local maximum; the eight local results are merged through LDS.
-#include "attn_common.hpp"
+#include "attn_merge.hpp"
 
 namespace l3 {
 
 namespace {
 
 constexpr int kCombineWaves = 8;
-constexpr int kCombineRows = 32;  // splits a wavefront merges per pass (their loads are all in flight at once)
 
 // CG = column groups: with few (batch, query head) pairs the head dimension is dealt to CG
 // workgroups (blockIdx.y), each merging HD / CG columns of every split, so that more than
@@ -120,18 +119,13 @@ attn_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__
 
 // At most 32 splits per (batch, query head) pair: one WAVEFRONT per pair, four pairs per workgroup, no
 // LDS and no barrier -- with many pairs the eight-wavefront form above would launch thousands of
-// workgroups that each merge two or three rows, with few it waits at its barrier for nothing.  Same arithmetic, in the same order, as one
-// wavefront of that kernel.
+// workgroups that each merge two or three rows, with few it waits at its barrier for nothing.  The merge itself
+// (merge_pair_rows) is shared with the split kernel's single-launch form, so both give the same bits.
 template <int HD>
 __global__ void __launch_bounds__(4 * kWaveSize)
 attn_combine_rows_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
                          uint16_t* __restrict__ out, int QH, int n_rows, int64_t total_pairs, int64_t o_sb,
                          int64_t o_sh, const int* __restrict__ seqlen_dev, int tokens_per_split, int producer_groups) {
-    constexpr int TPR = HD / 4;             // lanes covering a partial row with float4 loads
-    constexpr int RPL = kWaveSize / TPR;    // rows per wavefront-wide load
-    constexpr int NLD = kCombineRows / RPL; // row loads per pass
-
-    const int lane = threadIdx.x & (kWaveSize - 1);
     const int wave = threadIdx.x / kWaveSize;
     // A workgroup takes four consecutive pairs.  Workgroups go to the eight XCDs in turn (id % 8), each with an L2
     // of its own, and so did the streaming split kernel's: its workgroup (head group g of G, batch b, split group z)
@@ -150,56 +144,10 @@ attn_combine_rows_kernel(const float* __restrict__ part_o, const float2* __restr
     if (bq >= total_pairs) return;   // whole wavefront; the kernel has no barrier
     int n = n_rows;
     if (seqlen_dev) n = min(n_rows, max(1, (*seqlen_dev + tokens_per_split - 1) / tokens_per_split));
-    const float2* ml = part_ml + bq * n_rows;
-    const float4* po = reinterpret_cast<const float4*>(part_o + bq * n_rows * HD);
-    const int dq = lane % TPR;
-    const int sub = lane / TPR;
-
-    float m_w = kMaskedScore, l_w = 0.f;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int r0 = 0; r0 < n; r0 += kCombineRows) {
-        float2 st = make_float2(kMaskedScore, 0.f);
-        if (lane < kCombineRows && r0 + lane < n) st = ml[r0 + lane];
-        float4 x[NLD];
-#pragma unroll
-        for (int u = 0; u < NLD; ++u) {
-            x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (r0 + u * RPL < n) {   // wavefront-uniform: loads past the last split are not issued
-                const int r = min(r0 + u * RPL + sub, n - 1);   // rows past the end get weight 0 below
-                x[u] = po[int64_t(r) * TPR + dq];
-            }
-        }
-        const float m_new = fmaxf(m_w, wave_max(st.x));
-        const float alpha = fast_exp2(m_w - m_new);
-        const float wgt = fast_exp2(st.x - m_new);
-        l_w = fmaf(l_w, alpha, wave_sum(st.y * wgt));
-        acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
-        m_w = m_new;
-#pragma unroll
-        for (int u = 0; u < NLD; ++u) {
-            const float w = __shfl(wgt, u * RPL + sub, kWaveSize);
-            acc.x = fmaf(w, x[u].x, acc.x);
-            acc.y = fmaf(w, x[u].y, acc.y);
-            acc.z = fmaf(w, x[u].z, acc.z);
-            acc.w = fmaf(w, x[u].w, acc.w);
-        }
-    }
-#pragma unroll
-    for (int off = TPR; off < kWaveSize; off <<= 1) {
-        acc.x += __shfl_xor(acc.x, off, kWaveSize);
-        acc.y += __shfl_xor(acc.y, off, kWaveSize);
-        acc.z += __shfl_xor(acc.z, off, kWaveSize);
-        acc.w += __shfl_xor(acc.w, off, kWaveSize);
-    }
-    if (lane < TPR) {
-        const float inv = 1.0f / l_w;
-        uint2 packed;
-        packed.x = pack_bf16x2(acc.x * inv, acc.y * inv);
-        packed.y = pack_bf16x2(acc.z * inv, acc.w * inv);
-        const int64_t b = bq / QH;
-        const int qh = int(bq % QH);
-        *reinterpret_cast<uint2*>(out + b * o_sb + int64_t(qh) * o_sh + lane * 4) = packed;
-    }
+    const int64_t b = bq / QH;
+    const int qh = int(bq % QH);
+    merge_pair_rows<HD, PlainReader>(part_o + bq * n_rows * HD, part_ml + bq * n_rows, n,
+                                     out + b * o_sb + int64_t(qh) * o_sh);
 }
 
 }  // namespace

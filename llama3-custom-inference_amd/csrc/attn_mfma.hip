@@ -15,6 +15,7 @@
 // The 16 columns of the MFMA tiles carry the R <= 8 query heads of the GQA group (columns R..15
 // are zero padding; the matrix cores have room to spare on a memory-bound kernel), so each K/V
 // byte is fetched once per group.
+#include "attn_merge.hpp"
 #include "attn_mfma_core.hpp"
 
 namespace l3 {
@@ -60,9 +61,14 @@ attn_splitkv_mfma_kernel(const int R, const int hpw_log2, const AttnParams p) {
     }
     const int t_begin = split * p.tokens_per_split;
     const int S = p.seqlen_dev ? max(1, min(*p.seqlen_dev, p.S)) : p.S;  // wave-uniform; a length below 1 counts as 1
+    // Single-launch form (cooperative workgroups with p.arrive set): the workgroup that finishes a (batch,
+    // kv head) last merges its partials, and every split of the plan is counted as an arrival -- also one
+    // that a device-side KV length leaves without tokens (it streams and writes nothing, the merge skips its row).
+    const bool merge_here = COOP && p.arrive != nullptr;
     // A split past the plan (last workgroup of the streaming form: whole wavefront, no barrier follows)
-    // or past a device-side KV length (whole workgroup when COOP): the combine skips it.
-    if (split >= p.num_splits || t_begin >= S) return;
+    // or, with a combine launch to follow, past a device-side KV length (whole workgroup when COOP).
+    if (split >= p.num_splits || (!merge_here && t_begin >= S)) return;
+    const bool has_tokens = t_begin < S;
     const int t_end = min(S, t_begin + p.tokens_per_split);
     const float c = p.scale_log2e;
 
@@ -97,6 +103,7 @@ attn_splitkv_mfma_kernel(const int R, const int hpw_log2, const AttnParams p) {
         __shared__ float s_m[kMfmaWaves][kAttnMaxRatio];
         __shared__ float s_l[kMfmaWaves][kAttnMaxRatio];
         __shared__ __align__(16) float s_o[kMfmaWaves][kAttnMaxRatio][HD];
+        __shared__ int s_last;
         if (fn < R) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
@@ -128,10 +135,37 @@ attn_splitkv_mfma_kernel(const int R, const int hpw_log2, const AttnParams p) {
                 const float inv = 1.0f / L;
                 *reinterpret_cast<uint32_t*>(p.out + b * p.o_sb + int64_t(qh) * p.o_sh + d) =
                     pack_bf16x2(o0 * inv, o1 * inv);
-            } else {
+            } else if (has_tokens) {
                 const int64_t row = attn_partial_row(p, b, qh, split);
                 *reinterpret_cast<float2*>(p.part_o + row * HD + d) = make_float2(o0, o1);
                 if (d == 0) p.part_ml[row] = make_float2(M, L);
+            }
+        }
+        if (merge_here) {
+            // the workgroup that arrives last at its (batch, kv head) merges the head's partial rows out of
+            // the XCD's L2: the eight wavefronts share the R query heads, 8 / R column groups per head
+            wait_stores_in_l2();
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                bool same_xcd = true;
+                s_last = arrive_is_last(p.arrive + (int64_t(b) * p.KVH + kvh) * kAttnArriveStride, p.num_splits, &same_xcd);
+                if (!same_xcd) atomicAdd(p.arrive + kAttnDiagSlot * kAttnArriveStride, 1u);
+            }
+            __syncthreads();
+            if (s_last) {
+                const int n = min(p.num_splits, (S + p.tokens_per_split - 1) / p.tokens_per_split);
+                auto merge = [&](auto cgs) {
+                    constexpr int CG = decltype(cgs)::value;
+                    const int qh = kvh * R + wave / CG;
+                    const int64_t row0 = attn_partial_row(p, b, qh, 0);
+                    merge_pair_rows<HD, L2Reader, CG>(p.part_o + row0 * HD, p.part_ml + row0, n,
+                                                      p.out + b * p.o_sb + int64_t(qh) * p.o_sh, wave % CG);
+                };
+                if (R == 8) merge(std::integral_constant<int, 1>{});
+                else if (R == 4) merge(std::integral_constant<int, 2>{});
+                else if (R == 2) merge(std::integral_constant<int, 4>{});
+                else if (R == 1) merge(std::integral_constant<int, 8>{});
+                else if (wave < R) merge(std::integral_constant<int, 1>{});   // R = 3
             }
         }
     } else if (fn < R) {
@@ -159,7 +193,37 @@ attn_splitkv_mfma_kernel(const int R, const int hpw_log2, const AttnParams p) {
     }
 }
 
+// Workgroup i of a 1-D grid reports the XCD it runs on.
+__global__ void xcd_probe_kernel(unsigned* where, int stride_words) {
+    if (threadIdx.x == 0) where[int64_t(blockIdx.x) * stride_words] = xcc_id();
+}
+
+__global__ void fill_zero_u32_kernel(unsigned* dst, size_t n) {
+    const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = 0u;
+}
+
 }  // namespace
+
+int launch_xcd_probe(unsigned* where, int n, int stride_words, hipStream_t stream) {
+    hipLaunchKernelGGL(xcd_probe_kernel, dim3(unsigned(n)), dim3(kWaveSize), 0, stream, where, stride_words);
+    return int(hipGetLastError());
+}
+
+int launch_fill_zero_u32(unsigned* dst, size_t n, hipStream_t stream) {
+    hipLaunchKernelGGL(fill_zero_u32_kernel, dim3(unsigned((n + 255) / 256)), dim3(256), 0, stream, dst, n);
+    return int(hipGetLastError());
+}
+
+bool attn_mfma_can_merge_in_launch(int B, int KVH, bool coop, int num_splits) {
+    // Cooperative form only: a workgroup per (batch, kv head, split) with linear id kvh + KVH (b + B split),
+    // and a last arriver that merges in one pass.  (In the streaming form the arrivals would be single
+    // wavefronts; built and measured on 16 sequences of 4096 tokens, a lone wavefront merging its head's four
+    // query heads took longer than the combine launch it saved: 25.0 against 24.5 us.)
+    if (!coop || num_splits < 2 || num_splits > kCombineRows) return false;
+    if (B > 65535 || int64_t(B) * KVH > kAttnDiagSlot) return false;   // one launch, one counter per (batch, kv head)
+    return (int64_t(KVH) * B) % 8 == 0;
+}
 
 int attn_mfma_heads_per_wg(int KVH) {
     for (int h = kMfmaWaves; h > 1; h /= 2) {

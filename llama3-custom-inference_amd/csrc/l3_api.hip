@@ -40,10 +40,12 @@ int check_attn_shape(int B, int QH, int KVH, int S, int HD) {
     return L3_OK;
 }
 
-size_t attn_workspace_bytes(int B, int QH, int HD, int num_splits) {
+// With `counters` the workspace starts with the arrival counters of the single-launch form.
+size_t attn_workspace_bytes(int B, int QH, int HD, int num_splits, bool counters) {
     if (num_splits <= 1) return 0;
     const size_t rows = size_t(B) * size_t(QH) * size_t(num_splits);
-    return round_up(rows * HD * sizeof(float), kWorkspaceAlign) + round_up(rows * sizeof(float2), kWorkspaceAlign);
+    return (counters ? size_t(L3_ATTN_COUNTER_BYTES) : 0) + round_up(rows * HD * sizeof(float), kWorkspaceAlign) +
+           round_up(rows * sizeof(float2), kWorkspaceAlign);
 }
 
 }  // namespace
@@ -58,6 +60,40 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];
+// Per device: 0 = not probed yet, 1 = the workgroups of a grid go to the 8 XCDs in turn, so that workgroups
+// whose ids agree modulo 8 share an XCD (the single-launch attention form may be used), -1 = they do not.
+std::atomic<int> g_xcd_state[kMaxDevices];
+
+int current_device_index() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return dev;
+}
+
+// Launches a probe grid that records the XCD of each workgroup into `counters` (the counter region
+// of a workspace, used as scratch), waits for it and compares with the rule.  Synchronises `st`.
+int probe_xcd_mapping(int dev, unsigned* counters, hipStream_t st) {
+    constexpr int kProbe = 256;
+    static_assert(kProbe <= kAttnArriveSlots, "one counter slot per probe workgroup");
+    if (launch_xcd_probe(counters, kProbe, kAttnArriveStride, st) != 0) return L3_ERR_HIP;
+    static unsigned host[kProbe * kAttnArriveStride];
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (hipStreamSynchronize(st) != hipSuccess ||
+        hipMemcpy(host, counters, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        return L3_ERR_HIP;
+    }
+    bool ok = true;
+    // round robin from whichever XCD the dispatcher starts this grid on
+    const unsigned first = host[0];
+    ok = first < 8u;
+    for (int i = 0; i < kProbe; ++i) ok = ok && host[i * kAttnArriveStride] == (first + unsigned(i)) % 8u;
+    g_xcd_state[dev].store(ok ? 1 : -1, std::memory_order_release);
+    return L3_OK;
+}
 
 // Device address of the current device's copy of the array, looked up once per device (null on failure).
 void* static_scratch_ptr() {
@@ -76,6 +112,25 @@ void* static_scratch_ptr() {
         return nullptr;
     }
     g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    return ptr;
+}
+
+// The static array starts with its arrival counters, which the loader zeroed.  On the first call on a
+// device (outside stream capture, as that call has to be anyway) the XCD rule is probed there and the
+// words the probe used are cleared again.
+void* static_scratch_ready() {
+    void* ptr = static_scratch_ptr();
+    const int dev = current_device_index();
+    if (!ptr || dev < 0) return nullptr;
+    if (g_xcd_state[dev].load(std::memory_order_acquire) == 0) {
+        unsigned* counters = static_cast<unsigned*>(ptr);
+        if (probe_xcd_mapping(dev, counters, nullptr) != L3_OK) return nullptr;
+        if (launch_fill_zero_u32(counters, L3_ATTN_COUNTER_BYTES / sizeof(unsigned), nullptr) != 0 ||
+            hipStreamSynchronize(nullptr) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+    }
     return ptr;
 }
 }  // namespace
@@ -99,12 +154,20 @@ namespace {
 // The split-KV kernel a call's flags ask for (the library keeps no such choice between calls).
 int attn_impl_of(int flags) { return (flags & L3_ATTN_FLAG_KERNEL_FMA) ? kAttnImplFma : kAttnImplMfma; }
 bool attn_flags_ok(int flags) {
-    return (flags & ~(L3_ATTN_FLAG_KERNEL_FMA | L3_ATTN_FLAG_PREFILL_MASK)) == 0 &&
-           (flags & L3_ATTN_FLAG_PREFILL_MASK) != L3_ATTN_FLAG_PREFILL_MASK;
+    constexpr int known = L3_ATTN_FLAG_KERNEL_FMA | L3_ATTN_FLAG_PREFILL_MASK | L3_ATTN_FLAG_WS_COUNTERS |
+                          L3_ATTN_FLAG_TWO_LAUNCHES | L3_ATTN_FLAG_FORM_MASK;
+    return (flags & ~known) == 0 && (flags & L3_ATTN_FLAG_PREFILL_MASK) != L3_ATTN_FLAG_PREFILL_MASK &&
+           (flags & L3_ATTN_FLAG_FORM_MASK) != L3_ATTN_FLAG_FORM_MASK;
+}
+// Whether the plan may count on the merge inside the split launch (the MFMA kernel with a counter
+// region in the workspace, not switched off for the call).
+bool attn_merge_in_launch_wanted(int flags) {
+    return (flags & L3_ATTN_FLAG_WS_COUNTERS) && !(flags & (L3_ATTN_FLAG_TWO_LAUNCHES | L3_ATTN_FLAG_KERNEL_FMA));
 }
 }  // namespace
 
-AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl) {
+AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl, int form,
+                        bool merge_in_launch) {
     const int tile = attn_tile_tokens(HD, impl);
     const int tiles = ceil_div(S, tile);
     AttnPlan plan;
@@ -112,6 +175,8 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
     int splits;
     if (requested > 0) {
         splits = requested;
+        // a requested count is streamed unless the call asks for cooperative workgroups
+        plan.coop = impl == kAttnImplMfma && form == L3_ATTN_FLAG_FORM_COOP;
     } else if (impl == kAttnImplMfma) {
         // Short sequences are latency-bound.  With at most one tile per wavefront of a workgroup (or two,
         // when there are too many heads for each to get a second workgroup) and not already enough
@@ -242,15 +307,17 @@ int l3_attn_choose_splits(int B, int KVH, int S, int HD, int num_cus, int flags)
     if (B <= 0 || KVH <= 0 || S <= 0) return L3_ERR_SHAPE;
     if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
     if (num_cus <= 0) num_cus = current_device_cus();
-    return attn_make_plan(B, KVH, S, HD, 0, num_cus, attn_impl_of(flags)).num_splits;
+    return attn_make_plan(B, KVH, S, HD, 0, num_cus, attn_impl_of(flags), flags & L3_ATTN_FLAG_FORM_MASK,
+                          attn_merge_in_launch_wanted(flags)).num_splits;
 }
 
 size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int num_splits, int flags) {
     if (check_attn_shape(B, QH, KVH, S, HD) != L3_OK) return 0;
     if (num_splits < 0 || num_splits > L3_ATTN_MAX_SPLITS || !attn_flags_ok(flags)) return 0;
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
-    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, attn_impl_of(flags));
-    return attn_workspace_bytes(B, QH, HD, plan.num_splits);
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, attn_impl_of(flags),
+                                         flags & L3_ATTN_FLAG_FORM_MASK, attn_merge_in_launch_wanted(flags));
+    return attn_workspace_bytes(B, QH, HD, plan.num_splits, (flags & L3_ATTN_FLAG_WS_COUNTERS) != 0);
 }
 
 namespace {
@@ -302,6 +369,7 @@ void fill_attn_params(AttnParams& p, const void* q, const void* k, const void* v
     p.o_sb = out_strides ? out_strides[0] : 0;
     p.o_sh = out_strides ? out_strides[1] : 0;
     p.scale_log2e = scale * 1.4426950408889634f;
+    p.arrive = nullptr;
 }
 
 int launch_split_stage(const AttnParams& p, int HD, int R, int impl, bool coop, hipStream_t st) {
@@ -323,14 +391,17 @@ int attn_decode_impl(const void* q, const void* k, const void* v, void* out, voi
     if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
     if (!scale_ok(scale)) return L3_ERR_SCALE;
     const int impl = attn_impl_of(flags);
+    if (static_scratch) flags |= L3_ATTN_FLAG_WS_COUNTERS;   // the static array always starts with its counters
+    const bool counters = (flags & L3_ATTN_FLAG_WS_COUNTERS) != 0;
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
-    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
-    const size_t need = attn_workspace_bytes(B, QH, HD, plan.num_splits);
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl, flags & L3_ATTN_FLAG_FORM_MASK,
+                                         attn_merge_in_launch_wanted(flags));
+    const size_t need = attn_workspace_bytes(B, QH, HD, plan.num_splits, counters);
     if (static_scratch) {
         // the partials go to this device's copy of the static array; nothing is allocated
         if (need > L3_ATTN_STATIC_SCRATCH_BYTES) return L3_ERR_SCRATCH;
         if (need > 0) {
-            workspace = static_scratch_ptr();
+            workspace = static_scratch_ready();
             if (!workspace) return L3_ERR_HIP;
         }
     } else if (need > 0) {
@@ -340,16 +411,24 @@ int attn_decode_impl(const void* q, const void* k, const void* v, void* out, voi
     AttnParams p;
     fill_attn_params(p, q, k, v, out, B, QH, KVH, S, q_strides, k_strides, v_strides, out_strides, scale, plan);
     p.seqlen_dev = seqlen_dev;
+    bool merge_in_launch = false;
     if (plan.num_splits > 1) {
         const size_t rows = size_t(B) * size_t(QH) * size_t(plan.num_splits);
-        char* ws = static_cast<char*>(workspace);
+        char* ws = static_cast<char*>(workspace) + (counters ? size_t(L3_ATTN_COUNTER_BYTES) : 0);
         p.part_o = reinterpret_cast<float*>(ws);
         p.part_ml = reinterpret_cast<float2*>(ws + round_up(rows * HD * sizeof(float), kWorkspaceAlign));
+        // One launch instead of two: only with prepared counters, on a device whose workgroup placement has
+        // been confirmed, and for a grid that keeps every (batch, kv head) on one XCD.
+        if (attn_merge_in_launch_wanted(flags) && attn_mfma_can_merge_in_launch(B, KVH, plan.coop, plan.num_splits)) {
+            const int dev = current_device_index();
+            merge_in_launch = dev >= 0 && g_xcd_state[dev].load(std::memory_order_acquire) == 1;
+        }
+        if (merge_in_launch) p.arrive = static_cast<unsigned*>(workspace);
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     int err = launch_split_stage(p, HD, QH / KVH, impl, plan.coop, st);
     const int groups = (impl == kAttnImplMfma && !plan.coop && B <= 65535) ? KVH / attn_mfma_heads_per_wg(KVH) : 0;
-    if (err == 0 && plan.num_splits > 1) err = launch_attn_combine(p, HD, groups, st);
+    if (err == 0 && plan.num_splits > 1 && !merge_in_launch) err = launch_attn_combine(p, HD, groups, st);
     return err == 0 ? L3_OK : L3_ERR_HIP;
 }
 }  // namespace
@@ -368,6 +447,38 @@ int l3_attn_decode_static(const void* q, const void* k, const void* v, void* out
                           int flags, void* stream) {
     return attn_decode_impl(q, k, v, out, nullptr, 0, B, QH, KVH, S, HD, q_strides, k_strides, v_strides,
                             out_strides, scale, num_splits, flags, nullptr, stream, true);
+}
+
+int l3_attn_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+    if (!workspace) return L3_ERR_NULL_POINTER;
+    if (workspace_bytes < L3_ATTN_COUNTER_BYTES) return L3_ERR_WORKSPACE;
+    if (!aligned(workspace, kWorkspaceAlign)) return L3_ERR_ALIGNMENT;
+    const int dev = current_device_index();
+    if (dev < 0) return L3_ERR_HIP;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    unsigned* counters = static_cast<unsigned*>(workspace);
+    if (g_xcd_state[dev].load(std::memory_order_acquire) == 0) {
+        if (int rc = probe_xcd_mapping(dev, counters, st); rc != L3_OK) return rc;
+    }
+    if (launch_fill_zero_u32(counters, L3_ATTN_COUNTER_BYTES / sizeof(unsigned), st) != 0) return L3_ERR_HIP;
+    return L3_OK;
+}
+
+int l3_attn_merge_in_launch_available(void) {
+    const int dev = current_device_index();
+    return dev >= 0 && g_xcd_state[dev].load(std::memory_order_acquire) == 1;
+}
+
+int64_t l3_attn_placement_errors(const void* workspace) {
+    if (!workspace) workspace = static_scratch_ptr();
+    if (!workspace) return L3_ERR_HIP;
+    unsigned n = 0;
+    const char* word = static_cast<const char*>(workspace) + size_t(kAttnDiagSlot) * kAttnArriveStride * sizeof(unsigned);
+    if (hipMemcpy(&n, word, sizeof(n), hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        return L3_ERR_HIP;
+    }
+    return int64_t(n);
 }
 
 int l3_attn_decode_devlen(const void* q, const void* k, const void* v, void* out, void* workspace,
@@ -441,7 +552,8 @@ int l3_attn_split(const void* q, const void* k, const void* v, float* part_o, fl
     if (!scale_ok(scale)) return L3_ERR_SCALE;
     const int impl = attn_impl_of(flags);
     const int cus = (num_splits == 0) ? current_device_cus() : 0;
-    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl);
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, impl, flags & L3_ATTN_FLAG_FORM_MASK,
+                                         attn_merge_in_launch_wanted(flags));
     AttnParams p;
     fill_attn_params(p, q, k, v, nullptr, B, QH, KVH, S, q_strides, k_strides, v_strides, nullptr, scale, plan);
     p.part_o = part_o;

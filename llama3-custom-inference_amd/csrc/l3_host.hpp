@@ -37,7 +37,10 @@ constexpr int attn_tile_tokens(int HD, int impl) {
 int attn_mfma_heads_per_wg(int KVH);
 
 // Pure integer logic (no HIP): the plan for `requested` splits (0 = automatic).
-AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl);
+// `form`: L3_ATTN_FLAG_FORM_* bits of the call (which form a requested count is run in);
+// `merge_in_launch`: the call can merge inside the split launch where the grid allows it.
+AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cus, int impl, int form = 0,
+                        bool merge_in_launch = false);
 
 // Compute units of the current device, 256 when no device can be queried.
 int current_device_cus();
@@ -59,7 +62,16 @@ struct AttnParams {
     float* part_o;    // [B][QH][num_splits][HD] unnormalised partial outputs; null = write `out` directly
     float2* part_ml;  // [B][QH][num_splits] (max in log2 units, sum of exp2)
     int64_t o_sb, o_sh;
+    // Single-launch form of the MFMA kernel: arrival counters, one per (batch, kv head) at a stride of
+    // kAttnArriveStride words, all zero between launches; null = partials only, a combine launch follows.
+    unsigned* arrive;
 };
+
+// The counters sit a cache line apart (units on different XCDs never share a line); the last slot
+// counts workgroups that found themselves on another XCD than their id implies (a diagnostic).
+constexpr int kAttnArriveStride = 32;
+constexpr int kAttnArriveSlots = int(L3_ATTN_COUNTER_BYTES / (kAttnArriveStride * sizeof(unsigned)));
+constexpr int kAttnDiagSlot = kAttnArriveSlots - 1;
 
 struct PrefillParams {
     const uint16_t* q;   // (B, QH, T, HD) with {batch, head, token} strides
@@ -125,6 +137,12 @@ int launch_attn_splitkv_mfma(const AttnParams& p, int HD, int R, bool coop, hipS
 // producer_groups: head groups per batch entry of the streaming MFMA split kernel that wrote the partials (its
 // grid's x extent), 0 when another kernel or a caller produced them
 int launch_attn_combine(const AttnParams& p, int HD, int producer_groups, hipStream_t stream);
+// True when every workgroup of a (batch, kv head) of the MFMA kernel's grid has the same linear id modulo 8
+// (runs on one XCD) and the counters suffice: the condition for merging inside the split launch.
+bool attn_mfma_can_merge_in_launch(int B, int KVH, bool coop, int num_splits);
+// Writes the XCD each of `n` workgroups of a 1-D grid ran on to where[i * stride_words]; and a zero fill.
+int launch_xcd_probe(unsigned* where, int n, int stride_words, hipStream_t stream);
+int launch_fill_zero_u32(unsigned* dst, size_t n, hipStream_t stream);
 int launch_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups, hipStream_t stream);
 int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
                     bool vec_ok, hipStream_t stream);

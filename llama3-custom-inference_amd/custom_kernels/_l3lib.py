@@ -28,6 +28,12 @@ L3_LINEAR_MAX_ROWS = 16         # one launch, any matrix shape, optional input n
 L3_LINEAR_SPLITK_MAX_ROWS = 64
 L3_LINEAR_STAGE_ELEMS = 24576   # activations (rows padded by 8) the fused input norm can stage in LDS
 L3_ATTN_FLAG_KERNEL_FMA = 0x1
+L3_ATTN_FLAG_WS_COUNTERS = 0x2
+L3_ATTN_FLAG_FORM_COOP = 0x4
+L3_ATTN_FLAG_FORM_STREAM = 0x8
+L3_ATTN_FLAG_FORM_MASK = 0xc
+L3_ATTN_FLAG_TWO_LAUNCHES = 0x40
+L3_ATTN_COUNTER_BYTES = 128 << 10
 L3_ATTN_FLAG_PREFILL_WAVE = 0x10
 L3_ATTN_FLAG_PREFILL_TILED = 0x20
 L3_ATTN_FLAG_PREFILL_MASK = 0x30
@@ -47,6 +53,9 @@ SIGNATURES = {
          _c_i64p, _c_i64p, _c_i64p, _c_i64p,                                  # strides
          ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],        # scale splits flags stream
     ),
+    "l3_attn_workspace_init": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "l3_attn_merge_in_launch_available": (ctypes.c_int, []),
+    "l3_attn_placement_errors": (ctypes.c_int64, [ctypes.c_void_p]),
     "l3_attn_decode_static": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,  # q k v out

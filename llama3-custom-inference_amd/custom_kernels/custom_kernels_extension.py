@@ -91,21 +91,58 @@ def _workspace(device, stream_ptr: int, nbytes: int):
     return ws
 
 
+_attn_workspaces = {}  # (device index, stream handle) -> uint8 tensor that starts with prepared arrival counters
+
+
+def _attn_workspace(lib, device, stream_ptr: int, flags: int, size_of):
+    """Workspace and flags for a decode-attention call.  Outside stream capture the workspace is one kept per
+    (device, stream) whose head holds the arrival counters of the single-launch form, prepared once by
+    l3_attn_workspace_init when the buffer is (re)allocated -- that call synchronises, which a capture
+    would not allow, so a call under capture takes a plain buffer from the graph's pool and runs split
+    kernel + combine.  ``size_of(flags)`` returns the bytes the call needs with those flags."""
+    if torch.cuda.is_current_stream_capturing():
+        flags &= ~_l3lib.L3_ATTN_FLAG_WS_COUNTERS
+        nbytes = size_of(flags)
+        return (_workspace(device, stream_ptr, nbytes) if nbytes else None), nbytes, flags
+    flags |= _l3lib.L3_ATTN_FLAG_WS_COUNTERS
+    nbytes = size_of(flags)
+    if nbytes == 0:
+        return None, 0, flags
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
+    ws = _attn_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 4 << 20), dtype=torch.uint8, device=device)
+        rc = lib.l3_attn_workspace_init(ws.data_ptr(), ws.numel(), stream_ptr)
+        if rc != 0:
+            _fail(rc, "l3_attn_workspace_init")
+        _attn_workspaces[key] = ws
+    return ws, nbytes, flags
+
+
 # Flags the attention operators pass to the library when the caller gives none: a context-local
 # value (per thread / per asyncio task), never a process-wide switch.  The library itself keeps no
 # option between calls.
 _attn_flags = contextvars.ContextVar("l3_attn_flags", default=0)
 
-_FLAG_NAMES = {"mfma": 0, "fma": _l3lib.L3_ATTN_FLAG_KERNEL_FMA, "auto": 0, "wave": _l3lib.L3_ATTN_FLAG_PREFILL_WAVE,
-               "tiled": _l3lib.L3_ATTN_FLAG_PREFILL_TILED}
+_KERNEL_BITS = {"mfma": 0, "fma": _l3lib.L3_ATTN_FLAG_KERNEL_FMA}
+_PREFILL_BITS = {"auto": 0, "wave": _l3lib.L3_ATTN_FLAG_PREFILL_WAVE, "tiled": _l3lib.L3_ATTN_FLAG_PREFILL_TILED}
+_LAUNCH_BITS = {"auto": 0, "two": _l3lib.L3_ATTN_FLAG_TWO_LAUNCHES}
 
 
 @contextlib.contextmanager
-def attention_flags(kernel: str = "mfma", prefill: str = "auto"):
+def attention_flags(kernel=None, prefill=None, launches=None):
     """Within the block, attention calls of this thread that pass no ``flags`` use the named
-    split-KV kernel ("mfma" / "fma") and prefill form ("auto" / "wave" / "tiled").
-    For measurements and tests; the defaults are the library's own choices."""
-    token = _attn_flags.set(_FLAG_NAMES[kernel] | _FLAG_NAMES[prefill])
+    split-KV kernel ("mfma" / "fma"), prefill form ("auto" / "wave" / "tiled") and launch scheme
+    ("auto" / "two": always split kernel + combine kernel).  An argument that is not given keeps what
+    an enclosing block chose, so blocks nest.  For measurements and tests; the defaults are the
+    library's own choices."""
+    bits = _attn_flags.get()
+    for name, table, mask in ((kernel, _KERNEL_BITS, _l3lib.L3_ATTN_FLAG_KERNEL_FMA),
+                              (prefill, _PREFILL_BITS, _l3lib.L3_ATTN_FLAG_PREFILL_MASK),
+                              (launches, _LAUNCH_BITS, _l3lib.L3_ATTN_FLAG_TWO_LAUNCHES)):
+        if name is not None:
+            bits = (bits & ~mask) | table[name]
+    token = _attn_flags.set(bits)
     try:
         yield
     finally:
@@ -159,9 +196,10 @@ def flash_attention_decode(query, keys, values, num_splits: int = 0, flags=None)
 
     with _on_device(query.device):
         # num_splits == 0 lets the library plan for the current device (split count and kernel form)
-        ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, num_splits, flags)
         stream_ptr = _stream_ptr(query.device)
-        ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None
+        ws, ws_bytes, flags = _attn_workspace(
+            lib, query.device, stream_ptr, flags,
+            lambda f: lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, num_splits, f))
         rc = lib.l3_attn_decode(
             query.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr(),
             ws.data_ptr() if ws is not None else None, ws_bytes,
@@ -322,9 +360,10 @@ def flash_attention_decode_devlen(query, keys, values, kv_len, num_splits: int =
     else:
         _check_out(out, query, "flash_attention_decode_devlen")
     with _on_device(query.device):
-        ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, L, HD, num_splits, flags)
         stream_ptr = _stream_ptr(query.device)
-        ws = _workspace(query.device, stream_ptr, ws_bytes) if ws_bytes else None
+        ws, ws_bytes, flags = _attn_workspace(
+            lib, query.device, stream_ptr, flags,
+            lambda f: lib.l3_attn_decode_workspace_bytes(B, QH, KVH, L, HD, num_splits, f))
         rc = lib.l3_attn_decode_devlen(
             query.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr(),
             ws.data_ptr() if ws is not None else None, ws_bytes, B, QH, KVH, L, HD,

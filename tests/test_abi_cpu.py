@@ -235,7 +235,7 @@ def test_stage_entry_points_argument_checks():
         == _l3lib.L3_ERR_HEAD_SIZE
     assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE + 4, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, 0, None) \
         == _l3lib.L3_ERR_ALIGNMENT
-    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, 2, None) \
+    assert lib.l3_attn_split(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 32, 8, 256, 64, qs, ks, ks, 0.125, 1, 0x80, None) \
         == _l3lib.L3_ERR_FLAGS
     assert lib.l3_attn_combine(FAKE, FAKE, None, 1, 32, 64, 4, qs, None) == _l3lib.L3_ERR_NULL_POINTER
     assert lib.l3_attn_combine(FAKE, FAKE, FAKE, 1, 32, 96, 4, qs, None) == _l3lib.L3_ERR_HEAD_SIZE
@@ -256,8 +256,9 @@ def test_prefill_argument_checks():
 
     assert call(scale=0.0) == _l3lib.L3_ERR_SCALE
 
-    assert call(flags=0x40) == _l3lib.L3_ERR_FLAGS
+    assert call(flags=0x80) == _l3lib.L3_ERR_FLAGS
     assert call(flags=0x30) == _l3lib.L3_ERR_FLAGS          # both prefill bits: no such form
+    assert call(flags=0xc) == _l3lib.L3_ERR_FLAGS           # both form bits
     assert call(out=None) == _l3lib.L3_ERR_NULL_POINTER
     assert call(HD=96) == _l3lib.L3_ERR_HEAD_SIZE
     assert call(QH=40) == _l3lib.L3_ERR_HEAD_RATIO      # ratio 5
