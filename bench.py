@@ -50,18 +50,18 @@ MIN_TIMED_S = 0.05
 # this file (the summaries, their commands and the copy-kernel calibration are under profiles/).
 # An entry is reported only while the split plan it was measured with is the plan of this run.
 MEASURED_TRAFFIC = {
-    "c2": {"bytes": 39390000, "plan": [8, 16, 32, 32, 32, 171, 205],
+    "c2": {"bytes": 39390000, "plan": [8, 16, 32, 32, 32, 171, 205], "flags": 0,
            "profile": "profiles/attn_splitkv_mfma_c2_sweep_hbm_traffic.md"},
-    "c3a": {"bytes": 136660000, "plan": [1], "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
-    "c3b": {"bytes": 135870000, "plan": [11], "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
-    "rms": {"bytes": 67250000, "plan": None, "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
-    "rope": {"bytes": 68200000, "plan": None, "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
+    "c3a": {"flags": 2, "bytes": 136660000, "plan": [1], "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
+    "c3b": {"flags": 2, "bytes": 135870000, "plan": [11], "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
+    "rms": {"flags": 2, "bytes": 67250000, "plan": None, "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
+    "rope": {"flags": 2, "bytes": 68200000, "plan": None, "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
 }
 
 
 def measured_traffic(name, plan=None):
     rec = MEASURED_TRAFFIC.get(name)
-    if rec is None or ATTN_FLAGS or FORCE_SPLITS or (rec["plan"] is not None and rec["plan"] != plan):
+    if rec is None or (ATTN_FLAGS & ~rec.get("flags", 0)) or FORCE_SPLITS or (rec["plan"] is not None and rec["plan"] != plan):
         return None, None
     return rec["bytes"], rec["profile"]
 
@@ -309,6 +309,31 @@ def measure_read_stream(torch, lib, dev, pool, chunk_bytes=128 << 20):
             "kernel": "hbm_read_stream_kernel (16-byte non-temporal loads, no stores, no arithmetic)"}
 
 
+def measure_rw_stream(torch, lib, dev, nbytes):
+    """The read + write yardstick: the library's copy-through kernel (16-byte non-temporal loads, plain 16-byte
+    stores) over cold source / destination pairs of `nbytes` each, graph-replayed: what a row-wise operator
+    that reads and writes every element once can reach."""
+    nbytes = (nbytes + 255) // 256 * 256
+    copies = cold_slots(2 * nbytes, floor=2)
+    src = [torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(i & 0xff) for i in range(copies)]
+    dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(copies)]
+
+    def walk():
+        sp = torch.cuda.current_stream().cuda_stream
+        for a, b in zip(src, dst):
+            rc = lib.l3_hbm_rw_stream(a.data_ptr(), b.data_ptr(), nbytes, 0, sp)
+            if rc != 0:
+                raise RuntimeError(f"l3_hbm_rw_stream failed: {rc}")
+    walk()
+    gph = capture_graph(torch, walk)
+    ms, reps = timed_replays(torch, gph)
+    ms /= copies
+    del gph
+    gbps = 2 * nbytes / (ms * 1e-3) / 1e9
+    return {"bytes_read_and_written": 2 * nbytes, "us": round(ms * 1e3, 3), "GBps": round(gbps, 1),
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "launches_timed": reps * copies}
+
+
 ATTN_WORKLOADS = {
     # name: (B, HD, KV lengths, label)
     "c2": (1, 128, [512, 1024, 2048, 4096, 8192, 16384, 32768],
@@ -365,21 +390,47 @@ def run_attention(args, torch, lib, l3, dev, name, pool):
         }
 
     one_pass(0)
-    graph = capture_graph(torch, lambda: [one_pass(s) for s in range(passes)])
-    # the headline: wall clock around the replays, device synchronised on both sides; at least
-    # args.steps passes and at least MIN_TIMED_S, after at least MIN_WARM_S (and args.warmup passes) untimed
-    for _ in range((args.warmup + passes - 1) // passes):
-        graph.replay()
-    ms_graph, reps = timed_replays(torch, graph, min_replays=(args.steps + passes - 1) // passes, wall=True)
-    steps = reps * passes
-    ms_per_step = ms_graph / passes
-    value = pass_bytes / (ms_per_step * 1e-3) / 1e9
-    # HIP-event timing of the same replays (events on the stream the kernels run on)
-    ev_ms = event_time_ms(torch, graph.replay, reps) / passes
-    op_gbps = pass_bytes / (ev_ms * 1e-3) / 1e9
-    del graph
+    # The headline: exactly args.steps passes, wall clock with a device synchronisation on both sides, after at
+    # least args.warmup passes and MIN_WARM_S untimed.  The passes are recorded in HIP graphs (launch-bound
+    # otherwise): a main graph of a whole number of rotations over the K/V copies, replayed, plus one shorter
+    # graph for the remainder, so that the copies keep their order across replays.
+    g_passes = passes * max(1, min(args.steps, 512) // passes) if args.steps >= passes else 0
+    n_main = args.steps // g_passes if g_passes else 0
+    rem = args.steps - n_main * g_passes
+    main_graph = capture_graph(torch, lambda: [one_pass(s) for s in range(g_passes)]) if g_passes else None
+    rem_graph = capture_graph(torch, lambda: [one_pass(n_main * g_passes + s) for s in range(rem)]) if rem else None
 
-    # The dominant kernel on its own: the split-KV stage of every length, same regions, graph-replayed.
+    def timed_region():
+        for _ in range(n_main):
+            main_graph.replay()
+        if rem_graph is not None:
+            rem_graph.replay()
+
+    t_warm, warmed = time.perf_counter(), 0
+    while time.perf_counter() - t_warm < MIN_WARM_S or warmed < args.warmup:
+        timed_region()
+        torch.cuda.synchronize()
+        warmed += args.steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    timed_region()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    steps = args.steps
+    ms_per_step = wall_ms / steps
+    value = pass_bytes / (ms_per_step * 1e-3) / 1e9
+    # HIP-event timing of the same launches (events on the stream the kernels run on), over at least MIN_TIMED_S
+    ev_reps = max(1, int(math.ceil(MIN_TIMED_S * 1e3 / max(wall_ms, 1e-3))))
+    ev_ms = event_time_ms(torch, timed_region, ev_reps) / steps
+    op_gbps = pass_bytes / (ev_ms * 1e-3) / 1e9
+    del main_graph, rem_graph
+
+    # The dominant kernel on its own.  Where every length of the sweep runs as ONE launch (the split kernel
+    # merges its partials itself) that kernel is the whole call, timed above; otherwise the split-KV stage of
+    # every length (l3_attn_split: the same kernel writing partials only), same regions, graph-replayed.
+    plan = [c.num_splits for c in cases]
+    single_launch = [bool(lib.l3_attn_launches(B, QH, KVH, c.S, HD, c.req_splits, c.flags) == 1) for c in cases]
+
     def split_pass(slot):
         sp = torch.cuda.current_stream().cuda_stream
         for c in cases:
@@ -389,10 +440,10 @@ def run_attention(args, torch, lib, l3, dev, name, pool):
     sgraph = capture_graph(torch, lambda: [split_pass(s) for s in range(passes)])
     sms, sreps = timed_replays(torch, sgraph)
     split_ms = sms / passes
-    achieved = pass_bytes / (split_ms * 1e-3) / 1e9
-    split_kernel = "attn_splitkv_mfma_kernel" if attn_kernel_name() == "mfma" else "attn_splitkv_fma_kernel"
     del sgraph
-    plan = [c.num_splits for c in cases]
+    kernel_ms = ev_ms if all(single_launch) else split_ms
+    achieved = pass_bytes / (kernel_ms * 1e-3) / 1e9
+    split_kernel = "attn_splitkv_mfma_kernel" if attn_kernel_name() == "mfma" else "attn_splitkv_fma_kernel"
     traffic, traffic_src = measured_traffic(name, plan)
     del cases
 
@@ -420,18 +471,23 @@ def run_attention(args, torch, lib, l3, dev, name, pool):
     return {
         "metric": "decode_attn_hbm_GBps", "value": round(value, 1), "unit": "GB/s",
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-        "steps": steps, "steps_requested": args.steps, "ms_per_step": round(ms_per_step, 5), "dtype": "bf16",
+        "steps": steps, "ms_per_step": round(ms_per_step, 5), "dtype": "bf16",
         "config": {"workload": label, "kv_regions_per_length": passes, "cold_bytes_between_reuse": COLD_BYTES,
                    "accumulate": "f32", "launch": "hip graph", "seed": SEED,
-                   "timed_region_s": round(ms_graph * reps / 1e3, 4)},
+                   "timed_region_s": round(wall_ms / 1e3, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_profile": traffic_src,
                      "kernel": split_kernel, "launches_per_pass": len(lengths), "split_plan": plan,
-                     "avg_launch_us": round(split_ms * 1e3 / len(lengths), 3), "launches_timed": sreps * passes * len(lengths),
+                     "single_launch": single_launch,
+                     "timed_as": ("the whole call (one launch per length: the kernel merges its partials itself)"
+                                  if all(single_launch) else "the split stage alone (l3_attn_split)"),
+                     "avg_launch_us": round(kernel_ms * 1e3 / len(lengths), 3),
+                     "launches_timed": (ev_reps * steps if all(single_launch) else sreps * passes) * len(lengths),
                      "algorithmic_bytes_per_launch": pass_bytes // len(lengths),
-                     "split_plus_combine_GBps": round(op_gbps, 1),
-                     "split_plus_combine_frac": round(op_gbps / HBM_PEAK_GBPS, 4)},
+                     "split_stage_only_avg_us": round(split_ms * 1e3 / len(lengths), 3),
+                     "whole_call_GBps": round(op_gbps, 1),
+                     "whole_call_frac": round(op_gbps / HBM_PEAK_GBPS, 4)},
         "cpu_baseline": cpu, "per_length": detail,
     }
 
@@ -498,6 +554,12 @@ def rows_record(torch, lib, l3, dev, name, B, T, width):
     rec.update({"us": round(ms * 1e3, 3), "GBps": round(nbytes / ms / 1e6, 1),
                 "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "bytes": nbytes, "copies": copies,
                 "cold": bool(nbytes * (copies - 1) >= COLD_BYTES), "launches_timed": reps * copies})
+    # the read + write yardstick on the same byte count, launched the same way
+    del xs, ys
+    if name != "rms":
+        del bufs
+    torch.cuda.empty_cache()
+    rec["rw_stream_us"] = measure_rw_stream(torch, lib, dev, nbytes // 2)["us"]
     rec["_keep"] = keep
     rec["_ms"] = ms
     return rec
@@ -776,6 +838,8 @@ def main():
     ap.add_argument("--e2e-batch", type=int, default=1)
     ap.add_argument("--attn-kernel", default="default", choices=["default", "mfma", "fma"],
                     help="split-KV kernel to measure (default: the library's choice)")
+    ap.add_argument("--two-launches", action="store_true",
+                    help="decode attention always as split kernel + combine kernel (no merge inside the split launch)")
     ap.add_argument("--splits", type=int, default=0, help="force the split count (0 = the library's choice)")
     ap.add_argument("--lengths", default="", help="comma-separated KV lengths replacing the workload's own (experiments)")
     ap.add_argument("--cache-len", type=int, default=0,
@@ -799,8 +863,12 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    # every attention workspace of this file starts with prepared arrival counters (l3_attn_workspace_init)
+    ATTN_FLAGS = l3.L3_ATTN_FLAG_WS_COUNTERS
     if args.attn_kernel == "fma":
-        ATTN_FLAGS = l3.L3_ATTN_FLAG_KERNEL_FMA
+        ATTN_FLAGS |= l3.L3_ATTN_FLAG_KERNEL_FMA
+    if args.two_launches:
+        ATTN_FLAGS |= l3.L3_ATTN_FLAG_TWO_LAUNCHES
     attn_opts = {"split_kv_kernel": attn_kernel_name()}
     attention = args.workload in ATTN_WORKLOADS
     default_line = args.workload == "c2" and not args.lengths and not args.single_shot and not args.cache_len
@@ -841,17 +909,22 @@ def main():
 
         res = llama_arch.bench_e2e(args, torch, dev, None if args.no_cpu_baseline else cpu_op_table())
 
-    line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
+    head = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
             "steps": res.pop("steps"), "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": res.pop("dtype"),
             "data": "synthetic", "config": res.pop("config")}
-    line.update(res)
     if attention:
-        line["config"].update(attn_opts)
+        head["config"].update(attn_opts)
+    # The line is ordered for a reader who keeps only its end: the bulky per-shape detail first, the contract
+    # keys and the summaries ("roofline" with one row per shape of the target, "cpu_baseline") last.
+    roofline, cpu = res.pop("roofline", None), res.pop("cpu_baseline", None)
+    line = dict(res)
     if default_line:
         # the read bandwidth a pure stream reaches here: the practical ceiling the fractions are read against
         rs = measure_read_stream(torch, lib, dev, pool)
-        line["roofline"]["practical_read_peak"] = rs
+        roofline["practical_read_peak"] = rs
+        points = [[f"hd128_b1_s{r['kv_len']}", r["us"], r["frac"], r.get("read_stream_us")] for r in line["per_length"]
+                  if r["kv_len"] >= 4096]
         if not args.no_extras:
             ns = north_star_extras(args, torch, lib, l3, dev, pool)
             ns["rms_norm"] = [public(r) for r in ns["rms_norm"]]
@@ -864,8 +937,21 @@ def main():
             ns["points"] = len(pts)
             ns["longer_kv_points_at_or_above_target"] = sum(r["frac"] >= target for r in ns["longer_kv_b1"])
             line["north_star"] = ns
+            points += [[f"hd64_b1_s{r['kv_len']}", r["us"], r["frac"], r.get("read_stream_us")] for r in ns["hd64_b1"]]
+            points += [[f"hd{r['HD']}_b1_s{r['kv_len']}", r["us"], r["frac"], r.get("read_stream_us")]
+                       for r in ns["longer_kv_b1"]]
+            points += [[k, ns[k]["us"], ns[k]["frac"], ns[k].get("read_stream_us")]
+                       for k in ("c1_b1_hd64_s256", "c3a_b256_hd64_s256", "c3b_b16_hd64_s4096")]
+            points += [[f"rms_norm_{r['rows']}x{r['C']}", r["us"], r["frac"], r.get("rw_stream_us")] for r in ns["rms_norm"]]
+            points += [[f"rot_embed_{r['tokens']}x{r['NH']}x{r['HD']}", r["us"], r["frac"], r.get("rw_stream_us")]
+                       for r in ns["rot_embed"]]
             # the next row after the hot path: causal prefill attention (compute-bound, against the MFMA peak)
             line["prefill"] = prefill_summary(torch, dev)
+        # one row per shape of the target: [shape, us per call (split + merge, HBM-cold), fraction of 8 TB/s,
+        # us of the yardstick on the same byte count -- the read stream for attention, read + write for the row operators]
+        roofline["points"] = points
+        roofline["points_columns"] = ["shape", "us", "frac_of_8TBps", "yardstick_us"]
+        roofline["points_at_or_above_0.70"] = sum(1 for pt in points if pt[2] >= 0.70)
         del pool
         torch.cuda.empty_cache()
         if not args.no_e2e:
@@ -875,6 +961,11 @@ def main():
 
             line["e2e"] = llama_arch.e2e_summary(torch, dev, cpu_ops=None if args.no_cpu_baseline else cpu_op_table())
             line["e2e_tokens_per_s"] = {k: v["tok_per_s"] for k, v in line["e2e"].items() if k.startswith("bs")}
+    line.update(head)
+    line["roofline"] = roofline
+    line["cpu_baseline"] = cpu
+    if "e2e_tokens_per_s" in line:
+        line["e2e_tokens_per_s"] = line.pop("e2e_tokens_per_s")
     line["device"] = torch.cuda.get_device_name(0)
     print(json.dumps(line), flush=True)
 

@@ -119,8 +119,9 @@ size_t l3_attn_decode_workspace_bytes(int B, int QH, int KVH, int S, int HD, int
  *   num_splits : 0 = automatic, otherwise 1..L3_ATTN_MAX_SPLITS (the kernel may use fewer
  *            when S is short); results do not depend on it beyond float32 rounding
  *   workspace : >= l3_attn_decode_workspace_bytes(...) bytes, 256-byte aligned; may be NULL
- *            when that size is 0.  Contents on entry are ignored; calls that share a
- *            workspace must not overlap in time.
+ *            when that size is 0.  Contents on entry are ignored (with L3_ATTN_FLAG_WS_COUNTERS: except
+ *            the counters at its start, see l3_attn_workspace_init); calls that share a workspace
+ *            must not overlap in time.
  * Supported: HD in {64, 128}, QH/KVH in {1, 2, 3, 4, 8}, S >= 1.
  */
 int l3_attn_decode(const void* q, const void* k, const void* v, void* out,
@@ -136,22 +137,25 @@ int l3_attn_decode(const void* q, const void* k, const void* v, void* out,
  * that finishes a head last does it, out of the L2 of the XCD all workgroups of that head were placed on --
  * so that no combine kernel is launched (the reference always launches two kernels: custom_kernels.cu:274-275).
  *   l3_attn_workspace_init  zeroes the counters on `stream` and, on the first call per device, runs a probe
- *       launch that confirms the placement rule the scheme rests on (workgroup i of a grid runs on XCD i % 8)
- *       and WAITS for it: call it at set-up, outside stream capture.  workspace: 256-byte aligned, at least
+ *       launch that confirms the placement rule the scheme rests on (the workgroups of a grid go to the 8
+ *       XCDs in turn, so workgroups whose ids agree modulo 8 share an XCD) and WAITS for it: call it at set-up, outside stream capture.  workspace: 256-byte aligned, at least
  *       L3_ATTN_COUNTER_BYTES.  Every later l3_attn_decode / l3_attn_decode_devlen call on that workspace must
  *       pass L3_ATTN_FLAG_WS_COUNTERS (sizes from l3_attn_decode_workspace_bytes with the same flag); the
  *       counters are zero again when a call's kernels have finished, nothing else may write them, and calls
  *       that share a workspace must not overlap in time.  Where the probe did not confirm the rule, or the
  *       grid of a call does not keep a head on one XCD (B x KVH not a multiple of 8, more than 32 splits,
- *       more than 1023 (batch, kv head) pairs), the call runs split kernel + combine as without the flag.
+ *       a plan of streaming workgroups, more than 1023 (batch, kv head) pairs), the call runs split kernel + combine as without the flag.
  *   l3_attn_merge_in_launch_available  1 when the probe has confirmed the rule on the current device.
- *   l3_attn_placement_errors  number of workgroups that found themselves on another XCD than the rule says
- *       since the counters were prepared (always 0 on a device that passed the probe; a diagnostic that
- *       synchronises): workspace = a prepared workspace, or NULL for l3_attn_decode_static's array.
+ *   l3_attn_launches  kernels an l3_attn_decode call with these arguments launches on the current device
+ *       right now: 1 (a single split, or the merge inside the split launch) or 2 (split kernel + combine).
+ *   l3_attn_placement_errors  number of (batch, kv head) merges whose arrivals did not all come from the
+ *       merging workgroup's XCD since the counters were prepared (every arrival carries its XCC_ID; always 0
+ *       on a device that passed the probe; a diagnostic that synchronises): workspace = a prepared workspace, or NULL for l3_attn_decode_static's array.
  */
 #define L3_ATTN_COUNTER_BYTES (128u << 10)
 int l3_attn_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 int l3_attn_merge_in_launch_available(void);
+int l3_attn_launches(int B, int QH, int KVH, int S, int HD, int num_splits, int flags);
 int64_t l3_attn_placement_errors(const void* workspace);
 
 /*
@@ -449,6 +453,14 @@ int l3_rot_embed_append(const void* qkv, const float* freq_table, void* q_out, v
  * No counterpart in the reference.
  */
 int l3_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups, void* stream);
+
+/*
+ * The second yardstick: the same sweep, but every 16 bytes read from `src` are written once to `dst`
+ * (both 16-byte aligned, `bytes` a multiple of 16, no overlap): `bytes` read plus `bytes` written per
+ * launch, which is the traffic of a row-wise operator such as the RMSNorm and the rotary embedding.
+ * No counterpart in the reference.
+ */
+int l3_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, void* stream);
 
 #ifdef __cplusplus
 }

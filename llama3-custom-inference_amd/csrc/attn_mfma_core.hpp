@@ -107,13 +107,19 @@ __device__ __forceinline__ float column_max(float x) {
 // final tile, plus the lane's 16-byte chunk), so the loop spends two vector instructions per load on
 // addresses.  Every tile but the last issues the next tile's loads unconditionally, which lets the
 // K wait leave the V loads in flight.
-template <int HD, int LOADS = 8, bool STREAM = false>
+// ROTATE: the tiles are taken in rotated order -- the wavefront's i-th tile is tile (first + rot + i step)
+// modulo the number of tiles between t_first0 (the first token of the whole range the workgroup shares;
+// t_first = t_first0 + first tiles) and t_end, so that workgroups whose ranges start a power of two apart
+// do not all begin at addresses a power of two apart.  The order does not change the result beyond
+// float32 rounding: the softmax state is order-free.
+template <int HD, int LOADS = 8, bool STREAM = false, bool ROTATE = false>
 __device__ __forceinline__ void mfma_tile_loop(const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
                                                int64_t k_head, int64_t v_head, int64_t k_st, int64_t v_st,
                                                unsigned char* slab,
                                                const bf16x8_t (&qfrag)[MfmaTile<HD>::KC], int t_first, int t_end,
                                                int step, int col_limit, int col_limit_min, float c,
-                                               f32x4_t (&O)[MfmaTile<HD>::NB], float& m_run, float& l_part) {
+                                               f32x4_t (&O)[MfmaTile<HD>::NB], float& m_run, float& l_part,
+                                               int t_first0 = 0, int rot = 0) {
     using T = MfmaTile<HD, LOADS>;
     static_assert(T::WT % 32 == 0, "a tile is a whole number of 32-token steps of the second product");
     constexpr int LPR = T::LPR, G = T::G, U = T::U, WT = T::WT, NG = T::NG, KC = T::KC, NB = T::NB, KS = T::KS;
@@ -156,9 +162,8 @@ __device__ __forceinline__ void mfma_tile_loop(const uint16_t* __restrict__ k, c
         }
     };
 
-    auto tile = [&](const int t0, auto has_next) {
+    auto tile = [&](const int t0, const int tn, auto has_next) {
         constexpr bool NEXT = decltype(has_next)::value;
-        const int tn = t0 + step;
         // ---- K tile -> slab; its registers are free again, so the next K tile starts loading
 #pragma unroll
         for (int u = 0; u < U; ++u) *reinterpret_cast<uint4*>(wr_k + u * G * KPITCH) = kr[u];
@@ -269,11 +274,30 @@ __device__ __forceinline__ void mfma_tile_loop(const uint16_t* __restrict__ k, c
     };
 
     if (t_first >= t_end) return;   // a wavefront without a tile keeps its empty softmax state
-    int t0 = t_first;
-    load_tile(kr, kh, k_pitch, krow, t0);
-    load_tile(vr, vh, v_pitch, vrow, t0);
-    for (; t0 + step < t_end; t0 += step) tile(t0, std::true_type{});
-    tile(t0, std::false_type{});
+    if constexpr (ROTATE) {
+        t_first0 = wave_uniform(t_first0);
+        const int tiles = (t_end - t_first0 + WT - 1) / WT;              // of the whole range
+        const int tstep = step / WT;
+        int left = (tiles - (t_first - t_first0) / WT + tstep - 1) / tstep;   // tiles of this wavefront (>= 1)
+        int idx = ((t_first - t_first0) / WT + wave_uniform(rot)) % tiles;
+        int t0 = t_first0 + idx * WT;
+        load_tile(kr, kh, k_pitch, krow, t0);
+        load_tile(vr, vh, v_pitch, vrow, t0);
+        for (; left > 1; --left) {
+            idx += tstep;
+            if (idx >= tiles) idx -= tiles;
+            const int tn = t_first0 + idx * WT;
+            tile(t0, tn, std::true_type{});
+            t0 = tn;
+        }
+        tile(t0, t0, std::false_type{});
+    } else {
+        int t0 = t_first;
+        load_tile(kr, kh, k_pitch, krow, t0);
+        load_tile(vr, vh, v_pitch, vrow, t0);
+        for (; t0 + step < t_end; t0 += step) tile(t0, t0 + step, std::true_type{});
+        tile(t0, t0, std::false_type{});
+    }
 }
 
 }  // namespace l3

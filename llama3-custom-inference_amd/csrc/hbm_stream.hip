@@ -32,7 +32,33 @@ hbm_read_stream_kernel(const uint4* __restrict__ src, int64_t n16, uint32_t* __r
     if (acc == 0x9e3779b9u) *sink = acc;   // keeps the loads; practically never taken
 }
 
+// The same sweep with every 16 bytes read written once to `dst`: what a row-wise operator (one read
+// and one write per element, no arithmetic to speak of) can reach.  Stores are plain, as in the operators.
+__global__ void __launch_bounds__(kStreamThreads)
+hbm_rw_stream_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n16) {
+    constexpr int64_t kBlock = int64_t(kStreamThreads) * kStreamUnroll;
+    for (int64_t base = int64_t(blockIdx.x) * kBlock; base < n16; base += int64_t(gridDim.x) * kBlock) {
+        uint4 v[kStreamUnroll];
+#pragma unroll
+        for (int u = 0; u < kStreamUnroll; ++u) {
+            const int64_t i = base + u * kStreamThreads + threadIdx.x;
+            v[u] = (i < n16) ? load16_stream(reinterpret_cast<const uint16_t*>(src + i)) : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int u = 0; u < kStreamUnroll; ++u) {
+            const int64_t i = base + u * kStreamThreads + threadIdx.x;
+            if (i < n16) dst[i] = v[u];
+        }
+    }
+}
+
 }  // namespace
+
+int launch_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, hipStream_t stream) {
+    hipLaunchKernelGGL(hbm_rw_stream_kernel, dim3(unsigned(workgroups)), dim3(kStreamThreads), 0, stream,
+                       static_cast<const uint4*>(src), static_cast<uint4*>(dst), int64_t(bytes / 16));
+    return int(hipGetLastError());
+}
 
 int launch_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups, hipStream_t stream) {
     hipLaunchKernelGGL(hbm_read_stream_kernel, dim3(unsigned(workgroups)), dim3(kStreamThreads), 0, stream,

@@ -202,9 +202,21 @@ AttnPlan attn_make_plan(int B, int KVH, int S, int HD, int requested, int num_cu
             // batch 1, 8 kv heads) and 13.6 instead of 14.2 us at 12288; from two tiles per wavefront on
             // (16384: 17.9 against 16.2 us) the streaming form's whole-row reads win (head size 64, whose
             // per-head rows are 128 bytes: from one tile per wavefront).
-            const int64_t coop_tiles = int64_t(HD == 128 ? kMfmaWaves * 3 / 2 : kMfmaWaves / 2) * wgs;
+            // When the last workgroup of a head can merge inside the launch (merge_in_launch, and a grid that
+            // keeps a head on one XCD), the cooperative form has no combine launch to pay for and stays ahead
+            // much longer: up to four tiles per wavefront at head size 128 (32768 tokens over 8 kv heads:
+            // 24.8 against 25.6 us; 65536: level, left to the streaming form), one at head size 64 (16384
+            // tokens: 10.0 against 11.1 us; 32768: level), and with short sequences a tile per workgroup at
+            // head size 64 (1024 tokens in 16 splits: 4.6 against 4.9 us in 8).
+            // (Not at head size 64 with eight kv heads per streaming workgroup and fewer than four workgroups
+            // per head: 16 sequences of 1024 tokens took 11.1 us in two cooperative splits against 10.2 us streamed.)
+            const bool merges = merge_in_launch && attn_mfma_can_merge_in_launch(B, KVH, true, 2);
+            const bool longer = merges && !(HD == 64 && wgs < 4 && KVH % kMfmaWaves == 0);
+            const int64_t tiles_per_wg = longer ? (HD == 128 ? 4 * kMfmaWaves : kMfmaWaves)
+                                                : (HD == 128 ? kMfmaWaves * 3 / 2 : kMfmaWaves / 2);
+            const int64_t coop_tiles = tiles_per_wg * wgs;
             if (tiles <= coop_tiles) {
-                int coop_splits = std::min(wgs, ceil_div(tiles, 2));
+                int coop_splits = std::min(wgs, (merges && HD == 64) ? tiles : ceil_div(tiles, 2));
                 if (coop_splits > L3_ATTN_MAX_SPLITS) coop_splits = L3_ATTN_MAX_SPLITS;
                 const int tps = ceil_div(ceil_div(S, coop_splits), tile) * tile;
                 plan.coop = true;
@@ -467,6 +479,19 @@ int l3_attn_workspace_init(void* workspace, size_t workspace_bytes, void* stream
 int l3_attn_merge_in_launch_available(void) {
     const int dev = current_device_index();
     return dev >= 0 && g_xcd_state[dev].load(std::memory_order_acquire) == 1;
+}
+
+int l3_attn_launches(int B, int QH, int KVH, int S, int HD, int num_splits, int flags) {
+    if (int rc = check_attn_shape(B, QH, KVH, S, HD); rc != L3_OK) return rc;
+    if (num_splits < 0 || num_splits > L3_ATTN_MAX_SPLITS) return L3_ERR_SPLITS;
+    if (!attn_flags_ok(flags)) return L3_ERR_FLAGS;
+    const int cus = (num_splits == 0) ? current_device_cus() : 0;
+    const AttnPlan plan = attn_make_plan(B, KVH, S, HD, num_splits, cus, attn_impl_of(flags),
+                                         flags & L3_ATTN_FLAG_FORM_MASK, attn_merge_in_launch_wanted(flags));
+    if (plan.num_splits == 1) return 1;
+    const bool merge = attn_merge_in_launch_wanted(flags) && l3_attn_merge_in_launch_available() &&
+                       attn_mfma_can_merge_in_launch(B, KVH, plan.coop, plan.num_splits);
+    return merge ? 1 : 2;
 }
 
 int64_t l3_attn_placement_errors(const void* workspace) {
@@ -880,6 +905,15 @@ int l3_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups
     if (workgroups > (1 << 20)) return L3_ERR_SHAPE;
     return launch_hbm_read_stream(src, bytes, sink, workgroups, static_cast<hipStream_t>(stream)) == 0 ? L3_OK
                                                                                                        : L3_ERR_HIP;
+}
+
+int l3_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, void* stream) {
+    if (!src || !dst) return L3_ERR_NULL_POINTER;
+    if (bytes == 0 || bytes % 16 != 0) return L3_ERR_SHAPE;
+    if (!aligned(src, 16) || !aligned(dst, 16)) return L3_ERR_ALIGNMENT;
+    if (workgroups <= 0) workgroups = 4 * current_device_cus();
+    if (workgroups > (1 << 20)) return L3_ERR_SHAPE;
+    return launch_hbm_rw_stream(src, dst, bytes, workgroups, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
 }
 
 }  // extern "C"

@@ -55,6 +55,7 @@ SIGNATURES = {
     ),
     "l3_attn_workspace_init": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "l3_attn_merge_in_launch_available": (ctypes.c_int, []),
+    "l3_attn_launches": (ctypes.c_int, [ctypes.c_int] * 7),
     "l3_attn_placement_errors": (ctypes.c_int64, [ctypes.c_void_p]),
     "l3_attn_decode_static": (
         ctypes.c_int,
@@ -174,6 +175,9 @@ SIGNATURES = {
     ),
     "l3_hbm_read_stream": (
         ctypes.c_int, [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p],
+    ),
+    "l3_hbm_rw_stream": (
+        ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p],
     ),
 }
 

@@ -205,6 +205,48 @@ def test_split_planning():
     assert cke.attention_num_splits(16, 8, 4096, 64) == 11
 
 
+def test_attention_flag_contexts_nest():
+    """A block that names one choice keeps what the enclosing block chose for the others."""
+    from custom_kernels.custom_kernels_extension import _attn_flags
+
+    fma, tiled, two = _l3lib.L3_ATTN_FLAG_KERNEL_FMA, _l3lib.L3_ATTN_FLAG_PREFILL_TILED, _l3lib.L3_ATTN_FLAG_TWO_LAUNCHES
+    assert _attn_flags.get() == 0
+    with cke.attention_flags(kernel="fma"):
+        with cke.attention_flags(prefill="tiled"):
+            assert _attn_flags.get() == fma | tiled
+            with cke.attention_flags(kernel="mfma", launches="two"):
+                assert _attn_flags.get() == tiled | two
+            assert _attn_flags.get() == fma | tiled
+        assert _attn_flags.get() == fma
+    with cke.attention_flags(prefill="wave"):
+        with cke.attention_flags(kernel="fma"):
+            assert _attn_flags.get() == fma | _l3lib.L3_ATTN_FLAG_PREFILL_WAVE
+    assert _attn_flags.get() == 0
+
+
+def test_single_launch_entry_points_argument_checks():
+    lib = _l3lib.load()
+    W, TWO, COOP = _l3lib.L3_ATTN_FLAG_WS_COUNTERS, _l3lib.L3_ATTN_FLAG_TWO_LAUNCHES, _l3lib.L3_ATTN_FLAG_FORM_COOP
+    assert lib.l3_attn_workspace_init(None, 1 << 20, None) == _l3lib.L3_ERR_NULL_POINTER
+    assert lib.l3_attn_workspace_init(FAKE, _l3lib.L3_ATTN_COUNTER_BYTES - 1, None) == _l3lib.L3_ERR_WORKSPACE
+    assert lib.l3_attn_workspace_init(FAKE + 8, 1 << 20, None) == _l3lib.L3_ERR_ALIGNMENT
+    # the counters come on top of the partials, and only when the plan has more than one split
+    base = lib.l3_attn_decode_workspace_bytes(1, 32, 8, 4096, 128, 7, 0)
+    assert lib.l3_attn_decode_workspace_bytes(1, 32, 8, 4096, 128, 7, W) == base + _l3lib.L3_ATTN_COUNTER_BYTES
+    assert lib.l3_attn_decode_workspace_bytes(1, 32, 8, 200, 64, 1, W) == 0
+    # with the counters the plan keeps cooperative workgroups (at most 32 splits) where it used to stream
+    assert lib.l3_attn_choose_splits(1, 8, 16384, 128, 256, 0) == 171
+    assert lib.l3_attn_choose_splits(1, 8, 16384, 128, 256, W) == 32
+    assert lib.l3_attn_choose_splits(1, 8, 16384, 128, 256, W | TWO) == 171
+    assert lib.l3_attn_choose_splits(1, 3, 16384, 128, 256, W) == lib.l3_attn_choose_splits(1, 3, 16384, 128, 256, 0)
+    # no device has been probed in this process: two launches whatever the flags; one split is one launch
+    assert lib.l3_attn_launches(1, 32, 8, 4096, 128, 0, W) == 2
+    assert lib.l3_attn_launches(1, 32, 8, 200, 64, 0, W) == 1
+    assert lib.l3_attn_launches(1, 32, 8, 4096, 128, 600, W) == _l3lib.L3_ERR_SPLITS
+    assert lib.l3_attn_launches(1, 32, 8, 4096, 128, 4, COOP | _l3lib.L3_ATTN_FLAG_FORM_STREAM) == _l3lib.L3_ERR_FLAGS
+    assert lib.l3_attn_merge_in_launch_available() == 0
+
+
 def test_shim_rejects_cpu_tensors_and_has_no_fallback():
     import torch
 

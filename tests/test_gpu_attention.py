@@ -229,27 +229,45 @@ def test_runs_on_the_current_stream(gpu):
 
 
 # ---- the benchmark configurations at full size (oracle in float64, chunked over the batch)
+# name: (B, QH, KVH, S, HD, splits the MFMA plan makes on 256 compute units when the workspace carries
+# arrival counters, launches of that plan).  Every shape the benchmark line reports is here at its own size.
 FULL = {
-    "c1": (1, 32, 8, 256, 64),
-    "c2_s512": (1, 32, 8, 512, 128),
-    "c2_s4096": (1, 32, 8, 4096, 128),
-    "c2_s32768": (1, 32, 8, 32768, 128),
-    "c3a": (256, 32, 8, 256, 64),
-    "c3b": (16, 32, 8, 4096, 64),
+    "c1": (1, 32, 8, 256, 64, 1, 1),
+    "c2_s512": (1, 32, 8, 512, 128, 8, 1),
+    "c2_s1024": (1, 32, 8, 1024, 128, 16, 1),
+    "c2_s2048": (1, 32, 8, 2048, 128, 32, 1),
+    "c2_s4096": (1, 32, 8, 4096, 128, 32, 1),
+    "c2_s8192": (1, 32, 8, 8192, 128, 32, 1),
+    "c2_s16384": (1, 32, 8, 16384, 128, 32, 1),
+    "c2_s32768": (1, 32, 8, 32768, 128, 32, 1),
+    "hd128_s65536": (1, 32, 8, 65536, 128, 205, 2),
+    "hd64_s4096": (1, 32, 8, 4096, 64, 32, 1),
+    "hd64_s8192": (1, 32, 8, 8192, 64, 32, 1),
+    "hd64_s16384": (1, 32, 8, 16384, 64, 32, 1),
+    "hd64_s32768": (1, 32, 8, 32768, 64, 171, 2),
+    "hd64_s65536": (1, 32, 8, 65536, 64, 205, 2),
+    "c3a": (256, 32, 8, 256, 64, 1, 1),
+    "c3b": (16, 32, 8, 4096, 64, 11, 2),
 }
 
 
 @pytest.mark.parametrize("name", list(FULL))
-def test_baseline_shapes_full_size(gpu, name):
+def test_baseline_shapes_full_size(gpu, attn_kernel, name):
+    from custom_kernels import _l3lib
     from custom_kernels import custom_kernels_extension as cke
 
-    B, QH, KVH, S, HD = FULL[name]
+    B, QH, KVH, S, HD, plan_splits, plan_launches = FULL[name]
     print(f"full-size {name}: B={B} S={S} HD={HD}", flush=True)
+    if attn_kernel == "mfma":
+        # the test follows the plan: these are the split counts and launch counts the benchmark line reports
+        W = _l3lib.L3_ATTN_FLAG_WS_COUNTERS
+        assert cke.attention_num_splits(B, KVH, S, HD, 256, flags=W) == plan_splits
+        if torch.cuda.get_device_properties(gpu).multi_processor_count == 256:
+            assert _l3lib.load().l3_attn_launches(B, QH, KVH, S, HD, 0, W) == plan_launches
     q, k, v = make_qkv(B, QH, KVH, S, HD, seed=42)
     qg, kg, vg = make_qkv(B, QH, KVH, S, HD, seed=42, device=gpu)
     out = cke.flash_attention_decode(qg, kg, vg)
     torch.cuda.synchronize()
-    out_f = t2f32(out)
     worst = 0.0
     for b0 in range(0, B, 32):
         sl = slice(b0, min(B, b0 + 32))
