@@ -458,9 +458,11 @@ int l3_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups
  * The second yardstick: the same sweep, but every 16 bytes read from `src` are written once to `dst`
  * (both 16-byte aligned, `bytes` a multiple of 16, no overlap): `bytes` read plus `bytes` written per
  * launch, which is the traffic of a row-wise operator such as the RMSNorm and the rotary embedding.
+ * block_kib: what a workgroup moves per trip, 8, 16, 32 or 64 KiB (0 = 64); which is fastest depends on
+ * how the buffer divides over the compute units, so the benchmark takes the best of the four.
  * No counterpart in the reference.
  */
-int l3_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, void* stream);
+int l3_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, int block_kib, void* stream);
 
 #ifdef __cplusplus
 }

@@ -55,28 +55,34 @@ __device__ __forceinline__ bool arrive_is_last(unsigned* counter, int n, bool* s
 __device__ __forceinline__ void wait_stores_in_l2() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Loads of partials another compute unit wrote during this launch: buffer loads with sc0, which
-// miss the vector L1 and read the XCD's L2.  `base` is wave-uniform; offsets are bytes.
+// miss the vector L1 and read the XCD's L2.  `base` and `limit_bytes` are wave-uniform; offsets are
+// bytes; a 16-byte load that reaches past `limit_bytes` touches no memory and returns zeros.
 struct L2Reader {
     __amdgpu_buffer_rsrc_t rsrc;
     const char* base;
-    __device__ __forceinline__ explicit L2Reader(const void* b)
-        : rsrc(__builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(b), 0, 0x7fffffff, 0x00020000)),
+    __device__ __forceinline__ L2Reader(const void* b, uint32_t limit_bytes)
+        : rsrc(__builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(b), 0, int(limit_bytes), 0x00020000)),
           base(static_cast<const char*>(b)) {}
-    __device__ __forceinline__ f32x4v load16(uint32_t byte_off) const {
-        return __builtin_bit_cast(f32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, int(byte_off), 0, 1));
+    __device__ __forceinline__ f32x4v load16(uint32_t lane_off, uint32_t uniform_off) const {
+        return __builtin_bit_cast(f32x4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, int(lane_off), int(uniform_off), 1));
     }
-    // (an 8-byte load with the same policy: what a workgroup-scope atomic load compiles to on this target)
+    // (an 8-byte load with the same policy: what a workgroup-scope atomic load compiles to on this target;
+    // the caller keeps the offset inside the buffer)
     __device__ __forceinline__ float2 load8(uint32_t byte_off) const {
         const uint64_t bits = __hip_atomic_load(reinterpret_cast<const uint64_t*>(base + byte_off), __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_WORKGROUP);
         return make_float2(__builtin_bit_cast(float, uint32_t(bits)), __builtin_bit_cast(float, uint32_t(bits >> 32)));
     }
 };
+// Ordinary loads (a kernel of its own reads what an earlier kernel wrote): a 16-byte load past
+// `limit_bytes` is moved back onto the last 16 bytes inside (its row has weight zero).
 struct PlainReader {
     const char* base;
-    __device__ __forceinline__ explicit PlainReader(const void* b) : base(static_cast<const char*>(b)) {}
-    __device__ __forceinline__ f32x4v load16(uint32_t byte_off) const {
-        return *reinterpret_cast<const f32x4v*>(base + byte_off);
+    uint32_t last;
+    __device__ __forceinline__ PlainReader(const void* b, uint32_t limit_bytes)
+        : base(static_cast<const char*>(b)), last(limit_bytes - 16u) {}
+    __device__ __forceinline__ f32x4v load16(uint32_t lane_off, uint32_t uniform_off) const {
+        return *reinterpret_cast<const f32x4v*>(base + min(lane_off + uniform_off, last));
     }
     __device__ __forceinline__ float2 load8(uint32_t byte_off) const {
         return *reinterpret_cast<const float2*>(base + byte_off);
@@ -128,85 +134,70 @@ __device__ __forceinline__ float segment_reduce(float x) {
 }
 
 // One wavefront merges the n >= 1 partial rows po[i][HD] with statistics ml[i] = (max in log2
-// units, sum) of NP (batch, query head) pairs and writes their bf16 output rows -- or, with
-// CG > 1, column group cg of them (HD / CG columns), so that CG wavefronts share a pair and each
-// pulls 1 / CG of the bytes.  Pair j's rows start pair_rows * j rows after po / ml, its output
-// out_stride elements after out_row; pairs >= np are skipped.
+// units, sum) of one (batch, query head) pair and writes the bf16 output row -- or, with CG > 1,
+// column group cg of it (HD / CG columns), so that CG wavefronts share a pair and each pulls
+// 1 / CG of the bytes.
 // A wavefront-wide memory instruction costs the compute unit 16 cycles whatever its width, and the
 // last arriver of a head has nothing to overlap them with, so the merge is built from as few as
-// possible, all requested in one round trip before any weight is known: ONE load of statistics
-// (lane l holds row l % (64 / NP) of pair l / (64 / NP)) and 16-byte loads of the rows.  Weights
+// possible, all requested in one round trip before any weight is known and with nothing but a
+// constant between one request and the next: ONE load of statistics (lane l < 32 holds split l of
+// the pass) and 16-byte loads of the rows, whose lanes past the last split read zeros.  Weights
 // are formed in the statistics lanes and handed to the lanes that hold the rows through the LDS
-// crossbar; lanes that hold the same columns meet in coset_reduce.  More than NR splits take
+// crossbar; lanes that hold the same columns meet in coset_reduce.  More than 32 splits take
 // further passes with a running maximum.  All arguments are wave-uniform.
-template <int HD, typename Reader, int CG = 1, int NP = 1, int NR = kCombineRows>
+template <int HD, typename Reader, int CG = 1>
 __device__ __forceinline__ void merge_pair_rows(const float* __restrict__ po, const float2* __restrict__ ml, int n,
-                                                uint16_t* __restrict__ out_row, int cg = 0, int np = NP, int64_t pair_rows = 0, int64_t out_stride = 0) {
+                                                uint16_t* __restrict__ out_row, int cg = 0) {
+    constexpr int NR = kCombineRows;
     constexpr int RQ = HD / 4;              // 16-byte pieces of a whole partial row
     constexpr int TPR = RQ / CG;            // lanes covering this wavefront's columns of a row
     constexpr int RPL = kWaveSize / TPR;    // rows per wavefront-wide load
-    constexpr int NLD = NR / RPL;           // row loads per pair and pass
-    constexpr int SEG = kWaveSize / NP;     // statistics lanes per pair
+    constexpr int NLD = NR / RPL;           // row loads per pass
     static_assert(TPR >= 1 && kWaveSize % TPR == 0 && NR % RPL == 0 && NLD >= 1, "rows must divide over the lanes");
-    static_assert(SEG >= NR && SEG >= 16, "one lane per (pair, split) in the statistics load");
     const int lane = threadIdx.x & (kWaveSize - 1);
     const int dq = cg * TPR + lane % TPR;
     const int sub = lane / TPR;
-    const int sj = lane / SEG;              // as a statistics lane: pair ...
-    const int sr = lane % SEG;              // ... and split within the pass
-    const Reader rows(po), stats(ml);
+    const Reader rows(po, uint32_t(n) * uint32_t(HD * 4)), stats(ml, uint32_t(n) * 8u);
+    const uint32_t lane_off = uint32_t(sub * RQ + dq) * 16u;
 
-    float m_w = kMaskedScore, l_w = 0.f;    // running statistics of pair sj (uniform over its segment)
-    f32x4v acc[NP];
-#pragma unroll
-    for (int j = 0; j < NP; ++j) acc[j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    float m_w = kMaskedScore, l_w = 0.f;    // running statistics (the same in every lane)
+    f32x4v acc = {0.f, 0.f, 0.f, 0.f};
     for (int r0 = 0; r0 < n; r0 += NR) {
         // (unconditional, from a clamped index: a load inside a divergent branch would be waited for there)
-        float2 st = stats.load8(uint32_t(min(sj, np - 1) * pair_rows + min(r0 + sr, n - 1)) * 8u);
-        if (sr >= NR || r0 + sr >= n || sj >= np) st = make_float2(kMaskedScore, 0.f);
-        f32x4v x[NP][NLD];
+        float2 st = stats.load8(uint32_t(min(r0 + lane, n - 1)) * 8u);
+        if (lane >= NR || r0 + lane >= n) st = make_float2(kMaskedScore, 0.f);
+        f32x4v x[NLD];
 #pragma unroll
-        for (int j = 0; j < NP; ++j) {
-#pragma unroll
-            for (int u = 0; u < NLD; ++u) {
-                x[j][u] = f32x4v{0.f, 0.f, 0.f, 0.f};
-                if (j < np && r0 + u * RPL < n) {   // wavefront-uniform: nothing is requested past the last split
-                    const int r = min(r0 + u * RPL + sub, n - 1);   // a row past the end gets weight 0 below
-                    x[j][u] = rows.load16(uint32_t((j * pair_rows + r) * RQ + dq) * 16u);
-                }
-            }
+        for (int u = 0; u < NLD; ++u) {
+            x[u] = f32x4v{0.f, 0.f, 0.f, 0.f};
+            // wavefront-uniform: nothing is requested past the last split
+            if (r0 + u * RPL < n) x[u] = rows.load16(lane_off, uint32_t(r0 + u * RPL) * uint32_t(HD * 4));
         }
-        const float m_new = fmaxf(m_w, segment_reduce<SEG, true>(st.x));
+        const float m_new = fmaxf(m_w, segment_reduce<kWaveSize, true>(st.x));
         const float alpha = fast_exp2(m_w - m_new);
         const float wgt = fast_exp2(st.x - m_new);   // absent splits: 2^(-1e30 - m) = 0
-        l_w = fmaf(l_w, alpha, segment_reduce<SEG, false>(st.y * wgt));
+        l_w = fmaf(l_w, alpha, segment_reduce<kWaveSize, false>(st.y * wgt));
         m_w = m_new;
+        if (r0 > 0) acc *= alpha;
 #pragma unroll
-        for (int j = 0; j < NP; ++j) {
-            if (r0 > 0) acc[j] *= __shfl(alpha, j * SEG, kWaveSize);
-#pragma unroll
-            for (int u = 0; u < NLD; ++u) {
-                const float w = __shfl(wgt, j * SEG + u * RPL + sub, kWaveSize);
-                acc[j].x = fmaf(w, x[j][u].x, acc[j].x);
-                acc[j].y = fmaf(w, x[j][u].y, acc[j].y);
-                acc[j].z = fmaf(w, x[j][u].z, acc[j].z);
-                acc[j].w = fmaf(w, x[j][u].w, acc[j].w);
-            }
+        for (int u = 0; u < NLD; ++u) {
+            const float w = __shfl(wgt, u * RPL + sub, kWaveSize);
+            acc.x = fmaf(w, x[u].x, acc.x);
+            acc.y = fmaf(w, x[u].y, acc.y);
+            acc.z = fmaf(w, x[u].z, acc.z);
+            acc.w = fmaf(w, x[u].w, acc.w);
         }
     }
-#pragma unroll
-    for (int j = 0; j < NP; ++j) {
-        const float inv = 1.0f / __shfl(l_w, j * SEG, kWaveSize);
-        const float o0 = coset_reduce<TPR, false>(acc[j].x) * inv;
-        const float o1 = coset_reduce<TPR, false>(acc[j].y) * inv;
-        const float o2 = coset_reduce<TPR, false>(acc[j].z) * inv;
-        const float o3 = coset_reduce<TPR, false>(acc[j].w) * inv;
-        if (j < np && lane < TPR) {
-            uint2 packed;
-            packed.x = pack_bf16x2(o0, o1);
-            packed.y = pack_bf16x2(o2, o3);
-            *reinterpret_cast<uint2*>(out_row + j * out_stride + dq * 4) = packed;
-        }
+    const float inv = 1.0f / l_w;
+    const float o0 = coset_reduce<TPR, false>(acc.x) * inv;
+    const float o1 = coset_reduce<TPR, false>(acc.y) * inv;
+    const float o2 = coset_reduce<TPR, false>(acc.z) * inv;
+    const float o3 = coset_reduce<TPR, false>(acc.w) * inv;
+    if (lane < TPR) {
+        uint2 packed;
+        packed.x = pack_bf16x2(o0, o1);
+        packed.y = pack_bf16x2(o2, o3);
+        *reinterpret_cast<uint2*>(out_row + dq * 4) = packed;
     }
 }
 

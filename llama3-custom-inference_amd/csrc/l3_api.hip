@@ -907,13 +907,16 @@ int l3_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups
                                                                                                        : L3_ERR_HIP;
 }
 
-int l3_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, void* stream) {
+int l3_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, int block_kib, void* stream) {
     if (!src || !dst) return L3_ERR_NULL_POINTER;
     if (bytes == 0 || bytes % 16 != 0) return L3_ERR_SHAPE;
     if (!aligned(src, 16) || !aligned(dst, 16)) return L3_ERR_ALIGNMENT;
+    if (block_kib == 0) block_kib = 64;
+    if (block_kib != 8 && block_kib != 16 && block_kib != 32 && block_kib != 64) return L3_ERR_SHAPE;
     if (workgroups <= 0) workgroups = 4 * current_device_cus();
     if (workgroups > (1 << 20)) return L3_ERR_SHAPE;
-    return launch_hbm_rw_stream(src, dst, bytes, workgroups, static_cast<hipStream_t>(stream)) == 0 ? L3_OK : L3_ERR_HIP;
+    return launch_hbm_rw_stream(src, dst, bytes, workgroups, block_kib, static_cast<hipStream_t>(stream)) == 0 ? L3_OK
+                                                                                                               : L3_ERR_HIP;
 }
 
 }  // extern "C"

@@ -144,7 +144,7 @@ bool attn_mfma_can_merge_in_launch(int B, int KVH, bool coop, int num_splits);
 int launch_xcd_probe(unsigned* where, int n, int stride_words, hipStream_t stream);
 int launch_fill_zero_u32(unsigned* dst, size_t n, hipStream_t stream);
 int launch_hbm_read_stream(const void* src, size_t bytes, void* sink, int workgroups, hipStream_t stream);
-int launch_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, hipStream_t stream);
+int launch_hbm_rw_stream(const void* src, void* dst, size_t bytes, int workgroups, int block_kib, hipStream_t stream);
 int launch_rms_norm(const uint16_t* x, const uint16_t* w, uint16_t* y, int64_t rows, int C, float eps,
                     bool vec_ok, hipStream_t stream);
 int launch_add_rms_norm(const uint16_t* x, const uint16_t* res, const uint16_t* w, uint16_t* sum_out, uint16_t* y,

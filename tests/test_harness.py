@@ -235,6 +235,28 @@ def test_full_size_logits_match_cpu_model(gpu, full_size_model):
 
 
 @pytest.mark.gpu
+def test_full_size_logits_match_cpu_model_on_the_split_k_route(gpu, full_size_model):
+    """Batch 5 is the first batch size whose output and down projections take the split-K kernels (float32
+    partial products summed by the operator that follows) and whose qkv / gate|up linears run with more than
+    four activation rows: a 16-token prompt and two decode steps at the 1B shape against the float32 CPU
+    model, within 4 % of the logit range."""
+    dut = full_size_model
+    assert la.LlamaDecoder.FUSED_MAX_ROWS < 5 <= la.LlamaDecoder.QKV_FUSED_MAX_ROWS
+    cfg = la.LlamaConfig(max_model_len=256, max_gen_batch_size=5)
+    ref = la.LlamaDecoder(cfg, CpuOps, "cpu", dtype=torch.float32, weights_from=dut)
+    ids = torch.tensor(la.random_prompts(5, 18, cfg.vocab_size, 23))
+    with torch.inference_mode():
+        for (lo, hi, sp) in [(0, 16, 0), (16, 17, 16), (17, 18, 17)]:
+            print(f"full-size logits, batch 5: tokens {lo}..{hi} at {sp}", flush=True)
+            a = ref.forward(ids[:, lo:hi], start_pos=sp)
+            b = dut.forward(ids[:, lo:hi].to(gpu), start_pos=sp).cpu()
+            scale = a.abs().max().item()
+            err = (a - b).abs().max().item()
+            assert err <= 0.04 * scale, f"step at {sp}: logits differ by {err} (scale {scale})"
+    del ref
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("batch", [1, 64])
 def test_full_size_graphed_loop_matches_eager(gpu, full_size_model, batch):
     """128 prompt ids + 128 greedy tokens at batch 1 (fused single-launch linears) and batch 64
@@ -255,7 +277,7 @@ def test_full_size_graphed_loop_matches_eager(gpu, full_size_model, batch):
             if x != y:
                 break
             common += 1
-        assert common >= 16, f"graphed and eager streams diverge after {common} tokens"
+        assert common >= 100, f"graphed and eager streams diverge after {common} tokens"
         agree += common
         total += len(a)
-    assert agree >= 0.8 * total, f"only {agree} of {total} tokens lie in common prefixes"
+    assert agree >= 0.98 * total, f"only {agree} of {total} tokens lie in common prefixes"
