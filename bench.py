@@ -899,11 +899,11 @@ def main():
     elif args.workload == "copy":
         res = run_copy(args, torch, dev)
     elif args.workload == "readstream":
-        rs = {str(mb): measure_read_stream(torch, lib, dev, pool, mb << 20) for mb in (16, 64, 128, 512)}
+        rs = {str(mb): measure_read_stream(torch, lib, dev, pool, mb << 20) for mb in (16, 32, 64, 128, 256, 512)}
         head = rs["128"]
         res = {"metric": "read_stream_hbm_GBps", "value": head["GBps"], "unit": "GB/s", "frac_of_hbm_peak": head["frac"],
                "steps": head["launches_timed"], "ms_per_step": round(head["us"] / 1e3, 5), "dtype": "u8",
-               "config": {"workload": "pure read stream over a 1 GiB pool in chunks of 128 MiB (16 / 64 / 512 MiB beside it), "
+               "config": {"workload": "pure read stream over a 1 GiB pool in chunks of 128 MiB (16 ... 512 MiB beside it), "
                                       "each chunk cold", "launch": "hip graph"},
                "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                             "frac": head["frac"], "traffic": None, "kernel": "hbm_read_stream_kernel",

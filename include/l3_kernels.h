@@ -161,18 +161,21 @@ int64_t l3_attn_placement_errors(const void* workspace);
 /*
  * l3_attn_decode for callers that cannot allocate device memory and have no workspace to pass
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the
- * float32 partials live in a static device array of L3_ATTN_STATIC_SCRATCH_BYTES inside the
- * library instead of a caller's workspace, and the call allocates and frees nothing.  It has no
- * counterpart in the reference, whose launcher allocates three temporaries per call
- * (custom_kernels.cu:269-271).  Same arguments, kernels and results (bit for bit) as
- * l3_attn_decode.  A problem whose plan needs more scratch than the array holds returns
- * L3_ERR_SCRATCH (size it with l3_attn_decode_workspace_bytes; every BASELINE shape needs under
- * 5 MiB).  Every GPU the library runs on holds its own copy of the array from the first call on
- * that GPU until the process ends; the address is looked up once per device on that first call,
- * so make one call outside stream capture first.  All calls on one GPU share the array: calls
- * that overlap in time on the same GPU (different streams or threads) race.  Nothing in the
- * array has to start at zero -- every row a combine reads was written by the same call's split
- * kernel -- so the previous call's contents are simply overwritten.
+ * float32 partials and the arrival counters live in a static device array of
+ * L3_ATTN_STATIC_SCRATCH_BYTES inside the library instead of a caller's workspace, and the call
+ * allocates and frees nothing.  It has no counterpart in the reference, whose launcher allocates
+ * three temporaries per call (custom_kernels.cu:269-271).  Same arguments, kernels and results (bit
+ * for bit) as l3_attn_decode with L3_ATTN_FLAG_WS_COUNTERS on a workspace prepared by
+ * l3_attn_workspace_init (the flag is implied here).  A problem whose plan needs more scratch than
+ * the array holds returns L3_ERR_SCRATCH (size it with l3_attn_decode_workspace_bytes and that flag;
+ * every BASELINE shape needs under 5 MiB).  Every GPU the library runs on holds its own copy of the
+ * array from the first call on that GPU until the process ends; on that first call the address is
+ * looked up and the placement probe of l3_attn_workspace_init runs (and is waited for), so make one
+ * call outside stream capture first.  All calls on one GPU share the array: calls that overlap in
+ * time on the same GPU (different streams or threads) race.  The counters at its start are zero when
+ * the library is loaded and every call leaves them at zero; the partial rows need no clearing --
+ * every row a merge reads was written by the same call -- so the previous call's contents are
+ * simply overwritten.
  */
 #define L3_ATTN_STATIC_SCRATCH_BYTES (16u << 20)
 int l3_attn_decode_static(const void* q, const void* k, const void* v, void* out,

@@ -1,7 +1,8 @@
-"""l3_attn_decode_static -- decode attention whose partials live in the library's static device
-array, so that the call allocates nothing -- against l3_attn_decode with a caller's workspace,
-through the C ABI.  Same plan and kernels, so the outputs must agree bit for bit; two calls in a
-row, the second on a smaller problem, show that what the first call left in the array does no harm."""
+"""l3_attn_decode_static -- decode attention whose partials and arrival counters live in the library's
+static device array, so that the call allocates nothing -- against l3_attn_decode with a caller's
+prepared workspace (l3_attn_workspace_init, L3_ATTN_FLAG_WS_COUNTERS), through the C ABI.  Same plan
+and kernels, so the outputs must agree bit for bit; two calls in a row, the second on a smaller
+problem, show that what the first call left in the array does no harm."""
 
 import math
 
@@ -24,17 +25,28 @@ def _both(lib, dev, B, QH, KVH, S, HD, seed, splits=0):
     q, k, v = make_qkv(B, QH, KVH, S, HD, seed=seed, cache_len=S + 37, device=dev)
     scale = 1.0 / math.sqrt(HD)
     stream = torch.cuda.current_stream().cuda_stream
-    ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, splits, 0)
-    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+    from custom_kernels import _l3lib
+
+    W = _l3lib.L3_ATTN_FLAG_WS_COUNTERS
+    ws_bytes = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, splits, W)
+    ws = torch.empty(max(ws_bytes, _l3lib.L3_ATTN_COUNTER_BYTES), dtype=torch.uint8, device=dev)
+    assert lib.l3_attn_workspace_init(ws.data_ptr(), ws.numel(), stream) == 0
     want = torch.full_like(q, float("nan"))
     got = torch.full_like(q, float("nan"))
-    args = (B, QH, KVH, S, HD, _strides(q, 2), _strides(k, 3), _strides(v, 3), _strides(want, 2), scale, splits, 0, stream)
-    rc = lib.l3_attn_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), want.data_ptr(), ws.data_ptr(), ws_bytes, *args)
+    plain = torch.full_like(q, float("nan"))
+    shape = (B, QH, KVH, S, HD, _strides(q, 2), _strides(k, 3), _strides(v, 3), _strides(want, 2), scale, splits)
+    rc = lib.l3_attn_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), want.data_ptr(), ws.data_ptr(), ws_bytes,
+                            *shape, W, stream)
     assert rc == 0, rc
-    rc = lib.l3_attn_decode_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), got.data_ptr(), *args)
+    rc = lib.l3_attn_decode_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), got.data_ptr(), *shape, 0, stream)
+    assert rc == 0, rc
+    # the entry point without counters (always split kernel + combine kernel) on a workspace of its own
+    pb = lib.l3_attn_decode_workspace_bytes(B, QH, KVH, S, HD, splits, 0)
+    pws = torch.empty(max(pb, 256), dtype=torch.uint8, device=dev)
+    rc = lib.l3_attn_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), plain.data_ptr(), pws.data_ptr(), pb, *shape, 0, stream)
     assert rc == 0, rc
     torch.cuda.synchronize()
-    return want, got, ws_bytes, (q, k, v)
+    return want, got, plain, ws_bytes, (q, k, v)
 
 
 @pytest.mark.gpu
@@ -47,10 +59,12 @@ def test_static_scratch_entry_matches_the_workspace_entry(gpu):
     # it: a smaller problem (24 rows of partials) that lands on what the first one left there
     for (B, QH, KVH, S, HD, splits, seed) in ((1, 32, 8, 8192, 128, 0, 901), (2, 12, 4, 700, 64, 3, 902)):
         print(f"static scratch: B={B} QH={QH} KVH={KVH} S={S} HD={HD} splits={splits}", flush=True)
-        want, got, ws_bytes, (q, k, v) = _both(lib, gpu, B, QH, KVH, S, HD, seed, splits)
+        want, got, plain, ws_bytes, (q, k, v) = _both(lib, gpu, B, QH, KVH, S, HD, seed, splits)
         assert 0 < ws_bytes <= _l3lib.L3_ATTN_STATIC_SCRATCH_BYTES
         assert not torch.isnan(got.float()).any()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), "static scratch and workspace paths differ"
+        # against the two-launch form: another merge order of the same float32 partials, the last bf16 bit at most
+        assert (got.float() - plain.float()).abs().max().item() <= 2.0 ** -8 * max(1e-3, plain.float().abs().max().item())
         assert_attn_close(got, attention_decode_ref(t2f32(q.cpu()), t2f32(k.cpu()), t2f32(v.cpu())),
                           what="static scratch vs oracle", min_kv_len=S)
     # and through the Python operator, into the caller's output
