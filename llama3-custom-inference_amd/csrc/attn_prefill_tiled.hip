@@ -69,9 +69,18 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     const int wg_pos = NW * CB * ppw;                    // query positions per workgroup
     const int wgs_per_head = (p.T + wg_pos - 1) / wg_pos;
     const int heads = p.B * p.KVH;
-    // the workgroups with the longest token ranges are dispatched first
-    const int wg = wgs_per_head - 1 - int(blockIdx.x) / heads;
-    const int bh = int(blockIdx.x) % heads;
+    // The workgroups with the longest token ranges are dispatched first.  A launch that the device holds (almost)
+    // all at once gets no balancing from the dispatcher: workgroup r lands on compute unit r % snake, which
+    // would collect the longest block of every round.  Every second round of `snake` ranks is therefore taken
+    // in reverse, so that a unit's blocks add up to about the same length (2 x 2048 tokens at head size 64:
+    // 47.8 -> 45.3 us; launches of many rounds are left alone: -1 % there).
+    int rank = int(blockIdx.x);
+    if (p.snake > 0) {
+        const int k = rank / p.snake, j = rank % p.snake;
+        if ((k & 1) && (k + 1) * p.snake <= int(gridDim.x)) rank = k * p.snake + (p.snake - 1 - j);
+    }
+    const int wg = wgs_per_head - 1 - rank / heads;
+    const int bh = rank % heads;
     const int kvh = bh % p.KVH;
     const int b = bh / p.KVH;
 
@@ -300,7 +309,10 @@ int launch_blocks(Kernel kernel, const PrefillParams& p, int waves, int col_bloc
     const int wg_pos = waves * col_blocks * (16 / R);
     const int wgs_per_head = (p.T + wg_pos - 1) / wg_pos;
     const dim3 grid(unsigned(p.B) * unsigned(p.KVH) * unsigned(wgs_per_head));
-    hipLaunchKernelGGL(kernel, grid, dim3(waves * kWaveSize), 0, stream, p);
+    PrefillParams q = p;
+    const int cus = current_device_cus();
+    q.snake = (int64_t(grid.x) <= 4 * int64_t(cus)) ? cus : 0;
+    hipLaunchKernelGGL(kernel, grid, dim3(waves * kWaveSize), 0, stream, q);
     return int(hipGetLastError());
 }
 

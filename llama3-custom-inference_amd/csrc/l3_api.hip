@@ -548,6 +548,7 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     p.v_sb = v_strides[0]; p.v_sh = v_strides[1]; p.v_st = v_strides[2];
     p.o_sb = out_strides[0]; p.o_sh = out_strides[1]; p.o_st = out_strides[2];
     p.scale_log2e = scale * 1.4426950408889634f;
+    p.snake = 0;
     // Which form (graph-timed sweeps over B 1 ... 256, T 16 ... 8192, head ratios 1, 3, 4 and 8): a prompt
     // that does not exceed one workgroup of the tiled form per kv head, with few enough wavefronts for the
     // device to hold them all at once, runs as independent wavefronts with no barrier (4.2 against 4.8 us

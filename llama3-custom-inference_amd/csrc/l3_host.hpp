@@ -84,6 +84,7 @@ struct PrefillParams {
     int64_t v_sb, v_sh, v_st;
     int64_t o_sb, o_sh, o_st;
     float scale_log2e;
+    int snake;   // tiled form: ranks per round of the reversed-every-second-round order, 0 = plain (set by the launcher)
 };
 
 struct LinearParams {
