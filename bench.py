@@ -50,7 +50,7 @@ MIN_TIMED_S = 0.05
 # this file (the summaries, their commands and the copy-kernel calibration are under profiles/).
 # An entry is reported only while the split plan it was measured with is the plan of this run.
 MEASURED_TRAFFIC = {
-    "c2": {"bytes": 39390000, "plan": [8, 16, 32, 32, 32, 171, 205], "flags": 0,
+    "c2": {"bytes": 39150000, "plan": [8, 16, 32, 32, 32, 32, 32], "flags": 2,
            "profile": "profiles/attn_splitkv_mfma_c2_sweep_hbm_traffic.md"},
     "c3a": {"flags": 2, "bytes": 136660000, "plan": [1], "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},
     "c3b": {"flags": 2, "bytes": 135870000, "plan": [11], "profile": "profiles/hbm_traffic_batched_attention_rms_norm_rot_embed.md"},

@@ -18,11 +18,11 @@ def test_measured_traffic_belongs_to_the_plan_the_library_makes():
     plans must be what the library plans for a 256-unit device, or the key silently becomes null."""
     lib = _l3lib.load()
     B, HD, lengths, _ = bench.ATTN_WORKLOADS["c2"]
-    plan = [lib.l3_attn_choose_splits(B, 8, S, HD, 256, 0) for S in lengths]
-    assert plan == bench.MEASURED_TRAFFIC["c2"]["plan"]
-    for name in ("c3a", "c3b"):
+    for name in ("c2", "c3a", "c3b"):
+        rec = bench.MEASURED_TRAFFIC[name]
+        assert rec["flags"] == _l3lib.L3_ATTN_FLAG_WS_COUNTERS, "profiled with other flags than the default run uses"
         B, HD, lengths, _ = bench.ATTN_WORKLOADS[name]
-        assert [lib.l3_attn_choose_splits(B, 8, S, HD, 256, 0) for S in lengths] == bench.MEASURED_TRAFFIC[name]["plan"]
+        assert [lib.l3_attn_choose_splits(B, 8, S, HD, 256, rec["flags"]) for S in lengths] == rec["plan"]
 
 
 def test_measured_traffic_quotes_its_profile():
