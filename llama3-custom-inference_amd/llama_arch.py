@@ -472,15 +472,20 @@ class GraphedDecodeLoop:
             gc.collect()
             gc_was_enabled = gc.isenabled()
             gc.disable()
+            ok = True
             try:
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph):
                     out = m.forward(self.tokens[:, :T], start_pos=0)
+            except RuntimeError:
+                # an operator of the prompt pass refused to be recorded (the context manager has ended the
+                # capture): this length stays eager
+                ok = False
+                torch.cuda.synchronize(dev)
             finally:
                 if gc_was_enabled:
                     gc.enable()
-            ok = True
-            for _ in range(2):
+            for _ in range(2 if ok else 0):
                 graph.replay()
                 torch.cuda.synchronize(dev)
                 ok = ok and bool(torch.equal(out, ref))
