@@ -55,6 +55,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     constexpr int LOADS = TK * CPR / kWaveSize;  // wavefront-wide loads per operand tile
     static_assert(LOADS % NW == 0, "a tile must divide evenly over the wavefronts");
     constexpr int IPW = LOADS / NW;
+    constexpr bool PF = WPE <= 2;                // operand reads requested a phase ahead (needs the registers)
     __shared__ __align__(1024) unsigned char s_stage0[STAGE];
     __shared__ __align__(1024) unsigned char s_stage1[STAGE];
 
@@ -186,18 +187,63 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     // One tile on its LDS stage: S = K Q^T, the online softmax of S, O^T += V^T P.
     auto tile = [&](const unsigned char* stage, int t0) __attribute__((always_inline)) {
         f32x4_t S[CB][NG];
+        s16x8_t vt[PF ? KS : 1][NB];
+        auto v_operands = [&](int ks, s16x8_t (&vv)[NB]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int tg = 0; tg < NG; ++tg) {
+            for (int nb = 0; nb < NB; ++nb) {
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
+                vv[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        };
+        auto pin_operands = [&](s16x8_t (&vv)[NB]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) asm volatile("" : "+v"(vv[nb]));
+        };
+        if constexpr (PF) {
+            // With registers to spare (two wavefronts per SIMD): all K operands of the tile are requested
+            // before the first product, and the V^T operands of the tile's first 32 tokens before the
+            // softmax, so that one LDS latency per tile is exposed and not one per operand (the scheduler,
+            // left alone, sinks every read next to the product that uses it and waits there).
+            uint4 ka[NG][KC];
 #pragma unroll
             for (int m = 0; m < KC; ++m) {
-                const uint4 a = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[cb][tg];
-                    S[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[cb][m],
-                                                                        acc, 0, 0, 0);
+                for (int tg = 0; tg < NG; ++tg) ka[tg][m] = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int m = 0; m < KC; ++m) {
+#pragma unroll
+                for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) {
+                        const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[cb][tg];
+                        S[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka[tg][m]),
+                                                                            qfrag[cb][m], acc, 0, 0, 0);
+                    }
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
+            v_operands(0, vt[0]);
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+#pragma unroll
+            for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                for (int m = 0; m < KC; ++m) {
+                    const uint4 a = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) {
+                        const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[cb][tg];
+                        S[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[cb][m],
+                                                                            acc, 0, 0, 0);
+                    }
+                }
+            }
+
         }
 
         // causal mask (only tiles that reach past the wavefront's first position) and softmax
@@ -250,19 +296,39 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
 
         // O^T += V^T P; the k slots of a 32-token step pair (fg, i) with token 4*fg + i of the step's first
         // 16-token group for i < 4 and of its second group for i >= 4
+        if constexpr (PF) {
+            // the operands of step ks + 1 are requested before the products of step ks
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
+            for (int ks = 0; ks < KS; ++ks) {
+                // (the empty asm makes the wait for step ks precede the requests of step ks + 1)
+                __builtin_amdgcn_sched_barrier(0);
+                pin_operands(vt[ks]);
+                if (ks + 1 < KS) v_operands(ks + 1, vt[ks + 1]);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
-                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
-                const s16x8_t vv = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pfrag[cb][ks],
-                                                                        O[cb][nb], 0, 0, 0);
+                    for (int cb = 0; cb < CB; ++cb) {
+                        O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vt[ks][nb]),
+                                                                            pfrag[cb][ks], O[cb][nb], 0, 0, 0);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
+                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
+                    const s16x8_t vv = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) {
+                        O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pfrag[cb][ks],
+                                                                            O[cb][nb], 0, 0, 0);
+                    }
                 }
             }
         }
