@@ -55,7 +55,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     constexpr int LOADS = TK * CPR / kWaveSize;  // wavefront-wide loads per operand tile
     static_assert(LOADS % NW == 0, "a tile must divide evenly over the wavefronts");
     constexpr int IPW = LOADS / NW;
-    constexpr bool PF = WPE <= 2;                // operand reads requested a phase ahead (needs the registers)
+    constexpr bool PF = WPE <= 2;                // the interleaved tile below (needs the registers of two wavefronts per SIMD)
     __shared__ __align__(1024) unsigned char s_stage0[STAGE];
     __shared__ __align__(1024) unsigned char s_stage1[STAGE];
 
@@ -187,63 +187,18 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     // One tile on its LDS stage: S = K Q^T, the online softmax of S, O^T += V^T P.
     auto tile = [&](const unsigned char* stage, int t0) __attribute__((always_inline)) {
         f32x4_t S[CB][NG];
-        s16x8_t vt[PF ? KS : 1][NB];
-        auto v_operands = [&](int ks, s16x8_t (&vv)[NB]) __attribute__((always_inline)) {
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
-                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
-                vv[nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-        };
-        auto pin_operands = [&](s16x8_t (&vv)[NB]) __attribute__((always_inline)) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) asm volatile("" : "+v"(vv[nb]));
-        };
-        if constexpr (PF) {
-            // With registers to spare (two wavefronts per SIMD): all K operands of the tile are requested
-            // before the first product, and the V^T operands of the tile's first 32 tokens before the
-            // softmax, so that one LDS latency per tile is exposed and not one per operand (the scheduler,
-            // left alone, sinks every read next to the product that uses it and waits there).
-            uint4 ka[NG][KC];
+        for (int tg = 0; tg < NG; ++tg) {
 #pragma unroll
             for (int m = 0; m < KC; ++m) {
+                const uint4 a = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
 #pragma unroll
-                for (int tg = 0; tg < NG; ++tg) ka[tg][m] = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int m = 0; m < KC; ++m) {
-#pragma unroll
-                for (int tg = 0; tg < NG; ++tg) {
-#pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[cb][tg];
-                        S[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka[tg][m]),
-                                                                            qfrag[cb][m], acc, 0, 0, 0);
-                    }
+                for (int cb = 0; cb < CB; ++cb) {
+                    const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[cb][tg];
+                    S[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[cb][m],
+                                                                        acc, 0, 0, 0);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
-            v_operands(0, vt[0]);
-            __builtin_amdgcn_sched_barrier(0);
-        } else {
-#pragma unroll
-            for (int tg = 0; tg < NG; ++tg) {
-#pragma unroll
-                for (int m = 0; m < KC; ++m) {
-                    const uint4 a = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
-#pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[cb][tg];
-                        S[cb][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[cb][m],
-                                                                            acc, 0, 0, 0);
-                    }
-                }
-            }
-
         }
 
         // causal mask (only tiles that reach past the wavefront's first position) and softmax
@@ -296,41 +251,144 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
 
         // O^T += V^T P; the k slots of a 32-token step pair (fg, i) with token 4*fg + i of the step's first
         // 16-token group for i < 4 and of its second group for i >= 4
-        if constexpr (PF) {
-            // the operands of step ks + 1 are requested before the products of step ks
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                // (the empty asm makes the wait for step ks precede the requests of step ks + 1)
-                __builtin_amdgcn_sched_barrier(0);
-                pin_operands(vt[ks]);
-                if (ks + 1 < KS) v_operands(ks + 1, vt[ks + 1]);
-                __builtin_amdgcn_sched_barrier(0);
+        for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
+            for (int nb = 0; nb < NB; ++nb) {
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
+                const s16x8_t vv = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vt[ks][nb]),
-                                                                            pfrag[cb][ks], O[cb][nb], 0, 0, 0);
+                for (int cb = 0; cb < CB; ++cb) {
+                    O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pfrag[cb][ks],
+                                                                        O[cb][nb], 0, 0, 0);
+                }
+            }
+        }
+    };
+    // The same tile for wavefronts with registers to spare (two per SIMD, head size 128), laid out so that the
+    // vector work of one column block issues between the matrix instructions of the other:
+    //   K operands (all of the tile, one wait)    S0 = K Q0^T
+    //   [S1 = K Q1^T          | exponentials of S0]      V^T operands of the first 32 tokens requested half way
+    //   [O0^T += V^T P0       | exponentials of S1]      V^T operands of the last 32 tokens requested first
+    //    O1^T += V^T P1
+    // A matrix instruction occupies its pipe for 16 cycles and the wavefront may issue independent vector
+    // instructions meanwhile; left to itself the compiler keeps the phases apart and puts every LDS read next
+    // to the product that needs it, with a full wait.  sched_barrier(0) pins the order written here.
+    auto tile_pf = [&](const unsigned char* stage, int t0, auto mask_tag) __attribute__((always_inline)) {
+        constexpr bool MASK = decltype(mask_tag)::value;
+        static_assert(CB == 2, "two column blocks take turns");
+        constexpr int NQ = KC * NG;   // matrix instructions of a column block's scores
+        constexpr int NP = KS * NB;   // ... and of its output
+        constexpr int NS = NG * 4;    // scores per lane and column block
+        static_assert(NS % NQ == 0 && NS % NP == 0, "whole scores per matrix instruction");
+        f32x4_t S[CB][NG];
+        uint4 ka[NG][KC];
+#pragma unroll
+        for (int m = 0; m < KC; ++m) {
+#pragma unroll
+            for (int tg = 0; tg < NG; ++tg) ka[tg][m] = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < KC; ++m) {
+#pragma unroll
+            for (int tg = 0; tg < NG; ++tg) {
+                const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[0][tg];
+                S[0][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka[tg][m]), qfrag[0][m], acc, 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // mask, running maximum and (rarely) the rescaling of one column block; returns the exponent offset
+        auto head = [&](int cb) __attribute__((always_inline)) -> float {
+            if constexpr (MASK) {
+                const int visible = col_limit[cb] - t0 - 4 * fg;
+#pragma unroll
+                for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (tg * 16 + j >= visible) S[cb][tg][j] = kMaskedScore;
                     }
                 }
             }
-        } else {
+            float mloc = S[cb][0][0];
+#pragma unroll
+            for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) mloc = maximum(mloc, S[cb][tg][j]);
+            }
+            mloc = column_maximum(mloc);
+            if (__builtin_amdgcn_ballot_w64(mloc > m_run[cb] + slack) != 0) {
+                const float m_new = maximum(m_run[cb], mloc);
+                const float alpha = fast_exp2((m_run[cb] - m_new) * c);
+                L[cb] *= alpha;
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) O[cb][nb] *= alpha;
+                m_run[cb] = m_new;
+            }
+            return m_run[cb] * c;
+        };
+        uint32_t pw[CB][NS / 2];
+        auto score = [&](int cb, int i, float mc) __attribute__((always_inline)) {
+            const int tg = i / 4, j = i % 4;
+            S[cb][tg][j] = fast_exp2(fmaf(S[cb][tg][j], c, -mc));   // masked scores give exactly 0
+            if (j & 1) pw[cb][i / 2] = pack_bf16x2(S[cb][tg][j - 1], S[cb][tg][j]);
+        };
+        bf16x8_t pfrag[CB][KS];
+        auto weights = [&](int cb) __attribute__((always_inline)) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
-                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
-                    const s16x8_t vv = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pfrag[cb][ks],
-                                                                            O[cb][nb], 0, 0, 0);
-                    }
-                }
+                pfrag[cb][ks] = __builtin_bit_cast(bf16x8_t, make_uint4(pw[cb][4 * ks], pw[cb][4 * ks + 1], pw[cb][4 * ks + 2], pw[cb][4 * ks + 3]));
+                L[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pfrag[cb][ks], L[cb], 0, 0, 0);
             }
+        };
+        s16x8_t vt[KS][NB];
+        auto v_operands = [&](int ks) __attribute__((always_inline)) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
+                vt[ks][nb] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        };
+
+        const float mc0 = head(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int m = q / NG, tg = q % NG;
+            const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : S[1][tg];
+            S[1][tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka[tg][m]), qfrag[1][m], acc, 0, 0, 0);
+#pragma unroll
+            for (int i = q * (NS / NQ); i < (q + 1) * (NS / NQ); ++i) score(0, i, mc0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (q == NQ / 2 - 1) {   // half of the K operands are spent: their registers take the first V^T operands
+                v_operands(0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        weights(0);
+        const float mc1 = head(1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) asm volatile("" : "+v"(vt[0][nb]));   // the wait for these precedes the next requests
+        v_operands(1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int ks = q / NB, nb = q % NB;
+            O[0][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vt[ks][nb]), pfrag[0][ks], O[0][nb], 0, 0, 0);
+#pragma unroll
+            for (int i = q * (NS / NP); i < (q + 1) * (NS / NP); ++i) score(1, i, mc1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        weights(1);
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int ks = q / NB, nb = q % NB;
+            O[1][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vt[ks][nb]), pfrag[1][ks], O[1][nb], 0, 0, 0);
         }
     };
     // One barrier per tile: the loads of tile i + 1 are issued before the arithmetic on tile i and land in
@@ -338,7 +396,16 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     auto step = [&](auto parity_tag, int t0) __attribute__((always_inline)) {
         constexpr int PAR = decltype(parity_tag)::value;
         if (t0 + TK < wg_t_end) dma(t0 + TK, PAR ? s_stage0 : s_stage1);   // workgroup-uniform
-        if (t0 < wave_t_end) tile(PAR ? s_stage1 : s_stage0, t0);          // wave-uniform
+        if (t0 < wave_t_end) {                                              // wave-uniform
+            const unsigned char* stage = PAR ? s_stage1 : s_stage0;
+            if constexpr (PF) {
+                // only tiles that reach past the wavefront's first position need the causal mask
+                if (t0 + TK > wave_limit_min) tile_pf(stage, t0, std::true_type{});
+                else tile_pf(stage, t0, std::false_type{});
+            } else {
+                tile(stage, t0);
+            }
+        }
         __builtin_amdgcn_s_waitcnt(0xF70);   // vmcnt(0): this wavefront's part of the next stage has landed
         __syncthreads();
     };
