@@ -309,6 +309,35 @@ def measure_read_stream(torch, lib, dev, pool, chunk_bytes=128 << 20):
             "kernel": "hbm_read_stream_kernel (16-byte non-temporal loads, no stores, no arithmetic)"}
 
 
+def weights_read_floor_us(torch, lib, dev):
+    """What a decode step of the 1B architecture would take if it did nothing but read its weights: the
+    read-only kernel launched once per linear kernel of the step, on that kernel's weight bytes (qkv, output
+    projection, gate|up pair, down projection per layer, then the vocabulary projection), each region its own
+    part of a 2.5 GB buffer, so that a replay finds every byte as cold as the real step finds its weights."""
+    C, FF, V, LAYERS, KV = 2048, 8192, 128256, 16, 512
+    sizes = [((C + 2 * KV) * C * 2), C * C * 2, 2 * FF * C * 2, C * FF * 2] * LAYERS + [V * C * 2]
+    offsets, total = [], 0
+    for n in sizes:
+        offsets.append(total)
+        total += (n + 4095) // 4096 * 4096
+    buf = torch.empty(total, dtype=torch.uint8, device=dev)
+    buf.random_(0, 255)
+    sink = torch.zeros(16, dtype=torch.int32, device=dev)
+
+    def walk():
+        sp = torch.cuda.current_stream().cuda_stream
+        for off, n in zip(offsets, sizes):
+            rc = lib.l3_hbm_read_stream(buf.data_ptr() + off, n, sink.data_ptr(), 0, sp)
+            if rc != 0:
+                raise RuntimeError(f"l3_hbm_read_stream failed: {rc}")
+    walk()
+    gph = capture_graph(torch, walk)
+    ms, _ = timed_replays(torch, gph)
+    del gph, buf
+    torch.cuda.empty_cache()
+    return round(ms * 1e3, 1), len(sizes), sum(sizes)
+
+
 def measure_rw_stream(torch, lib, dev, nbytes):
     """The read + write yardstick: the library's copy-through kernel (16-byte non-temporal loads, plain 16-byte
     stores) over cold source / destination pairs of `nbytes` each, graph-replayed: what a row-wise operator
@@ -966,6 +995,10 @@ def main():
 
             line["e2e"] = llama_arch.e2e_summary(torch, dev, cpu_ops=None if args.no_cpu_baseline else cpu_op_table())
             line["e2e_tokens_per_s"] = {k: v["tok_per_s"] for k, v in line["e2e"].items() if k.startswith("bs")}
+            floor_us, launches, wbytes = weights_read_floor_us(torch, lib, dev)
+            line["e2e"]["weights_read_stream_floor"] = {
+                "us_per_step": floor_us, "launches": launches, "bytes": wbytes,
+                "what": "the read-only kernel once per linear kernel of a batch-1 decode step, on that kernel's weight bytes, cold"}
     line.update(head)
     line["roofline"] = roofline
     line["cpu_baseline"] = cpu
