@@ -111,38 +111,38 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     }
 
     // global -> LDS: load j of a wavefront covers slots inst*64 .. +63 of the tile, slot = row * CPR + position.
-    // An address is a scalar tile base plus a 32-bit lane offset that does not change from tile to tile
-    // (token strides are below 2^24 elements); rows past the data are clamped to the last row and masked.
+    // The loads are buffer loads: the resource describes the tile (a scalar base and the bytes from there to the
+    // end of the kv head's data), the lane offset never changes from tile to tile (token strides are below 2^24
+    // elements), so a load costs no vector instruction, and rows past the data come back as zeros (they are
+    // masked: no query sees a token beyond the KV length).
     const char* kb = reinterpret_cast<const char*>(p.k) + wave_uniform((b * p.k_sb + kvh * p.k_sh) * 2);
     const char* vb = reinterpret_cast<const char*>(p.v) + wave_uniform((b * p.v_sb + kvh * p.v_sh) * 2);
     const int64_t k_pitch = wave_uniform(int(p.k_st)) * int64_t(2);   // bytes from a token to the next
     const int64_t v_pitch = wave_uniform(int(p.v_st)) * int64_t(2);
     const int wave_u = wave_uniform(wave);
     auto swz_key = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
-    uint32_t krow[IPW], vrow[IPW], chunk16[IPW];
+    uint32_t koff[IPW], voff[IPW];
 #pragma unroll
     for (int j = 0; j < IPW; ++j) {
         const int slot = (wave_u * IPW + j) * kWaveSize + lane;
         const int row = slot / CPR;
-        krow[j] = uint32_t(row) * uint32_t(k_pitch);
-        vrow[j] = uint32_t(row) * uint32_t(v_pitch);
-        chunk16[j] = uint32_t((slot % CPR) ^ swz_key(row)) * 16u;
+        const uint32_t chunk16 = uint32_t((slot % CPR) ^ swz_key(row)) * 16u;
+        koff[j] = uint32_t(row) * uint32_t(k_pitch) + chunk16;
+        voff[j] = uint32_t(row) * uint32_t(v_pitch) + chunk16;
     }
     auto dma = [&](int t0, unsigned char* stage) {
-        const int last_row = min(p.S - 1 - t0, TK - 1);                  // scalar
-        const char* kt = kb + int64_t(t0) * k_pitch;
-        const char* vt = vb + int64_t(t0) * v_pitch;
-        const uint32_t k_last = uint32_t(last_row) * uint32_t(k_pitch);
-        const uint32_t v_last = uint32_t(last_row) * uint32_t(v_pitch);
+        const int64_t rows_left = p.S - t0;                              // scalar, at least 1
+        const int64_t k_bytes = min((rows_left - 1) * k_pitch + ROWB, int64_t(0xffffffffLL));
+        const int64_t v_bytes = min((rows_left - 1) * v_pitch + ROWB, int64_t(0xffffffffLL));
+        const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char*>(kb + int64_t(t0) * k_pitch), 0, int(uint32_t(k_bytes)), 0x00020000);
+        const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char*>(vb + int64_t(t0) * v_pitch), 0, int(uint32_t(v_bytes)), 0x00020000);
 #pragma unroll
         for (int j = 0; j < IPW; ++j) {
             const int inst = wave_u * IPW + j;
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(kt + (min(krow[j], k_last) + chunk16[j])),
-                L3_LDS_PTR(void, stage + inst * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(vt + (min(vrow[j], v_last) + chunk16[j])),
-                L3_LDS_PTR(void, stage + KBYTES + inst * 1024), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, L3_LDS_PTR(void, stage + inst * 1024), 16, int(koff[j]), 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, L3_LDS_PTR(void, stage + KBYTES + inst * 1024), 16, int(voff[j]), 0, 0, 0);
         }
     };
     // operand addresses within a stage.  K: lane (fn, fg) reads chunk 4m + fg of row 16 tg + fn, whose
@@ -182,7 +182,8 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     // below 256, which bf16 and the float32 sums hold as well as values below 1 -- and the accumulators
     // need no rescaling.  O / L is the same quotient either way.
     const float slack = 8.0f / c;
-    const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+    bf16x8_t ones = __builtin_bit_cast(bf16x8_t, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+    asm volatile("" : "+v"(ones));   // kept in registers: rebuilt from constants it costs two moves per use
 
     // One tile on its LDS stage: S = K Q^T, the online softmax of S, O^T += V^T P.
     auto tile = [&](const unsigned char* stage, int t0) __attribute__((always_inline)) {
