@@ -168,10 +168,12 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     // spared one addition per score; P enters both sums rounded to bf16, so the weights of a column add
     // up to one exactly.
     f32x4_t O[CB][NB], L[CB];
+    float Lsum[CB];    // the hand-laid tile keeps the denominator as one number per column (it looks at a tile's sum first)
     float m_run[CB];
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
         m_run[cb] = kMaskedScore;
+        Lsum[cb] = 0.f;
         L[cb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) O[cb][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -269,6 +271,69 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
             }
         }
     };
+    // Pieces of the hand-laid tile below.  It computes no maximum as long as the reference maximum is good enough:
+    // the exponentials are taken against the reference as it stands, and the column sum of the tile's weights,
+    // which the matrix pipe forms anyway (against a block of ones), tells whether that was safe -- a sum of at
+    // most kTileSumLimit means every weight stayed below it, which bf16 and the float32 sums hold as well as values
+    // below 1, and O / L is the same quotient for any reference.  Only when a column's sum exceeds the limit or is
+    // not a number (the first tile, whose reference is still the masked score; a score that leaves the reference
+    // far behind) the scores of that column block are formed once more, their maximum becomes the reference, the
+    // accumulators are rescaled and the weights redone.
+    constexpr float kTileSumLimit = 1024.0f;
+    auto mask_scores = [&](f32x4_t (&Z)[NG], int visible) __attribute__((always_inline)) {
+#pragma unroll
+        for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (tg * 16 + j >= visible) Z[tg][j] = kMaskedScore;   // this lane's scores 16 tg + j beyond `visible` do not count
+            }
+        }
+    };
+    auto redo_column_block = [&](const unsigned char* stage, int cb, f32x4_t (&Z)[NG], int visible, bool masked,
+                                 bf16x8_t (&pf)[KS]) __attribute__((always_inline)) -> float {
+#pragma unroll
+        for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+            for (int m = 0; m < KC; ++m) {
+                const uint4 a = *reinterpret_cast<const uint4*>(stage + ak[m] + tg * 16 * ROWB);
+                const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : Z[tg];
+                Z[tg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[cb][m], acc, 0, 0, 0);
+            }
+        }
+        if (masked) mask_scores(Z, visible);
+        float mloc = Z[0][0];
+#pragma unroll
+        for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) mloc = maximum(mloc, Z[tg][j]);
+        }
+        mloc = column_maximum(mloc);
+        const float m_new = maximum(m_run[cb], mloc);
+        const float alpha = fast_exp2((m_run[cb] - m_new) * c);
+        Lsum[cb] *= alpha;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) O[cb][nb] *= alpha;
+        m_run[cb] = m_new;
+        const float mc = m_new * c;
+#pragma unroll
+        for (int tg = 0; tg < NG; ++tg) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) Z[tg][j] = fast_exp2(fmaf(Z[tg][j], c, -mc));
+        }
+        f32x4_t sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            uint4 pw;
+            pw.x = pack_bf16x2(Z[2 * ks][0], Z[2 * ks][1]);
+            pw.y = pack_bf16x2(Z[2 * ks][2], Z[2 * ks][3]);
+            pw.z = pack_bf16x2(Z[2 * ks + 1][0], Z[2 * ks + 1][1]);
+            pw.w = pack_bf16x2(Z[2 * ks + 1][2], Z[2 * ks + 1][3]);
+            pf[ks] = __builtin_bit_cast(bf16x8_t, pw);
+            sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pf[ks], sum, 0, 0, 0);
+        }
+        return sum[0];
+    };
+
     // The same tile for wavefronts with registers to spare (two per SIMD, head size 128), laid out so that the
     // vector work of one column block issues between the matrix instructions of the other:
     //   K operands (all of the tile, one wait)    S0 = K Q0^T
@@ -302,35 +367,6 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        // mask, running maximum and (rarely) the rescaling of one column block; returns the exponent offset
-        auto head = [&](int cb) __attribute__((always_inline)) -> float {
-            if constexpr (MASK) {
-                const int visible = col_limit[cb] - t0 - 4 * fg;
-#pragma unroll
-                for (int tg = 0; tg < NG; ++tg) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (tg * 16 + j >= visible) S[cb][tg][j] = kMaskedScore;
-                    }
-                }
-            }
-            float mloc = S[cb][0][0];
-#pragma unroll
-            for (int tg = 0; tg < NG; ++tg) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) mloc = maximum(mloc, S[cb][tg][j]);
-            }
-            mloc = column_maximum(mloc);
-            if (__builtin_amdgcn_ballot_w64(mloc > m_run[cb] + slack) != 0) {
-                const float m_new = maximum(m_run[cb], mloc);
-                const float alpha = fast_exp2((m_run[cb] - m_new) * c);
-                L[cb] *= alpha;
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) O[cb][nb] *= alpha;
-                m_run[cb] = m_new;
-            }
-            return m_run[cb] * c;
-        };
         uint32_t pw[CB][NS / 2];
         auto score = [&](int cb, int i, float mc) __attribute__((always_inline)) {
             const int tg = i / 4, j = i % 4;
@@ -339,11 +375,17 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         };
         bf16x8_t pfrag[CB][KS];
         auto weights = [&](int cb) __attribute__((always_inline)) {
+            f32x4_t sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 pfrag[cb][ks] = __builtin_bit_cast(bf16x8_t, make_uint4(pw[cb][4 * ks], pw[cb][4 * ks + 1], pw[cb][4 * ks + 2], pw[cb][4 * ks + 3]));
-                L[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pfrag[cb][ks], L[cb], 0, 0, 0);
+                sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pfrag[cb][ks], sum, 0, 0, 0);
             }
+            float tile_sum = sum[0];   // every entry of the block is its column's sum
+            if (__builtin_amdgcn_ballot_w64(!(tile_sum <= kTileSumLimit)) != 0) {
+                tile_sum = redo_column_block(stage, cb, S[cb], col_limit[cb] - t0 - 4 * fg, MASK, pfrag[cb]);
+            }
+            Lsum[cb] += tile_sum;
         };
         s16x8_t vt[KS][NB];
         auto v_operands = [&](int ks) __attribute__((always_inline)) {
@@ -355,7 +397,8 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
             }
         };
 
-        const float mc0 = head(0);
+        if constexpr (MASK) mask_scores(S[0], col_limit[0] - t0 - 4 * fg);
+        const float mc0 = m_run[0] * c;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
@@ -370,8 +413,9 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        if constexpr (MASK) mask_scores(S[1], col_limit[1] - t0 - 4 * fg);
+        const float mc1 = m_run[1] * c;
         weights(0);
-        const float mc1 = head(1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) asm volatile("" : "+v"(vt[0][nb]));   // the wait for these precedes the next requests
@@ -424,7 +468,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         if (col_limit[cb] > 0) {
             const int qi = wave_first_qi + cb * ppw + fn / R;
             const int qh = kvh * R + fn % R;
-            const float inv = 1.0f / L[cb][0];
+            const float inv = 1.0f / (PF ? Lsum[cb] : L[cb][0]);
             uint16_t* orow = p.out + b * p.o_sb + int64_t(qh) * p.o_sh + int64_t(qi) * p.o_st + fg * 4;
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
