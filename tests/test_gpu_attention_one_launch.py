@@ -190,3 +190,58 @@ def test_one_launch_under_graph_replay(l3, call, gpu):
         assert call.counters_are_zero()
         call(qg, kg, vg, 5, l3.L3_ATTN_FLAG_FORM_COOP)   # eager work on the same workspace between replays
     assert call.placement_errors() == 0
+
+
+def test_calls_on_two_streams_at_once(l3, gpu):
+    """Two callers with their own workspaces on two streams, long enough kernels (256 workgroups each, 15 and
+    25 us) and deep enough queues that their launches overlap on the device, and matrix products on a third
+    stream: the placement of a grid's workgroups on the XCDs must not depend on what else is being dispatched.
+    Every call must reproduce the bits of the same call made alone, leave its counters at zero and report no
+    head whose arrivals came from several XCDs."""
+    lib = l3.load()
+    W = l3.L3_ATTN_FLAG_WS_COUNTERS
+
+    class StreamCaller:
+        def __init__(self, S, seed):
+            B, QH, KVH, HD = 1, 32, 8, 128
+            self.stream = torch.cuda.Stream()
+            self.q, self.k, self.v = make_qkv(B, QH, KVH, S, HD, seed=seed, device=gpu)
+            self.ws = torch.empty(32 << 20, dtype=torch.uint8, device=gpu)
+            assert lib.l3_attn_workspace_init(self.ws.data_ptr(), self.ws.numel(), self.stream.cuda_stream) == 0
+            torch.cuda.synchronize()
+            self.out = torch.empty_like(self.q)
+            self.bad = torch.zeros(1, dtype=torch.int64, device=gpu)
+            q, k, v, out = self.q, self.k, self.v, self.out
+            self.args = [q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), B, QH, KVH,
+                         S, HD, l3.i64_array((q.stride(0), q.stride(1))), l3.i64_array((k.stride(0), k.stride(1), k.stride(2))),
+                         l3.i64_array((v.stride(0), v.stride(1), v.stride(2))), l3.i64_array((out.stride(0), out.stride(1))),
+                         1.0 / math.sqrt(HD), 0, W]
+            assert lib.l3_attn_launches(B, QH, KVH, S, HD, 0, W) == 1
+            self.call()
+            torch.cuda.synchronize()
+            self.alone = self.out.clone()
+
+        def call(self):
+            assert lib.l3_attn_decode(*self.args, self.stream.cuda_stream) == 0
+
+        def check(self):
+            with torch.cuda.stream(self.stream):
+                self.bad += (self.out.view(torch.int16) != self.alone.view(torch.int16)).sum()
+                self.out.zero_()
+
+    a, b = StreamCaller(32768, 31), StreamCaller(16384, 32)
+    side = torch.cuda.Stream()
+    x = torch.randn(2048, 2048, device=gpu, dtype=torch.bfloat16)
+    for it in range(150):
+        for c in (a, b):
+            for _ in range(4):
+                c.call()
+            c.check()
+        if it % 3 == 0:
+            with torch.cuda.stream(side):
+                _ = x @ x
+    torch.cuda.synchronize()
+    for c in (a, b):
+        assert int(c.bad.item()) == 0
+        assert int(c.ws[: l3.L3_ATTN_COUNTER_BYTES - 128].view(torch.int32).count_nonzero().item()) == 0
+        assert lib.l3_attn_placement_errors(c.ws.data_ptr()) == 0
