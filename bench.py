@@ -520,6 +520,9 @@ def run_attention(args, torch, lib, l3, dev, name, pool):
                      "launches_timed": (ev_reps * steps if all(single_launch) else sreps * passes) * len(lengths),
                      "algorithmic_bytes_per_launch": pass_bytes // len(lengths),
                      "split_stage_only_avg_us": round(split_ms * 1e3 / len(lengths), 3),
+                     # the same quotient for the split stage alone (partials written, nothing merged): what this key
+                     # measured while the merge was a launch of its own
+                     "split_stage_only_frac": round(pass_bytes / (split_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                      "whole_call_GBps": round(op_gbps, 1),
                      "whole_call_frac": round(op_gbps / HBM_PEAK_GBPS, 4)},
         "cpu_baseline": cpu, "per_length": detail,
