@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import assert_attn_close, make_qkv, randn_bf16, t2bits, t2f32
+from helpers import ATTN_REG_ATOL, ATTN_REG_FEW_TOKENS, ATTN_REG_RTOL, assert_attn_close, make_qkv, randn_bf16, t2bits, t2f32
 from oracle import attention_decode_ref
 
 pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("attn_kernel")]
@@ -479,6 +479,38 @@ def test_prefill_forms_agree_on_a_long_prompt(gpu):
                                    t2f32(v[:, :i + 1].transpose(1, 2)))
         assert_attn_close(outs["tiled"][:, :, i:i + 1], ref, what=f"long prefill row {i} (tiled)")
         assert_attn_close(outs["wave"][:, :, i:i + 1], ref, what=f"long prefill row {i} (wave)")
+
+
+@pytest.mark.parametrize("B,T,HD,gain", [(2, 2048, 64, 1.0), (1, 8192, 128, 1.0), (1, 8192, 64, 1.0),
+                                         (1, 8192, 128, 3.0), (1, 8192, 64, 3.0)])
+def test_prefill_timed_shapes_by_sampled_rows(gpu, B, T, HD, gain):
+    """The prompt shapes the benchmark times, at their own size: rows either side of every kind of tile
+    edge and the last rows against the float64 oracle, with unit-variance queries and with queries scaled
+    so that a row's maximum keeps moving by more than the kernel's rescaling slack over 128 tiles.  With
+    the scaled queries a few keys carry a row, and the head-size-128 kernel, which exponentiates against the
+    previous tile's reference, rounds the dominant weight to bf16 (2^-9 relative) where a maximum-first
+    kernel holds it as exactly 1: those rows are held to twice the regression bound's absolute part."""
+    from custom_kernels import custom_kernels_extension as cke
+    from oracle import attention_decode_ref
+
+    QH, KVH = 32, 8
+    print(f"prefill timed shape B={B} T={T} HD={HD} gain={gain}", flush=True)
+    q = (randn_bf16((B, T, QH, HD), 84).float() * gain).to(torch.bfloat16)
+    k = randn_bf16((B, T, KVH, HD), 85)
+    v = randn_bf16((B, T, KVH, HD), 86)
+    out = cke.flash_attention_prefill(q.to(gpu).transpose(1, 2), k.to(gpu).transpose(1, 2),
+                                      v.to(gpu).transpose(1, 2)).float().cpu()
+    rows = sorted({0, 15, 16, 63, 64, 65, 127, 128, 129, 255, 256, T // 2 - 1, T // 2, T // 2 + 1, T - 130,
+                   T - 65, T - 64, T - 2, T - 1})
+    for i in rows:
+        ref = attention_decode_ref(t2f32(q[:, i:i + 1].transpose(1, 2)), t2f32(k[:, :i + 1].transpose(1, 2)),
+                                   t2f32(v[:, :i + 1].transpose(1, 2)))
+        what = f"prefill B={B} T={T} HD={HD} gain={gain} row {i}"
+        assert_attn_close(out[:, :, i:i + 1], ref, what=what, min_kv_len=i + 1, regression=gain == 1.0)
+        if gain != 1.0:
+            err = np.abs(out[:, :, i:i + 1].numpy().astype(np.float64) - ref)
+            bound = 2 * ATTN_REG_ATOL + (0.0 if i >= 63 else ATTN_REG_FEW_TOKENS) + ATTN_REG_RTOL * np.abs(ref)
+            assert not (err > bound).any(), f"{what}: max err {err.max():.4g}, {(err > bound).sum()} outside the bound"
 
 
 def test_prefill_last_row_equals_decode(gpu):
