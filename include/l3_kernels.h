@@ -61,8 +61,11 @@ const char* l3_strerror(int code);
  *                            the same thing; the flag exists so that the comparison can be repeated
  *                            (the reference has one kernel and no counterpart of this choice).
  *   L3_ATTN_FLAG_PREFILL_*   prefill: force one form of l3_attn_prefill instead of the choice by
- *                            prompt length -- WAVE (every wavefront streams K/V on its own) or
- *                            TILED (a workgroup shares K/V tiles).
+ *                            prompt length -- WAVE (every wavefront streams K/V on its own), TILED (a
+ *                            workgroup shares K/V tiles) or TILED_NO_MAX (TILED, and at head size 64 the
+ *                            tiles that take no maximum whatever the size of the launch; left to itself
+ *                            the library uses them for launches of more workgroups than the device holds
+ *                            at once).  Same results within the stated tolerance; for tests and timing.
  *   L3_ATTN_FLAG_WS_COUNTERS decode: the workspace starts with L3_ATTN_COUNTER_BYTES of arrival counters
  *                            that l3_attn_workspace_init prepared (see there); the library may then merge
  *                            the split partials inside the split launch instead of launching a combine.
@@ -72,7 +75,7 @@ const char* l3_strerror(int code);
  *                            (COOP: a workgroup per (batch, kv head, split)) or streamed (STREAM, the default
  *                            for an explicit count: a wavefront per (batch, kv head, split)).  The automatic
  *                            plan chooses the form itself.
- * Any other bit, or both bits of a two-bit field at once, gives L3_ERR_FLAGS.
+ * Any other bit, or both bits of the FORM field at once, gives L3_ERR_FLAGS.
  */
 #define L3_ATTN_FLAG_KERNEL_FMA 0x1
 #define L3_ATTN_FLAG_WS_COUNTERS 0x2
@@ -82,6 +85,7 @@ const char* l3_strerror(int code);
 #define L3_ATTN_FLAG_TWO_LAUNCHES 0x40
 #define L3_ATTN_FLAG_PREFILL_WAVE 0x10
 #define L3_ATTN_FLAG_PREFILL_TILED 0x20
+#define L3_ATTN_FLAG_PREFILL_TILED_NO_MAX 0x30
 #define L3_ATTN_FLAG_PREFILL_MASK 0x30
 
 /*

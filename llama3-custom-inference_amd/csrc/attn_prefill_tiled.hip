@@ -44,7 +44,7 @@ __device__ __forceinline__ float column_maximum(float x) {
 // not padded; instead the 16-byte chunk c of token row r sits at chunk position c ^ key(r), which
 // spreads the rows that an operand read touches together over all banks.  The two stages are separate
 // arrays, so that the compiler can tell a read of one from the load in flight into the other.
-template <int HD, int CB, int NW, int TK, int WPE>
+template <int HD, int CB, int NW, int TK, int WPE, bool NOMAX>
 __global__ void __launch_bounds__(NW * kWaveSize) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 attn_prefill_tiled_kernel(const PrefillParams p) {
     constexpr int NG = TK / 16, KS = TK / 32, KC = HD / 32, NB = HD / 16;
@@ -334,6 +334,121 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         return sum[0];
     };
 
+    // The compiler-scheduled tile without a maximum (head size 64, launches of many workgroups): the weights are
+    // taken against the reference as it stands, 32 tokens at a time (their scores live in 16 registers), and
+    // their column sums, which the matrix pipe forms anyway, are checked before anything reaches the accumulators.
+    // A sum out of range or not a number stops the wavefront at that tile: nothing is repaired here, so that the
+    // loop carries no second path (with one, at 128 registers, the loop's invariants end up in scratch memory).
+    // The tiles from there on are done afterwards by the maximum-first tile above, which takes over m_run, O and
+    // the denominator as they stand.  The reference is the maximum of the first tile's scores, per column: a row
+    // leaves the range only when a later score exceeds everything among its first 64 by a factor of hundreds.
+    int first_careful_tile = NOMAX ? 0x7fffffff : 0;   // wave-uniform: the tile from which this wavefront takes the maximum first
+    auto scores32 = [&](const unsigned char* stage, int t0, int ks, f32x4_t (&Z)[CB][2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int m = 0; m < KC; ++m) {
+                const uint4 a = *reinterpret_cast<const uint4*>(stage + ak[m] + (2 * ks + h) * 16 * ROWB);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const f32x4_t acc = (m == 0) ? f32x4_t{0.f, 0.f, 0.f, 0.f} : Z[cb][h];
+                    Z[cb][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), qfrag[cb][m],
+                                                                       acc, 0, 0, 0);
+                }
+            }
+        }
+        if (t0 + TK > wave_limit_min) {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                const int visible = col_limit[cb] - t0 - 4 * fg;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if ((2 * ks + h) * 16 + j >= visible) Z[cb][h][j] = kMaskedScore;
+                    }
+                }
+            }
+        }
+    };
+    auto tile_lz = [&](const unsigned char* stage, int t0) __attribute__((always_inline)) {
+        bf16x8_t pfrag[CB][KS];
+        f32x4_t sum[CB];
+        float mc[CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            sum[cb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            mc[cb] = m_run[cb] * c;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            f32x4_t Z[CB][2];
+            scores32(stage, t0, ks, Z);
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) Z[cb][h][j] = fast_exp2(fmaf(Z[cb][h][j], c, -mc[cb]));
+                }
+                uint4 pw;
+                pw.x = pack_bf16x2(Z[cb][0][0], Z[cb][0][1]);
+                pw.y = pack_bf16x2(Z[cb][0][2], Z[cb][0][3]);
+                pw.z = pack_bf16x2(Z[cb][1][0], Z[cb][1][1]);
+                pw.w = pack_bf16x2(Z[cb][1][2], Z[cb][1][3]);
+                pfrag[cb][ks] = __builtin_bit_cast(bf16x8_t, pw);
+                sum[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pfrag[cb][ks], sum[cb], 0, 0, 0);
+            }
+        }
+        bool out_of_range = false;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) out_of_range = out_of_range || !(sum[cb][0] <= kTileSumLimit);
+        if (__builtin_amdgcn_ballot_w64(out_of_range) != 0) {   // nothing of this tile has reached the accumulators
+            first_careful_tile = t0;
+            return;
+        }
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) Lsum[cb] += sum[cb][0];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks) * 16 * ROWB));
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    L3_LDS_PTR(s16x4_t, stage + av[nb] + (2 * ks + 1) * 16 * ROWB));
+                const s16x8_t vv = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    O[cb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vv), pfrag[cb][ks],
+                                                                        O[cb][nb], 0, 0, 0);
+                }
+            }
+        }
+    };
+    auto reference_from_first_tile = [&](const unsigned char* stage) __attribute__((always_inline)) {
+        float mloc[CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) mloc[cb] = kMaskedScore;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            f32x4_t Z[CB][2];
+            scores32(stage, 0, ks, Z);
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) mloc[cb] = maximum(mloc[cb], Z[cb][h][j]);
+                }
+            }
+        }
+        // a column that belongs to no query (padding of the 16-column block, positions past the prompt) gets a
+        // reference that turns its weights to zero instead of one that every unmasked tile would overflow
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) m_run[cb] = col_limit[cb] > 0 ? column_maximum(mloc[cb]) : 1e30f;
+    };
+
     // The same tile for wavefronts with registers to spare (two per SIMD, head size 128), laid out so that the
     // vector work of one column block issues between the matrix instructions of the other:
     //   K operands (all of the tile, one wait)    S0 = K Q0^T
@@ -438,7 +553,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     };
     // One barrier per tile: the loads of tile i + 1 are issued before the arithmetic on tile i and land in
     // the other stage, which was last read before the previous barrier.
-    auto step = [&](auto parity_tag, int t0) __attribute__((always_inline)) {
+    auto step = [&](auto parity_tag, auto careful_tag, int t0) __attribute__((always_inline)) {
         constexpr int PAR = decltype(parity_tag)::value;
         if (t0 + TK < wg_t_end) dma(t0 + TK, PAR ? s_stage0 : s_stage1);   // workgroup-uniform
         if (t0 < wave_t_end) {                                              // wave-uniform
@@ -447,20 +562,57 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
                 // only tiles that reach past the wavefront's first position need the causal mask
                 if (t0 + TK > wave_limit_min) tile_pf(stage, t0, std::true_type{});
                 else tile_pf(stage, t0, std::false_type{});
+            } else if constexpr (decltype(careful_tag)::value) {
+                if (t0 >= first_careful_tile) tile(stage, t0);
             } else {
-                tile(stage, t0);
+                if (t0 < first_careful_tile) tile_lz(stage, t0);
             }
         }
         __builtin_amdgcn_s_waitcnt(0xF70);   // vmcnt(0): this wavefront's part of the next stage has landed
         __syncthreads();
     };
-
-    dma(0, s_stage0);
-    __builtin_amdgcn_s_waitcnt(0xF70);
-    __syncthreads();
-    for (int t0 = 0; t0 < wg_t_end; t0 += 2 * TK) {
-        step(std::integral_constant<int, 0>{}, t0);
-        if (t0 + TK < wg_t_end) step(std::integral_constant<int, 1>{}, t0 + TK);
+    // tiles from t_begin (a multiple of TK) on; the stage of a tile is its index's parity
+    auto tiles_from = [&](auto careful_tag, int t_begin) __attribute__((always_inline)) {
+        const bool odd = ((t_begin / TK) & 1) != 0;
+        dma(t_begin, odd ? s_stage1 : s_stage0);
+        __builtin_amdgcn_s_waitcnt(0xF70);
+        __syncthreads();
+        if constexpr (!PF && !decltype(careful_tag)::value) {
+            if (wave_t_end > 0) reference_from_first_tile(s_stage0);
+        }
+        int t0 = t_begin;
+        if (odd) {
+            step(std::integral_constant<int, 1>{}, careful_tag, t0);
+            t0 += TK;
+        }
+        for (; t0 < wg_t_end; t0 += 2 * TK) {
+            step(std::integral_constant<int, 0>{}, careful_tag, t0);
+            if (t0 + TK < wg_t_end) step(std::integral_constant<int, 1>{}, careful_tag, t0 + TK);
+        }
+    };
+    if constexpr (PF) {
+        tiles_from(std::false_type{}, 0);
+    } else if constexpr (!NOMAX) {
+        tiles_from(std::true_type{}, 0);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) Lsum[cb] = L[cb][0];
+    } else {
+        // First the tiles without a maximum; a wavefront whose column sums leave the range stops there with its
+        // accumulators untouched by that tile.  Then, from the earliest such tile of the workgroup on (the loads
+        // are the workgroup's), the tiles with the maximum taken first, each wavefront joining at its own tile.
+        __shared__ int s_first_careful;
+        if (tid == 0) s_first_careful = 0x7fffffff;
+        tiles_from(std::false_type{}, 0);
+        if (lane == 0 && first_careful_tile < wave_t_end) atomicMin(&s_first_careful, first_careful_tile);
+        __syncthreads();
+        const int t_begin = wave_uniform(s_first_careful);
+        if (t_begin < wg_t_end) {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) L[cb] = f32x4_t{Lsum[cb], Lsum[cb], Lsum[cb], Lsum[cb]};
+            tiles_from(std::true_type{}, t_begin);
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) Lsum[cb] = L[cb][0];
+        }
     }
 
 #pragma unroll
@@ -468,7 +620,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         if (col_limit[cb] > 0) {
             const int qi = wave_first_qi + cb * ppw + fn / R;
             const int qh = kvh * R + fn % R;
-            const float inv = 1.0f / (PF ? Lsum[cb] : L[cb][0]);
+            const float inv = 1.0f / Lsum[cb];
             uint16_t* orow = p.out + b * p.o_sb + int64_t(qh) * p.o_sh + int64_t(qi) * p.o_st + fg * 4;
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
@@ -500,8 +652,18 @@ int launch_attn_prefill_tiled(const PrefillParams& p, int HD, hipStream_t stream
     constexpr int CB = kPrefillColBlocks, NW = kPrefillTiledWaves;
     // tiles of 64 tokens; four wavefronts per SIMD at head size 64 (four workgroups per compute unit), two
     // at 128 (two workgroups: a stage pair is 64 KiB)
-    if (HD == 64) return launch_blocks(attn_prefill_tiled_kernel<64, CB, NW, 64, 4>, p, NW, CB, stream);
-    return launch_blocks(attn_prefill_tiled_kernel<128, CB, NW, 64, 2>, p, NW, CB, stream);
+    if (HD == 64) {
+        // The tiles that take no maximum gain where the device is refilled as workgroups finish (8192 tokens:
+        // -4.5 %, 2 x 4096: -2.9 %); a launch that it holds at once gains nothing from them.
+        const int R = p.QH / p.KVH;
+        const int wg_pos = NW * CB * (16 / R);
+        const int64_t wgs = int64_t(p.B) * p.KVH * ((p.T + wg_pos - 1) / wg_pos);
+        if (p.no_max_tiles || wgs > 4 * int64_t(current_device_cus())) {
+            return launch_blocks(attn_prefill_tiled_kernel<64, CB, NW, 64, 4, true>, p, NW, CB, stream);
+        }
+        return launch_blocks(attn_prefill_tiled_kernel<64, CB, NW, 64, 4, false>, p, NW, CB, stream);
+    }
+    return launch_blocks(attn_prefill_tiled_kernel<128, CB, NW, 64, 2, false>, p, NW, CB, stream);
 }
 
 }  // namespace l3

@@ -156,8 +156,7 @@ int attn_impl_of(int flags) { return (flags & L3_ATTN_FLAG_KERNEL_FMA) ? kAttnIm
 bool attn_flags_ok(int flags) {
     constexpr int known = L3_ATTN_FLAG_KERNEL_FMA | L3_ATTN_FLAG_PREFILL_MASK | L3_ATTN_FLAG_WS_COUNTERS |
                           L3_ATTN_FLAG_TWO_LAUNCHES | L3_ATTN_FLAG_FORM_MASK;
-    return (flags & ~known) == 0 && (flags & L3_ATTN_FLAG_PREFILL_MASK) != L3_ATTN_FLAG_PREFILL_MASK &&
-           (flags & L3_ATTN_FLAG_FORM_MASK) != L3_ATTN_FLAG_FORM_MASK;
+    return (flags & ~known) == 0 && (flags & L3_ATTN_FLAG_FORM_MASK) != L3_ATTN_FLAG_FORM_MASK;
 }
 // Whether the plan may count on the merge inside the split launch (the MFMA kernel with a counter
 // region in the workspace, not switched off for the call).
@@ -549,6 +548,7 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     p.o_sb = out_strides[0]; p.o_sh = out_strides[1]; p.o_st = out_strides[2];
     p.scale_log2e = scale * 1.4426950408889634f;
     p.snake = 0;
+    p.no_max_tiles = (flags & L3_ATTN_FLAG_PREFILL_MASK) == L3_ATTN_FLAG_PREFILL_TILED_NO_MAX;
     // Which form (graph-timed sweeps over B 1 ... 256, T 16 ... 8192, head ratios 1, 3, 4 and 8): a prompt
     // that does not exceed one workgroup of the tiled form per kv head, with few enough wavefronts for the
     // device to hold them all at once, runs as independent wavefronts with no barrier (4.2 against 4.8 us

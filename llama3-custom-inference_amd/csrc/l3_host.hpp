@@ -85,6 +85,7 @@ struct PrefillParams {
     int64_t o_sb, o_sh, o_st;
     float scale_log2e;
     int snake;   // tiled form: ranks per round of the reversed-every-second-round order, 0 = plain (set by the launcher)
+    int no_max_tiles;   // tiled form, head size 64: the tiles that take no maximum also for launches the device holds at once
 };
 
 struct LinearParams {

@@ -36,6 +36,7 @@ L3_ATTN_FLAG_TWO_LAUNCHES = 0x40
 L3_ATTN_COUNTER_BYTES = 128 << 10
 L3_ATTN_FLAG_PREFILL_WAVE = 0x10
 L3_ATTN_FLAG_PREFILL_TILED = 0x20
+L3_ATTN_FLAG_PREFILL_TILED_NO_MAX = 0x30
 L3_ATTN_FLAG_PREFILL_MASK = 0x30
 
 # name -> (restype, argtypes); mirrors include/l3_kernels.h line by line

@@ -125,14 +125,15 @@ def _attn_workspace(lib, device, stream_ptr: int, flags: int, size_of):
 _attn_flags = contextvars.ContextVar("l3_attn_flags", default=0)
 
 _KERNEL_BITS = {"mfma": 0, "fma": _l3lib.L3_ATTN_FLAG_KERNEL_FMA}
-_PREFILL_BITS = {"auto": 0, "wave": _l3lib.L3_ATTN_FLAG_PREFILL_WAVE, "tiled": _l3lib.L3_ATTN_FLAG_PREFILL_TILED}
+_PREFILL_BITS = {"auto": 0, "wave": _l3lib.L3_ATTN_FLAG_PREFILL_WAVE, "tiled": _l3lib.L3_ATTN_FLAG_PREFILL_TILED,
+                 "tiled-no-max": _l3lib.L3_ATTN_FLAG_PREFILL_TILED_NO_MAX}
 _LAUNCH_BITS = {"auto": 0, "two": _l3lib.L3_ATTN_FLAG_TWO_LAUNCHES}
 
 
 @contextlib.contextmanager
 def attention_flags(kernel=None, prefill=None, launches=None):
     """Within the block, attention calls of this thread that pass no ``flags`` use the named
-    split-KV kernel ("mfma" / "fma"), prefill form ("auto" / "wave" / "tiled") and launch scheme
+    split-KV kernel ("mfma" / "fma"), prefill form ("auto" / "wave" / "tiled" / "tiled-no-max") and launch scheme
     ("auto" / "two": always split kernel + combine kernel).  An argument that is not given keeps what
     an enclosing block chose, so blocks nest.  For measurements and tests; the defaults are the
     library's own choices."""

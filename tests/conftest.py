@@ -42,7 +42,7 @@ def attn_kernel(request):
         yield request.param
 
 
-@pytest.fixture(params=["auto", "wave", "tiled"])
+@pytest.fixture(params=["auto", "wave", "tiled", "tiled-no-max"])
 def prefill_form(request):
     """Run a prefill test once per form of the kernel (the library's own choice, and each forced)."""
     from custom_kernels import custom_kernels_extension as cke

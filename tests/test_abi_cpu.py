@@ -299,7 +299,6 @@ def test_prefill_argument_checks():
     assert call(scale=0.0) == _l3lib.L3_ERR_SCALE
 
     assert call(flags=0x80) == _l3lib.L3_ERR_FLAGS
-    assert call(flags=0x30) == _l3lib.L3_ERR_FLAGS          # both prefill bits: no such form
     assert call(flags=0xc) == _l3lib.L3_ERR_FLAGS           # both form bits
     assert call(out=None) == _l3lib.L3_ERR_NULL_POINTER
     assert call(HD=96) == _l3lib.L3_ERR_HEAD_SIZE

@@ -481,6 +481,39 @@ def test_prefill_forms_agree_on_a_long_prompt(gpu):
         assert_attn_close(outs["wave"][:, :, i:i + 1], ref, what=f"long prefill row {i} (wave)")
 
 
+@pytest.mark.parametrize("HD", [64, 128])
+@pytest.mark.parametrize("where", [(70,), (1500,), (2047,), (100, 900, 1800), (64, 65, 127, 128)])
+def test_prefill_scores_that_outgrow_the_reference(gpu, HD, where):
+    """A long prompt in which a few keys, past the first 64 tokens, each score some twenty nats above everything
+    before them for the queries of their group: the tiles that take no maximum (forced here; the library turns
+    to them only for large launches) have to notice, and go on with the maximum taken first from that tile
+    on without losing what they had.  Wavefronts of one workgroup meet such a key at different tiles or not
+    at all (queries before it never see it)."""
+    from custom_kernels import custom_kernels_extension as cke
+    from oracle import attention_prefill_ref
+
+    B, QH, KVH, T = 1, 8, 2, 2048
+    print(f"prefill outgrown reference HD={HD} where={where}", flush=True)
+    q = randn_bf16((B, T, QH, HD), 94)
+    k = randn_bf16((B, T, KVH, HD), 95)
+    v = randn_bf16((B, T, KVH, HD), 96)
+    unit = q[0, T - 1, 5].float() * (HD ** 0.5 / float((q[0, T - 1, 5].float() ** 2).sum()))   # scores 1 with that query
+    for n, w in enumerate(where):
+        k[0, w, 1] = (unit * 20.0 * (n + 1)).to(torch.bfloat16)
+    ref = attention_prefill_ref(t2f32(q.transpose(1, 2)), t2f32(k.transpose(1, 2)), t2f32(v.transpose(1, 2)))
+    outs = {}
+    for form in ("tiled", "tiled-no-max"):
+        with cke.attention_flags(prefill=form):
+            outs[form] = cke.flash_attention_prefill(q.to(gpu).transpose(1, 2), k.to(gpu).transpose(1, 2),
+                                                     v.to(gpu).transpose(1, 2))
+        torch.cuda.synchronize()
+        assert_attn_close(outs[form], ref, what=f"prefill outgrown reference HD={HD} where={where} {form}", regression=False)
+        # the last query of head 5 puts nearly all its weight on the last of those keys
+        assert np.abs(t2f32(outs[form])[0, 5, T - 1] - t2f32(v)[0, where[-1], 1]).max() < 0.05
+    if HD == 128:
+        assert torch.equal(outs["tiled"], outs["tiled-no-max"])   # one kernel at this head size
+
+
 @pytest.mark.parametrize("B,T,HD,gain", [(2, 2048, 64, 1.0), (1, 8192, 128, 1.0), (1, 8192, 64, 1.0),
                                          (1, 8192, 128, 3.0), (1, 8192, 64, 3.0)])
 def test_prefill_timed_shapes_by_sampled_rows(gpu, B, T, HD, gain):
