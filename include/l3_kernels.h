@@ -62,7 +62,9 @@ const char* l3_strerror(int code);
  *                            (the reference has one kernel and no counterpart of this choice).
  *   L3_ATTN_FLAG_PREFILL_*   prefill: force one form of l3_attn_prefill instead of the choice by
  *                            prompt length -- WAVE (every wavefront streams K/V on its own), TILED (a
- *                            workgroup shares K/V tiles) or TILED_NO_MAX (TILED, and at head size 64 the
+ *                            workgroup shares K/V tiles; forced, it is the kernel with two column blocks
+ *                            per wavefront, where the library's own choice runs one for launches that
+ *                            would leave much of the device empty) or TILED_NO_MAX (TILED, and at head size 64 the
  *                            tiles that take no maximum whatever the size of the launch; left to itself
  *                            the library uses them for launches of more workgroups than the device holds
  *                            at once).  Same results within the stated tolerance; for tests and timing.

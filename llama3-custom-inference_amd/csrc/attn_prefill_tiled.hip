@@ -55,7 +55,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     constexpr int LOADS = TK * CPR / kWaveSize;  // wavefront-wide loads per operand tile
     static_assert(LOADS % NW == 0, "a tile must divide evenly over the wavefronts");
     constexpr int IPW = LOADS / NW;
-    constexpr bool PF = WPE <= 2;                // the interleaved tile below (needs the registers of two wavefronts per SIMD)
+    constexpr bool PF = WPE <= 2 && CB == 2;                // the interleaved tile below (needs the registers of two wavefronts per SIMD)
     __shared__ __align__(1024) unsigned char s_stage0[STAGE];
     __shared__ __align__(1024) unsigned char s_stage1[STAGE];
 
@@ -652,16 +652,28 @@ int launch_attn_prefill_tiled(const PrefillParams& p, int HD, hipStream_t stream
     constexpr int CB = kPrefillColBlocks, NW = kPrefillTiledWaves;
     // tiles of 64 tokens; four wavefronts per SIMD at head size 64 (four workgroups per compute unit), two
     // at 128 (two workgroups: a stage pair is 64 KiB)
+    const int R = p.QH / p.KVH;
+    const int wg_pos = NW * CB * (16 / R);
+    const int64_t wgs = int64_t(p.B) * p.KVH * ((p.T + wg_pos - 1) / wg_pos);
+    const int64_t cus = current_device_cus();
+    // A launch that leaves much of the device empty runs with one column block per wavefront instead of two: twice
+    // the workgroups, each K/V operand read feeding one matrix instruction.  Graph-timed at head size 128 against
+    // the two-block kernel: 512 tokens -22 %, 1024 -14 %, 1536 -12 %, 1792 -2.5 %, 1920 +2 %; at head size 64:
+    // 1024 tokens -23 %, 2048 -17 %, 2560 -10 %, 2816 -3.5 %, 3072 +2 %, 5 x 512 +2.5 %.  Only the library's own
+    // choice does this: a forced TILED form is the two-block kernel whatever the size.
     if (HD == 64) {
         // The tiles that take no maximum gain where the device is refilled as workgroups finish (8192 tokens:
         // -4.5 %, 2 x 4096: -2.9 %); a launch that it holds at once gains nothing from them.
-        const int R = p.QH / p.KVH;
-        const int wg_pos = NW * CB * (16 / R);
-        const int64_t wgs = int64_t(p.B) * p.KVH * ((p.T + wg_pos - 1) / wg_pos);
-        if (p.no_max_tiles || wgs > 4 * int64_t(current_device_cus())) {
+        if (p.no_max_tiles || wgs > 4 * cus) {
             return launch_blocks(attn_prefill_tiled_kernel<64, CB, NW, 64, 4, true>, p, NW, CB, stream);
         }
+        if (p.auto_form && 4 * wgs <= 9 * cus) {
+            return launch_blocks(attn_prefill_tiled_kernel<64, 1, NW, 64, 4, false>, p, NW, 1, stream);
+        }
         return launch_blocks(attn_prefill_tiled_kernel<64, CB, NW, 64, 4, false>, p, NW, CB, stream);
+    }
+    if (p.auto_form && 4 * wgs <= 7 * cus) {
+        return launch_blocks(attn_prefill_tiled_kernel<128, 1, NW, 64, 2, false>, p, NW, 1, stream);
     }
     return launch_blocks(attn_prefill_tiled_kernel<128, CB, NW, 64, 2, false>, p, NW, CB, stream);
 }

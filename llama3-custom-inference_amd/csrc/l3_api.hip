@@ -549,15 +549,17 @@ int l3_attn_prefill(const void* q, const void* k, const void* v, void* out, int 
     p.scale_log2e = scale * 1.4426950408889634f;
     p.snake = 0;
     p.no_max_tiles = (flags & L3_ATTN_FLAG_PREFILL_MASK) == L3_ATTN_FLAG_PREFILL_TILED_NO_MAX;
-    // Which form (graph-timed sweeps over B 1 ... 256, T 16 ... 8192, head ratios 1, 3, 4 and 8): a prompt
-    // that does not exceed one workgroup of the tiled form per kv head, with few enough wavefronts for the
-    // device to hold them all at once, runs as independent wavefronts with no barrier (4.2 against 4.8 us
-    // for 16 tokens, 5.6 against 6.9 us for 32 at head size 128); everything else shares K/V tiles.
+    p.auto_form = (flags & L3_ATTN_FLAG_PREFILL_MASK) == 0;
+    // Which form (graph-timed sweeps over B 1 ... 256, T 8 ... 8192, head ratios 1, 3, 4 and 8): a prompt
+    // that does not exceed one workgroup of the tiled form's small variant (one column block per wavefront) per
+    // kv head, with few enough wavefronts for the device to hold them all at once, runs as independent
+    // wavefronts with no barrier (16 tokens at head size 128: 4.8 against 6.1 us); everything else shares K/V
+    // tiles (32 tokens: 5.2 against 5.9 us at head size 128, 4.2 against 5.1 us at 64).
     int form = flags & L3_ATTN_FLAG_PREFILL_MASK;
     if (form == 0) {
         const int R = QH / KVH;
         const int64_t private_waves = int64_t(B) * KVH * ((int64_t(T) * R + 15) / 16);
-        const bool tiny = T <= prefill_tiled_positions_per_wg(R) && private_waves <= 4 * int64_t(current_device_cus());
+        const bool tiny = T <= prefill_tiled_positions_per_wg(R) / 2 && private_waves <= 4 * int64_t(current_device_cus());
         form = tiny ? L3_ATTN_FLAG_PREFILL_WAVE : L3_ATTN_FLAG_PREFILL_TILED;
     }
     hipStream_t st = static_cast<hipStream_t>(stream);

@@ -86,6 +86,7 @@ struct PrefillParams {
     float scale_log2e;
     int snake;   // tiled form: ranks per round of the reversed-every-second-round order, 0 = plain (set by the launcher)
     int no_max_tiles;   // tiled form, head size 64: the tiles that take no maximum also for launches the device holds at once
+    int auto_form;      // the form was the library's choice (it may then run one column block per wavefront)
 };
 
 struct LinearParams {
