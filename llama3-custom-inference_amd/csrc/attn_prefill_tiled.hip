@@ -662,9 +662,11 @@ int launch_attn_prefill_tiled(const PrefillParams& p, int HD, hipStream_t stream
     // 1024 tokens -23 %, 2048 -17 %, 2560 -10 %, 2816 -3.5 %, 3072 +2 %, 5 x 512 +2.5 %.  Only the library's own
     // choice does this: a forced TILED form is the two-block kernel whatever the size.
     if (HD == 64) {
-        // The tiles that take no maximum gain where the device is refilled as workgroups finish (8192 tokens:
-        // -4.5 %, 2 x 4096: -2.9 %); a launch that it holds at once gains nothing from them.
-        if (p.no_max_tiles || wgs > 4 * cus) {
+        // The tiles that take no maximum gain where the device is refilled as workgroups finish and the rows are
+        // long (8192 tokens: -4.5 %, 6144: -4.2 %, 2 x 4096: -3 %); a launch that the device holds at once gains
+        // nothing, and short rows lose to the extra pass over the first tile (4 x 2048: 0, 32 x 256: +8 %,
+        // 64 x 128: +18 %).
+        if (p.no_max_tiles || (wgs > 4 * cus && p.S >= 4096)) {
             return launch_blocks(attn_prefill_tiled_kernel<64, CB, NW, 64, 4, true>, p, NW, CB, stream);
         }
         if (p.auto_form && 4 * wgs <= 9 * cus) {
