@@ -64,10 +64,11 @@ const char* l3_strerror(int code);
  *                            prompt length -- WAVE (every wavefront streams K/V on its own), TILED (a
  *                            workgroup shares K/V tiles; forced, it is the kernel with two column blocks
  *                            per wavefront, where the library's own choice runs one for launches that
- *                            would leave much of the device empty) or TILED_NO_MAX (TILED, and at head size 64 the
- *                            tiles that take no maximum whatever the size of the launch; left to itself
+ *                            would leave much of the device empty) or TILED_NO_MAX (the tiled kernels whose
+ *                            loop takes no maximum, whatever the size of the launch; left to itself
  *                            the library uses them for prompts of 4096 tokens or more in launches of more
- *                            workgroups than the device holds at once).  Same results within the stated tolerance; for tests and timing.
+ *                            workgroups than the device holds at once).  Same results within the stated
+ *                            tolerance; for tests and timing.
  *   L3_ATTN_FLAG_WS_COUNTERS decode: the workspace starts with L3_ATTN_COUNTER_BYTES of arrival counters
  *                            that l3_attn_workspace_init prepared (see there); the library may then merge
  *                            the split partials inside the split launch instead of launching a combine.

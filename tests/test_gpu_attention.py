@@ -510,8 +510,6 @@ def test_prefill_scores_that_outgrow_the_reference(gpu, HD, where):
         assert_attn_close(outs[form], ref, what=f"prefill outgrown reference HD={HD} where={where} {form}", regression=False)
         # the last query of head 5 puts nearly all its weight on the last of those keys
         assert np.abs(t2f32(outs[form])[0, 5, T - 1] - t2f32(v)[0, where[-1], 1]).max() < 0.05
-    if HD == 128:
-        assert torch.equal(outs["tiled"], outs["tiled-no-max"])   # one kernel at this head size
 
 
 @pytest.mark.parametrize("B,T,HD,gain", [(2, 2048, 64, 1.0), (1, 8192, 128, 1.0), (1, 8192, 64, 1.0),
