@@ -342,6 +342,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
     // The tiles from there on are done afterwards by the maximum-first tile above, which takes over m_run, O and
     // the denominator as they stand.  The reference is the maximum of the first tile's scores, per column: a row
     // leaves the range only when a later score exceeds everything among its first 64 by a factor of hundreds.
+    __shared__ int s_first_careful;   // the earliest tile at which a wavefront of the workgroup stopped (NOMAX)
     int first_careful_tile = NOMAX ? 0x7fffffff : 0;   // wave-uniform: the tile from which this wavefront takes the maximum first
     auto scores32 = [&](const unsigned char* stage, int t0, int ks, f32x4_t (&Z)[CB][2]) __attribute__((always_inline)) {
 #pragma unroll
@@ -405,6 +406,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         for (int cb = 0; cb < CB; ++cb) out_of_range = out_of_range || !(sum[cb][0] <= kTileSumLimit);
         if (__builtin_amdgcn_ballot_w64(out_of_range) != 0) {   // nothing of this tile has reached the accumulators
             first_careful_tile = t0;
+            if (lane == 0) atomicMin(&s_first_careful, t0);   // the workgroup looks at this every eighth tile
             return;
         }
 #pragma unroll
@@ -572,7 +574,7 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         __syncthreads();
     };
     // tiles from t_begin (a multiple of TK) on; the stage of a tile is its index's parity
-    auto tiles_from = [&](auto careful_tag, int t_begin) __attribute__((always_inline)) {
+    auto tiles_from = [&](auto careful_tag, int t_begin) __attribute__((always_inline)) -> int {
         const bool odd = ((t_begin / TK) & 1) != 0;
         dma(t_begin, odd ? s_stage1 : s_stage0);
         __builtin_amdgcn_s_waitcnt(0xF70);
@@ -588,7 +590,22 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         for (; t0 < wg_t_end; t0 += 2 * TK) {
             step(std::integral_constant<int, 0>{}, careful_tag, t0);
             if (t0 + TK < wg_t_end) step(std::integral_constant<int, 1>{}, careful_tag, t0 + TK);
+            if constexpr (NOMAX && !decltype(careful_tag)::value) {
+                // Every eighth tile: once a wavefront has stopped, the workgroup leaves this loop, so that the tiles
+                // it would only load and not use are few.  Read between two barriers: wavefronts write the word
+                // only inside a tile, so all of them see the same value here.
+                if (((t0 / (2 * TK)) & 3) == 3) {
+                    __syncthreads();
+                    const int stopped_at = wave_uniform(s_first_careful);
+                    __syncthreads();
+                    if (stopped_at != 0x7fffffff) {
+                        t0 += 2 * TK;
+                        break;
+                    }
+                }
+            }
         }
+        return t0;   // the first tile this loop has not been offered
     };
     if constexpr (PF) {
         tiles_from(std::false_type{}, 0);
@@ -598,11 +615,12 @@ attn_prefill_tiled_kernel(const PrefillParams p) {
         for (int cb = 0; cb < CB; ++cb) Lsum[cb] = L[cb][0];
     } else {
         // First the tiles without a maximum; a wavefront whose column sums leave the range stops there with its
-        // accumulators untouched by that tile.  Then, from the earliest such tile of the workgroup on (the loads
-        // are the workgroup's), the tiles with the maximum taken first, each wavefront joining at its own tile.
-        __shared__ int s_first_careful;
+        // accumulators untouched by that tile, and the workgroup ends that loop within eight tiles.  Then, from the
+        // earliest such tile of the workgroup on (the loads are the workgroup's), the tiles with the maximum taken
+        // first, each wavefront joining at its own tile.
         if (tid == 0) s_first_careful = 0x7fffffff;
-        tiles_from(std::false_type{}, 0);
+        const int offered = tiles_from(std::false_type{}, 0);
+        first_careful_tile = min(first_careful_tile, offered);   // a wavefront that had not stopped goes on from where the loop ended
         if (lane == 0 && first_careful_tile < wave_t_end) atomicMin(&s_first_careful, first_careful_tile);
         __syncthreads();
         const int t_begin = wave_uniform(s_first_careful);
@@ -666,7 +684,7 @@ int launch_attn_prefill_tiled(const PrefillParams& p, int HD, hipStream_t stream
         // long (8192 tokens: -4.5 %, 6144: -4.2 %, 2 x 4096: -3 %); a launch that the device holds at once gains
         // nothing, and short rows lose to the extra pass over the first tile (4 x 2048: 0, 32 x 256: +8 %,
         // 64 x 128: +18 %).
-        if (p.no_max_tiles || (wgs > 4 * cus && p.S >= 4096)) {
+        if (p.no_max_tiles || (p.auto_form && wgs > 4 * cus && p.S >= 4096)) {
             return launch_blocks(attn_prefill_tiled_kernel<64, CB, NW, 64, 4, true>, p, NW, CB, stream);
         }
         if (p.auto_form && 4 * wgs <= 9 * cus) {
