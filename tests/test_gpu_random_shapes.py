@@ -100,6 +100,40 @@ def test_prefill_attention_random_shapes(gpu, case):
     assert_attn_close(out, ref, what=f"prefill case {i}")
 
 
+def _draw_prefill_cases_all_forms(n, seed):
+    """Like the cases above, with the no-maximum loop among the forms, longer prompts now and then, and for a
+    third of the cases queries scaled so that a few keys carry a row (scores over tens of powers of two)."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n):
+        HD = int(rng.choice((64, 128)))
+        R = int(rng.choice(RATIOS))
+        KVH = int(rng.integers(1, 5))
+        B = int(rng.integers(1, 4))
+        T = int(rng.choice((int(rng.integers(2, 70)), int(rng.integers(70, 400)), int(rng.integers(400, 1500)))))
+        past = int(rng.choice((0, 0, 3, 64, 200)))
+        form = str(rng.choice(("auto", "tiled", "tiled-no-max", "tiled-no-max")))
+        gain = float(rng.choice((1.0, 1.0, 3.0)))
+        cases.append((i, B, R * KVH, KVH, T, T + past, HD, form, gain))
+    return cases
+
+
+@pytest.mark.parametrize("case", _draw_prefill_cases_all_forms(40, 78), ids=lambda c: f"q{c[0]}")
+def test_prefill_attention_random_shapes_all_forms(gpu, case):
+    from custom_kernels import custom_kernels_extension as cke
+
+    i, B, QH, KVH, T, S, HD, form, gain = case
+    print(f"prefill case q{i}: B={B} QH={QH} KVH={KVH} T={T} S={S} HD={HD} form={form} gain={gain}", flush=True)
+    q = (randn_bf16((B, T, QH, HD), 5000 + i).float() * gain).to(torch.bfloat16)
+    k = randn_bf16((B, S, KVH, HD), 6000 + i)
+    v = randn_bf16((B, S, KVH, HD), 7000 + i)
+    with cke.attention_flags(prefill=form):
+        out = cke.flash_attention_prefill(*(t.to(gpu).transpose(1, 2) for t in (q, k, v)))
+        torch.cuda.synchronize()
+    ref = attention_prefill_ref(*(t2f32(t.transpose(1, 2)) for t in (q, k, v)))
+    assert_attn_close(out, ref, what=f"prefill case q{i}", regression=gain == 1.0)
+
+
 def test_rms_norm_random_shapes(gpu):
     from custom_kernels import custom_kernels_extension as cke
 
