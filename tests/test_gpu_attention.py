@@ -416,7 +416,8 @@ def test_concurrent_streams_do_not_share_scratch(gpu):
 @pytest.mark.parametrize("B,QH,KVH,T,S", [(1, 32, 8, 128, 128), (2, 8, 2, 37, 37), (1, 4, 4, 16, 16), (3, 24, 8, 5, 5),
                                            (1, 16, 2, 130, 130), (2, 32, 8, 64, 200), (1, 8, 8, 2, 2),
                                            (1, 32, 8, 1000, 1000), (1, 6, 3, 33, 40), (1, 16, 16, 300, 300),
-                                           (1, 16, 2, 257, 321)])
+                                           (1, 16, 2, 257, 321), (3, 32, 8, 300, 300), (4, 8, 2, 100, 164),
+                                           (8, 32, 8, 64, 64)])
 def test_prefill_against_oracle(gpu, prefill_form, HD, B, QH, KVH, T, S):
     from custom_kernels import custom_kernels_extension as cke
     from oracle import attention_prefill_ref
